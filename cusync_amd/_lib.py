@@ -1,0 +1,125 @@
+"""ctypes binding of ``libcusync_amd.so`` (the C ABI in ``include/cusync_amd.h``).
+
+The library is loaded from ``cusync_amd/lib/`` inside the source tree; there is
+no fallback: if it has not been built (``python -c "import __graft_entry__ as g;
+g.build()"`` or ``make -C cusync_amd/csrc``) loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libcusync_amd.so")
+TEST_LIB_PATH = os.path.join(LIB_DIR, "libcusync_stage_tests.so")
+
+u32, i32, vp, sz = C.c_uint32, C.c_int32, C.c_void_p, C.c_size_t
+
+
+class Dim3(C.Structure):
+    _fields_ = [("x", u32), ("y", u32), ("z", u32)]
+
+    def tup(self):
+        return (self.x, self.y, self.z)
+
+
+class PolicyDesc(C.Structure):
+    _fields_ = [("kind", i32), ("order", i32), ("tileM", u32), ("tileN", u32),
+                ("waitValue", u32), ("postValue", u32), ("gridN", u32), ("stride", u32),
+                ("R", u32), ("S", u32), ("H", u32)]
+
+
+class StageDesc(C.Structure):
+    _fields_ = [("grid", Dim3), ("prodGrid", Dim3), ("tileSize", Dim3),
+                ("iter", i32), ("opts", i32), ("in_", PolicyDesc), ("out", PolicyDesc),
+                ("tileOrder", vp), ("tileCounter", vp), ("startCounter", vp),
+                ("kernelExecuted", vp), ("spinTimeouts", vp),
+                ("tileStatusWrite", vp), ("tileStatusRead", vp)]
+
+
+class GemmArgs(C.Structure):
+    _fields_ = [("stage", StageDesc), ("M", u32), ("N", u32), ("K", u32),
+                ("A", vp), ("lda", u32), ("B", vp), ("ldb", u32), ("D", vp), ("ldd", u32),
+                ("epilogue", i32), ("a_mode", i32), ("tile", i32), ("split_k", i32),
+                ("workspace", vp), ("max_workgroups", i32)]
+
+
+class MlpConfig(C.Structure):
+    _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
+                ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32)]
+
+
+# every symbol include/cusync_amd.h declares: name -> (restype, argtypes)
+SIGNATURES = {
+    "cusync_rt_last_error": (C.c_char_p, []),
+    "cusync_rt_device_count": (C.c_int, []),
+    "cusync_rt_device_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz), C.c_char_p, sz]),
+    "cusync_rt_malloc": (C.c_int, [C.POINTER(vp), sz]),
+    "cusync_rt_free": (C.c_int, [vp]),
+    "cusync_rt_memset": (C.c_int, [vp, C.c_int, sz]),
+    "cusync_rt_memcpy_h2d": (C.c_int, [vp, vp, sz]),
+    "cusync_rt_memcpy_d2h": (C.c_int, [vp, vp, sz]),
+    "cusync_rt_memcpy_d2d": (C.c_int, [vp, vp, sz]),
+    "cusync_rt_stream_create": (C.c_int, [C.POINTER(vp)]),
+    "cusync_rt_stream_destroy": (C.c_int, [vp]),
+    "cusync_rt_stream_sync": (C.c_int, [vp]),
+    "cusync_rt_device_sync": (C.c_int, []),
+    "cusync_rt_event_create": (C.c_int, [C.POINTER(vp)]),
+    "cusync_rt_event_destroy": (C.c_int, [vp]),
+    "cusync_rt_event_record": (C.c_int, [vp, vp]),
+    "cusync_rt_event_sync": (C.c_int, [vp]),
+    "cusync_rt_event_elapsed_us": (C.c_int, [vp, vp, C.POINTER(C.c_double)]),
+    "cusync_rt_stream_wait_event": (C.c_int, [vp, vp]),
+    "cusync_stage_alloc": (C.c_int, [C.POINTER(StageDesc), vp]),
+    "cusync_stage_free": (C.c_int, [C.POINTER(StageDesc)]),
+    "cusync_stage_create": (C.c_int, [C.POINTER(StageDesc), C.c_int]),
+    "cusync_set_producer_consumer_pair": (C.c_int, [C.POINTER(StageDesc), C.POINTER(StageDesc)]),
+    "cusync_invoke_wait_kernel": (C.c_int, [C.POINTER(StageDesc), vp]),
+    "cusync_wait_kernel": (C.c_int, [vp, u32, vp]),
+    "cusync_stage_read_state": (C.c_int, [C.POINTER(StageDesc), vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
+    "cusync_policy_tile_index": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),
+    "cusync_policy_wait_value": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),
+    "cusync_policy_post_value": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),
+    "cusync_policy_is_sync": (C.c_int, [C.POINTER(PolicyDesc), Dim3, Dim3]),
+    "cusync_order_block_index": (u32, [C.c_int, Dim3, Dim3]),
+    "cusync_order_tile_to_block": (Dim3, [C.c_int, Dim3]),
+    "cusync_gemm_tile_shape": (C.c_int, [C.c_int, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
+    "cusync_gemm_grid": (Dim3, [C.c_int, u32, u32, C.c_int]),
+    "cusync_gemm_can_implement": (C.c_int, [C.POINTER(GemmArgs)]),
+    "cusync_gemm_workspace_size": (sz, [C.POINTER(GemmArgs)]),
+    "cusync_gemm_max_resident": (C.c_int, [C.c_int]),
+    "cusync_gemm_run": (C.c_int, [C.POINTER(GemmArgs), vp]),
+    "cusync_mlp_create": (vp, [C.POINTER(MlpConfig), vp, vp]),
+    "cusync_mlp_destroy": (None, [vp]),
+    "cusync_mlp_run": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double)]),
+    "cusync_mlp_run_split": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "cusync_mlp_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
+    "cusync_mlp_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the C-ABI library and attach prototypes.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "cusync_amd: %s is missing — the HIP library has not been built "
+            "(run `make -C cusync_amd/csrc` or __graft_entry__.build()). "
+            "There is no CPU fallback." % LIB_PATH)
+    L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        f = getattr(L, name)          # AttributeError if the symbol is not exported
+        f.restype = res
+        f.argtypes = args
+    _lib = L
+    return L
+
+
+def load_stage_tests():
+    load()
+    if not os.path.exists(TEST_LIB_PATH):
+        raise RuntimeError("cusync_amd: %s is missing — build it first" % TEST_LIB_PATH)
+    return C.CDLL(TEST_LIB_PATH)

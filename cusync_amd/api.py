@@ -1,0 +1,243 @@
+"""Python mirror of the host-side CuSync interface, bound to the C ABI.
+
+Names follow the reference's C++ API (CuStage, setProducerConsumerPair,
+invokeWaitKernel, incrementIter; src/include/cusync/cusync.h:87-299) so that the
+parity tests read like the reference's own tests.  Nothing here computes on the
+CPU: every operation is a call into ``libcusync_amd.so``.
+"""
+import ctypes as C
+from types import SimpleNamespace
+
+from . import _lib
+from ._lib import Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
+
+ERR = SimpleNamespace(NOT_PRODUCER=0, NOT_CONSUMER=1, NOT_INITIALIZED=2,
+                      INVALID_LINEAR_BLOCK_INDEX=3, DEVICE=4, SUCCESS=5)
+OPT = SimpleNamespace(NONE=0, NO_ATOMIC_ADD=1, AVOID_WAIT_KERNEL=2, AVOID_CUSTOM_ORDER=4, REORDER_TILE_LOADS=8)
+ORDER = SimpleNamespace(IDENTITY=0, TRANSPOSE_XY=1)
+POLICY = SimpleNamespace(NOSYNC=0, ROWSYNC=1, TILESYNC=2, STRIDEDSYNC=3, CONV2DTILESYNC=4, CONSECUTIVESYNC=5)
+EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2)
+TILE = SimpleNamespace(T256x256x32=0, T256x128x64=1, T128x128x64=2, T64x128x64=3, T32x128x64=4,
+                       T128x256x64=5, T256x64x64=6, T128x64x64=7, COUNT=8)
+SYNC = SimpleNamespace(STREAM=0, ROW=1, TILE=2, STRIDED=3)
+MODEL = SimpleNamespace(GPT3=0, LLAMA=1)
+
+
+class CuSyncError(RuntimeError):
+    def __init__(self, code, what=""):
+        self.code = code
+        super().__init__("%s: cusync error %d (%s)" % (what, code, last_error()))
+
+
+def last_error():
+    return _lib.load().cusync_rt_last_error().decode()
+
+
+def check(code, what=""):
+    if code != ERR.SUCCESS:
+        raise CuSyncError(code, what)
+
+
+def d3(t):
+    t = tuple(int(v) for v in t) + (0,) * (3 - len(t))
+    return Dim3(*t)
+
+
+def device_info():
+    L = _lib.load()
+    cus, clk = C.c_int(0), C.c_int(0)
+    lds, hbm = C.c_size_t(0), C.c_size_t(0)
+    name = C.create_string_buffer(128)
+    if L.cusync_rt_device_info(C.byref(cus), C.byref(clk), C.byref(lds), C.byref(hbm), name, 128):
+        raise RuntimeError(last_error())
+    return dict(cus=cus.value, clock_khz=clk.value, lds_per_cu=lds.value, hbm_bytes=hbm.value, arch=name.value.decode())
+
+
+# ---- policies ------------------------------------------------------------------
+
+def policy_desc(kind, order=ORDER.TRANSPOSE_XY, tileM=1, tileN=1, waitValue=0, postValue=0,
+                gridN=0, stride=0, R=1, S=1, H=0):
+    return PolicyDesc(kind, order, tileM, tileN, waitValue, postValue, gridN, stride, R, S, H)
+
+
+def no_sync():
+    return policy_desc(POLICY.NOSYNC)
+
+
+def row_sync(tileM, waitValue=0, postValue=None):
+    if postValue is None:
+        postValue = 1 if waitValue else 0
+    return policy_desc(POLICY.ROWSYNC, ORDER.TRANSPOSE_XY, tileM, 1, waitValue, postValue)
+
+
+def tile_sync(order, tileM, tileN, waitValue=1, postValue=1):
+    return policy_desc(POLICY.TILESYNC, order, tileM, tileN, waitValue, postValue)
+
+
+def strided_sync(order, gridN, tileM, tileN, stride):
+    return policy_desc(POLICY.STRIDEDSYNC, order, tileM, tileN, stride, 1, gridN=gridN, stride=stride)
+
+
+def conv2d_tile_sync(order, R, S, tileM, tileN, waitValue=1, postValue=1):
+    return policy_desc(POLICY.CONV2DTILESYNC, order, tileM, tileN, waitValue, postValue, R=R, S=S)
+
+
+def consecutive_sync(order, H, tileM, tileN):
+    return policy_desc(POLICY.CONSECUTIVESYNC, order, tileM, tileN, (H // 8) // tileN, 1, H=H)
+
+
+def policy_tile_index(p, tile, grid):
+    return _lib.load().cusync_policy_tile_index(C.byref(p), d3(tile), d3(grid))
+
+
+def policy_wait_value(p, tile=(0, 0, 0), grid=(1, 1, 1)):
+    return _lib.load().cusync_policy_wait_value(C.byref(p), d3(tile), d3(grid))
+
+
+def policy_post_value(p, tile=(0, 0, 0), grid=(1, 1, 1)):
+    return _lib.load().cusync_policy_post_value(C.byref(p), d3(tile), d3(grid))
+
+
+def policy_is_sync(p, tile, grid=(1, 1, 1)):
+    return bool(_lib.load().cusync_policy_is_sync(C.byref(p), d3(tile), d3(grid)))
+
+
+# ---- stages ----------------------------------------------------------------------
+
+class Stage:
+    """CuStage<TileOrder, InputSyncPolicy, OutputSyncPolicy, Opts> (run-time form)."""
+
+    def __init__(self, grid, tile_size, input_policy, output_policy, order=ORDER.TRANSPOSE_XY, opts=OPT.NONE):
+        self.L = _lib.load()
+        self.order = order
+        self.desc = StageDesc()
+        self.desc.grid = d3(grid)
+        self.desc.tileSize = d3(tile_size)
+        self.desc.iter = 1
+        self.desc.opts = opts
+        self.desc.in_ = input_policy
+        self.desc.out = output_policy
+        self.status = self.L.cusync_stage_create(C.byref(self.desc), order)
+        if self.status not in (ERR.SUCCESS, ERR.INVALID_LINEAR_BLOCK_INDEX):
+            raise CuSyncError(self.status, "cusync_stage_create")
+        self._alive = True
+
+    def grid(self):
+        return self.desc.grid.tup()
+
+    def isProducer(self):
+        return self.desc.out.kind != POLICY.NOSYNC
+
+    def isConsumer(self):
+        return self.desc.in_.kind != POLICY.NOSYNC
+
+    def numTiles(self):
+        g = self.desc.grid
+        return g.x * g.y * g.z
+
+    def invokeWaitKernel(self, stream):
+        return self.L.cusync_invoke_wait_kernel(C.byref(self.desc), stream)
+
+    def incrementIter(self):
+        self.desc.iter += 1
+
+    def read_state(self):
+        import numpy as np
+        n = self.numTiles()
+        sems = np.zeros(n, np.uint32)
+        order = np.zeros((n, 3), np.uint32)
+        tc, sc, ke, to = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+        check(self.L.cusync_stage_read_state(
+            C.byref(self.desc), sems.ctypes.data_as(C.c_void_p) if self.isProducer() else None,
+            order.ctypes.data_as(C.c_void_p), C.byref(tc), C.byref(sc), C.byref(ke), C.byref(to)), "read_state")
+        return SimpleNamespace(sems=sems, tile_order=order, tile_counter=tc.value, start_counter=sc.value,
+                               kernel_executed=ke.value, spin_timeouts=to.value)
+
+    def destroy(self):
+        if self._alive:
+            self.L.cusync_stage_free(C.byref(self.desc))
+            self._alive = False
+
+
+def set_producer_consumer_pair(prod, cons):
+    """CuSync::setProducerConsumerPair; returns the CuSyncError code."""
+    return _lib.load().cusync_set_producer_consumer_pair(C.byref(prod.desc), C.byref(cons.desc))
+
+
+# ---- GEMM ------------------------------------------------------------------------
+
+def tile_shape(tile):
+    m, n, k = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    if _lib.load().cusync_gemm_tile_shape(tile, C.byref(m), C.byref(n), C.byref(k)):
+        raise ValueError("unknown tile id %r" % (tile,))
+    return m.value, n.value, k.value
+
+
+def gemm_grid(tile, M, N, split_k=1):
+    return _lib.load().cusync_gemm_grid(tile, M, N, split_k).tup()
+
+
+def gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, epilogue=EPI.NONE, a_mode=0, split_k=1,
+              max_workgroups=0):
+    a = GemmArgs()
+    a.stage = stage.desc
+    a.M, a.N, a.K = M, N, K
+    a.A, a.lda, a.B, a.ldb, a.D, a.ldd = A, lda, B, ldb, D, ldd
+    a.epilogue, a.a_mode, a.tile, a.split_k = epilogue, a_mode, tile, split_k
+    a.workspace = None
+    a.max_workgroups = max_workgroups
+    return a
+
+
+def gemm(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, stream=None, **kw):
+    """Launch one sync-aware GEMM; pointers are raw device addresses."""
+    a = gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, **kw)
+    return _lib.load().cusync_gemm_run(C.byref(a), stream)
+
+
+# ---- MLP chain -------------------------------------------------------------------
+
+class Mlp:
+    """Handle over cusync_mlp_* (the reference's libmlp C surface, src/ml-bench/transformer/mlp-lib.cu:555-618)."""
+
+    def __init__(self, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=-1, tile2=-1, opts=-1, activation=1):
+        self.L = _lib.load()
+        self.cfg = MlpConfig(model, batch, hidden, inner, sync, tile1, tile2, opts, activation)
+        self.h = self.L.cusync_mlp_create(C.byref(self.cfg), w1_ptr, w2_ptr)
+        if not self.h:
+            raise RuntimeError("cusync_mlp_create failed: " + last_error())
+
+    def run(self, x_ptr, h_ptr, y_ptr, runs=1, split=False):
+        times = (C.c_double * runs)()
+        if split:
+            g1 = (C.c_double * runs)()
+            g2 = (C.c_double * runs)()
+            check(self.L.cusync_mlp_run_split(self.h, x_ptr, h_ptr, y_ptr, runs, times, g1, g2), "cusync_mlp_run_split")
+            return list(times), list(g1), list(g2)
+        check(self.L.cusync_mlp_run(self.h, x_ptr, h_ptr, y_ptr, runs, times), "cusync_mlp_run")
+        return list(times)
+
+    def tiles(self):
+        a, b = C.c_int(0), C.c_int(0)
+        self.L.cusync_mlp_tiles(self.h, C.byref(a), C.byref(b))
+        return a.value, b.value
+
+    def stage_state(self, which):
+        import numpy as np
+        d = self.L.cusync_mlp_stage(self.h, which).contents
+        g = d.grid
+        n = g.x * g.y * g.z
+        sems = np.zeros(n, np.uint32)
+        order = np.zeros((n, 3), np.uint32)
+        tc, sc, ke, to = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+        producer = d.out.kind != POLICY.NOSYNC
+        check(self.L.cusync_stage_read_state(C.byref(d), sems.ctypes.data_as(C.c_void_p) if producer else None,
+                                             order.ctypes.data_as(C.c_void_p), C.byref(tc), C.byref(sc),
+                                             C.byref(ke), C.byref(to)), "read_state")
+        return SimpleNamespace(desc=d, grid=g.tup(), sems=sems, tile_order=order, tile_counter=tc.value,
+                               start_counter=sc.value, kernel_executed=ke.value, spin_timeouts=to.value)
+
+    def destroy(self):
+        if self.h:
+            self.L.cusync_mlp_destroy(self.h)
+            self.h = None

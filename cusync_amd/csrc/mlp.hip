@@ -1,0 +1,242 @@
+// MLP chain: two dependent GEMMs, X*W1 (+activation) -> H, H*W2 -> Y, run either
+// stream-ordered (kernel-boundary sync) or as a CuSync producer/consumer pair on
+// two streams.  Host code only; the kernels are launched through
+// cusync_gemm_run.  Stands in for the hot loops of the reference driver
+// (src/ml-bench/transformer/mlp.cu:411-491 runBaselineGPT3, :645-716
+// runCuSyncGPT3, :718-862 runCuSyncLLaMA) and for the C surface of
+// src/ml-bench/transformer/mlp-lib.cu:555-618.
+#include <hip/hip_runtime.h>
+
+#include <string.h>
+#include <string>
+
+#include "../../include/cusync_amd.h"
+#include "rt_internal.h"
+
+struct cusync_mlp {
+  cusync_mlp_config cfg;
+  const void* w1;
+  const void* w2;
+  int tile1, tile2;
+  uint32_t n1, k1, n2, k2;          // GEMM1 is [batch,k1]x[k1,n1], GEMM2 is [batch,k2]x[k2,n2]
+  uint32_t ldh;                      // row pitch of the intermediate
+  int epilogue1, aMode2;
+  cusync_stage_desc prod, cons;
+  hipStream_t sProd, sCons;
+  hipEvent_t eStart, eMid, eEnd;
+};
+
+namespace {
+
+using cusync::rt::setError;
+
+// Built-in choice of tile shapes per batch size for 256 CUs.  Rows of the output
+// decide the M extent; the N extent is picked so that the number of tiles of the
+// two GEMMs together stays close to a multiple of what the device holds.
+void pickTiles(const cusync_mlp_config& c, int* t1, int* t2) {
+  int t;
+  if (c.batch <= 32) t = CUSYNC_TILE_32x128x64;
+  else if (c.batch <= 64) t = CUSYNC_TILE_64x128x64;
+  else if (c.batch <= 128) t = CUSYNC_TILE_128x128x64;
+  else t = CUSYNC_TILE_256x128x64;
+  if (c.model == CUSYNC_MLP_LLAMA && c.inner % 128 != 0) {
+    // gate|up split must fall on a tile boundary (2752 = 43 * 64)
+    t = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
+  }
+  *t1 = c.tile1 >= 0 ? c.tile1 : t;
+  *t2 = c.tile2 >= 0 ? c.tile2 : (c.model == CUSYNC_MLP_LLAMA && c.inner % 128 != 0
+                                      ? (c.batch <= 128 ? CUSYNC_TILE_128x128x64 : CUSYNC_TILE_256x128x64) : t);
+}
+
+cusync_policy_desc noSync() {
+  cusync_policy_desc p;
+  memset(&p, 0, sizeof p);
+  p.kind = CUSYNC_POLICY_NOSYNC;
+  p.tileM = p.tileN = 1; p.R = p.S = 1;
+  return p;
+}
+
+cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h, void* y) {
+  cusync_gemm_args a;
+  memset(&a, 0, sizeof a);
+  a.M = m->cfg.batch;
+  a.split_k = 1;
+  if (which == 0) {
+    a.stage = m->prod;
+    a.N = m->n1; a.K = m->k1;
+    a.A = x; a.lda = m->k1;
+    a.B = m->w1; a.ldb = m->n1;
+    a.D = h; a.ldd = m->ldh;
+    a.epilogue = m->epilogue1;
+    a.a_mode = CUSYNC_A_PLAIN;
+    a.tile = m->tile1;
+  } else {
+    a.stage = m->cons;
+    a.N = m->n2; a.K = m->k2;
+    a.A = h; a.lda = m->ldh;
+    a.B = m->w2; a.ldb = m->n2;
+    a.D = y; a.ldd = m->n2;
+    a.epilogue = CUSYNC_EPILOGUE_NONE;
+    a.a_mode = m->aMode2;
+    a.tile = m->tile2;
+  }
+  return a;
+}
+
+}  // namespace
+
+extern "C" {
+
+cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, const void* w2) {
+  if (!cfg || !w1 || !w2) { setError("mlp: null argument"); return nullptr; }
+  if (cfg->batch == 0 || cfg->hidden == 0 || cfg->inner == 0) { setError("mlp: empty shape"); return nullptr; }
+  cusync_mlp* m = new cusync_mlp();
+  m->cfg = *cfg;
+  m->w1 = w1; m->w2 = w2;
+  const bool llama = cfg->model == CUSYNC_MLP_LLAMA;
+  m->k1 = cfg->hidden;
+  m->n1 = llama ? 2 * cfg->inner : cfg->inner;
+  m->k2 = cfg->inner;
+  m->n2 = cfg->hidden;
+  m->ldh = m->n1;
+  m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : CUSYNC_EPILOGUE_NONE;
+  m->aMode2 = (llama && cfg->activation) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  pickTiles(*cfg, &m->tile1, &m->tile2);
+
+  uint32_t tm1 = 0, tn1 = 0;
+  if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
+    setError("mlp: unknown tile id");
+    delete m;
+    return nullptr;
+  }
+
+  int sync = cfg->sync;
+  if (llama && sync == CUSYNC_SYNC_TILE && m->aMode2 == CUSYNC_A_SWIGLU) sync = CUSYNC_SYNC_STRIDED;
+  cusync_policy_desc pol = noSync();
+  int opts = 0;
+  const cusync_dim3 g1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, 1);
+  const cusync_dim3 g2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, 1);
+  switch (sync) {
+    case CUSYNC_SYNC_STREAM:
+      break;
+    case CUSYNC_SYNC_ROW:        // RowSync(gridDim1.n()), src/ml-bench/transformer/mlp.cu:1032-1034
+      pol.kind = CUSYNC_POLICY_ROWSYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      pol.tileM = tm1; pol.tileN = 1; pol.waitValue = g1.x; pol.postValue = 1;
+      break;
+    case CUSYNC_SYNC_TILE:       // TileSync<TransposeXY,kM,kN> + NoAtomicAdd + ReorderTileLoads, mlp.cu:9-16,111
+      pol.kind = CUSYNC_POLICY_TILESYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      pol.tileM = tm1; pol.tileN = tn1; pol.waitValue = 1; pol.postValue = 1;
+      opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
+      break;
+    case CUSYNC_SYNC_STRIDED:    // StridedSync<TransposeXY,d,kM,kN,2>, mlp.cu:109; atomic add kept (:9-14)
+      if (!llama) { setError("mlp: StridedSync is for the gate|up layout"); delete m; return nullptr; }
+      if (cfg->inner % tn1 != 0) { setError("mlp: StridedSync needs inner % tileN == 0"); delete m; return nullptr; }
+      pol.kind = CUSYNC_POLICY_STRIDEDSYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      pol.tileM = tm1; pol.tileN = tn1; pol.waitValue = 2; pol.postValue = 1;
+      pol.gridN = cfg->inner; pol.stride = 2;
+      opts = CUSYNC_OPT_REORDER_TILE_LOADS;
+      break;
+    default:
+      setError("mlp: unknown sync mode");
+      delete m;
+      return nullptr;
+  }
+  if (cfg->opts >= 0) opts |= cfg->opts;
+
+  memset(&m->prod, 0, sizeof m->prod);
+  memset(&m->cons, 0, sizeof m->cons);
+  m->prod.grid = g1; m->prod.tileSize = {1, 1, 1}; m->prod.iter = 1; m->prod.opts = opts;
+  m->prod.in = noSync(); m->prod.out = pol;
+  m->cons.grid = g2; m->cons.tileSize = {1, 1, 1}; m->cons.iter = 1; m->cons.opts = opts;
+  m->cons.in = pol; m->cons.out = noSync();
+  if (cusync_stage_create(&m->prod, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS ||
+      cusync_stage_create(&m->cons, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) {
+    delete m;
+    return nullptr;
+  }
+  if (sync != CUSYNC_SYNC_STREAM &&
+      cusync_set_producer_consumer_pair(&m->prod, &m->cons) != CUSYNC_SUCCESS) {
+    setError("mlp: pairing the stages failed");
+    delete m;
+    return nullptr;
+  }
+  if (CUSYNC_HIP(hipStreamCreateWithFlags(&m->sProd, hipStreamNonBlocking)) ||
+      CUSYNC_HIP(hipStreamCreateWithFlags(&m->sCons, hipStreamNonBlocking)) ||
+      CUSYNC_HIP(hipEventCreate(&m->eStart)) || CUSYNC_HIP(hipEventCreate(&m->eMid)) ||
+      CUSYNC_HIP(hipEventCreate(&m->eEnd))) {
+    delete m;
+    return nullptr;
+  }
+  return m;
+}
+
+void cusync_mlp_destroy(cusync_mlp* m) {
+  if (!m) return;
+  (void)hipStreamSynchronize(m->sProd);
+  (void)hipStreamSynchronize(m->sCons);
+  cusync_stage_free(&m->prod);
+  cusync_stage_free(&m->cons);
+  (void)hipEventDestroy(m->eStart); (void)hipEventDestroy(m->eMid); (void)hipEventDestroy(m->eEnd);
+  (void)hipStreamDestroy(m->sProd); (void)hipStreamDestroy(m->sCons);
+  delete m;
+}
+
+cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y, int runs,
+                                  double* times_us, double* gemm1_us, double* gemm2_us) {
+  if (!m || !x || !h || !y) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const bool overlapped = m->prod.out.kind != CUSYNC_POLICY_NOSYNC;
+  for (int r = 0; r < runs; r++) {
+    cusync_gemm_args a1 = gemmArgs(m, 0, x, h, y);
+    cusync_gemm_args a2 = gemmArgs(m, 1, x, h, y);
+    cusync_error e;
+    if (CUSYNC_HIP(hipEventRecord(m->eStart, m->sProd))) return CUSYNC_ERROR_DEVICE;
+    if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) return e;
+    if (overlapped) {
+      if ((e = cusync_invoke_wait_kernel(&m->prod, m->sCons)) != CUSYNC_SUCCESS) return e;
+      if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;
+      if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sCons))) return CUSYNC_ERROR_DEVICE;
+    } else {
+      if (CUSYNC_HIP(hipEventRecord(m->eMid, m->sProd))) return CUSYNC_ERROR_DEVICE;
+      if ((e = cusync_gemm_run(&a2, m->sProd)) != CUSYNC_SUCCESS) return e;
+      if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sProd))) return CUSYNC_ERROR_DEVICE;
+    }
+    if (CUSYNC_HIP(hipEventSynchronize(m->eEnd))) return CUSYNC_ERROR_DEVICE;
+    // The consumer finishing implies every producer tile was posted, but the
+    // producer kernel itself must have retired before its stage is reused.
+    if (overlapped && CUSYNC_HIP(hipStreamSynchronize(m->sProd))) return CUSYNC_ERROR_DEVICE;
+    float ms = 0;
+    if (times_us) {
+      if (CUSYNC_HIP(hipEventElapsedTime(&ms, m->eStart, m->eEnd))) return CUSYNC_ERROR_DEVICE;
+      times_us[r] = (double)ms * 1000.0;
+    }
+    if (!overlapped && gemm1_us) {
+      if (CUSYNC_HIP(hipEventElapsedTime(&ms, m->eStart, m->eMid))) return CUSYNC_ERROR_DEVICE;
+      gemm1_us[r] = (double)ms * 1000.0;
+    }
+    if (!overlapped && gemm2_us) {
+      if (CUSYNC_HIP(hipEventElapsedTime(&ms, m->eMid, m->eEnd))) return CUSYNC_ERROR_DEVICE;
+      gemm2_us[r] = (double)ms * 1000.0;
+    }
+    m->prod.iter += 1;     // incrementIter on both stages, mlp.cu:709-712
+    m->cons.iter += 1;
+  }
+  return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_mlp_run(cusync_mlp* m, const void* x, void* h, void* y, int runs, double* times_us) {
+  return cusync_mlp_run_split(m, x, h, y, runs, times_us, nullptr, nullptr);
+}
+
+const cusync_stage_desc* cusync_mlp_stage(const cusync_mlp* m, int which) {
+  if (!m) return nullptr;
+  return which == 0 ? &m->prod : &m->cons;
+}
+
+int cusync_mlp_tiles(const cusync_mlp* m, int* tile1, int* tile2) {
+  if (!m) return 1;
+  if (tile1) *tile1 = m->tile1;
+  if (tile2) *tile2 = m->tile2;
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,222 @@
+// Thin runtime layer of libcusync_amd.so: the only translation unit besides the
+// kernel launchers that calls the HIP runtime.  Implements the cusync_rt_*,
+// cusync_stage_* and wait-kernel entry points declared in include/cusync_amd.h.
+#include <hip/hip_runtime.h>
+
+#include <stdio.h>
+#include <string.h>
+#include <string>
+#include <vector>
+
+#include "../../include/cusync_amd.h"
+#include "../../include/cusync/device-functions.h"
+#include "policy_eval.h"
+#include "rt_internal.h"
+
+namespace cusync {
+namespace rt {
+
+static thread_local std::string g_last_error;
+
+void setError(const std::string& msg) { g_last_error = msg; }
+
+int check(hipError_t e, const char* what, const char* file, int line) {
+  if (e == hipSuccess) return 0;
+  char buf[512];
+  snprintf(buf, sizeof buf, "%s failed at %s:%d: %s", what, file, line, hipGetErrorString(e));
+  g_last_error = buf;
+  return (int)e;
+}
+
+}  // namespace rt
+}  // namespace cusync
+
+#define RT(call) CUSYNC_HIP(call)
+
+// One wave; lane 0 polls.  Same contract as waitKernel of the reference
+// (src/cusync.cu:11-19) with a bounded spin.
+__global__ void cusync_wait_kernel_impl(const uint32_t* semaphore, uint32_t value) {
+  if (threadIdx.x == 0) cusync::dev::spinUntilAtLeast(semaphore, value);
+}
+
+extern "C" {
+
+const char* cusync_rt_last_error(void) { return cusync::rt::g_last_error.c_str(); }
+
+int cusync_rt_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+int cusync_rt_device_info(int* num_cus, int* clock_khz, size_t* lds_per_cu, size_t* hbm_bytes,
+                          char* name, size_t name_len) {
+  hipDeviceProp_t p;
+  int dev = 0;
+  if (RT(hipGetDevice(&dev))) return 1;
+  if (RT(hipGetDeviceProperties(&p, dev))) return 1;
+  if (num_cus) *num_cus = p.multiProcessorCount;
+  if (clock_khz) *clock_khz = p.clockRate;
+  if (lds_per_cu) *lds_per_cu = p.maxSharedMemoryPerMultiProcessor;
+  if (hbm_bytes) *hbm_bytes = p.totalGlobalMem;
+  if (name && name_len) { strncpy(name, p.gcnArchName, name_len - 1); name[name_len - 1] = 0; }
+  return 0;
+}
+
+int cusync_rt_malloc(void** ptr, size_t bytes) { return RT(hipMalloc(ptr, bytes)); }
+int cusync_rt_free(void* ptr) { return RT(hipFree(ptr)); }
+int cusync_rt_memset(void* ptr, int value, size_t bytes) { return RT(hipMemset(ptr, value, bytes)); }
+int cusync_rt_memcpy_h2d(void* dst, const void* src, size_t bytes) { return RT(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); }
+int cusync_rt_memcpy_d2h(void* dst, const void* src, size_t bytes) { return RT(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); }
+int cusync_rt_memcpy_d2d(void* dst, const void* src, size_t bytes) { return RT(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice)); }
+// Default priority on purpose: the chain's forward progress does not depend on
+// queue priorities (see stage_device.h).
+int cusync_rt_stream_create(void** stream) { return RT(hipStreamCreateWithFlags((hipStream_t*)stream, hipStreamNonBlocking)); }
+int cusync_rt_stream_destroy(void* stream) { return RT(hipStreamDestroy((hipStream_t)stream)); }
+int cusync_rt_stream_sync(void* stream) { return RT(hipStreamSynchronize((hipStream_t)stream)); }
+int cusync_rt_device_sync(void) { return RT(hipDeviceSynchronize()); }
+int cusync_rt_event_create(void** event) { return RT(hipEventCreate((hipEvent_t*)event)); }
+int cusync_rt_event_destroy(void* event) { return RT(hipEventDestroy((hipEvent_t)event)); }
+int cusync_rt_event_record(void* event, void* stream) { return RT(hipEventRecord((hipEvent_t)event, (hipStream_t)stream)); }
+int cusync_rt_event_sync(void* event) { return RT(hipEventSynchronize((hipEvent_t)event)); }
+int cusync_rt_event_elapsed_us(void* start, void* end, double* us) {
+  float ms = 0;
+  int rc = RT(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)end));
+  if (us) *us = (double)ms * 1000.0;
+  return rc;
+}
+int cusync_rt_stream_wait_event(void* stream, void* event) { return RT(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)); }
+
+/* ---- stages --------------------------------------------------------------- */
+
+static uint32_t numTiles(const cusync_stage_desc* d) { return d->grid.x * d->grid.y * d->grid.z; }
+
+cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_tile_order) {
+  if (!d || !host_tile_order) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const uint32_t n = numTiles(d);
+  if (n == 0) { cusync::rt::setError("cusync_stage_alloc: empty grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr;
+  d->kernelExecuted = nullptr; d->spinTimeouts = nullptr; d->tileStatusWrite = nullptr;
+  // The three small counters share one allocation: [tileCounter, startCounter, spinTimeouts, kernelExecuted]
+  // each on its own 128-byte line so that polling one does not disturb the others.
+  const size_t line = 128;
+  char* counters = nullptr;
+  if (RT(hipMalloc((void**)&counters, 4 * line))) return CUSYNC_ERROR_DEVICE;
+  if (RT(hipMemset(counters, 0, 4 * line))) return CUSYNC_ERROR_DEVICE;
+  d->tileCounter = (uint32_t*)(counters);
+  d->startCounter = (uint32_t*)(counters + line);
+  d->spinTimeouts = (uint32_t*)(counters + 2 * line);
+  const bool producer = d->out.kind != CUSYNC_POLICY_NOSYNC;
+  if (producer && !(d->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) d->kernelExecuted = (uint32_t*)(counters + 3 * line);
+  if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return CUSYNC_ERROR_DEVICE;
+  if (RT(hipMemcpy(d->tileOrder, host_tile_order, sizeof(cusync_dim3) * n, hipMemcpyHostToDevice))) return CUSYNC_ERROR_DEVICE;
+  if (producer) {
+    if (RT(hipMalloc((void**)&d->tileStatusWrite, sizeof(uint32_t) * n))) return CUSYNC_ERROR_DEVICE;
+    if (RT(hipMemset(d->tileStatusWrite, 0, sizeof(uint32_t) * n))) return CUSYNC_ERROR_DEVICE;
+  }
+  return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_stage_free(cusync_stage_desc* d) {
+  if (!d) return CUSYNC_ERROR_NOT_INITIALIZED;
+  int bad = 0;
+  if (d->tileCounter) bad |= RT(hipFree(d->tileCounter));       // base of the counters block
+  if (d->tileOrder) bad |= RT(hipFree(d->tileOrder));
+  if (d->tileStatusWrite) bad |= RT(hipFree(d->tileStatusWrite));
+  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr;
+  d->kernelExecuted = nullptr; d->spinTimeouts = nullptr; d->tileStatusWrite = nullptr;
+  return bad ? CUSYNC_ERROR_DEVICE : CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_stage_create(cusync_stage_desc* d, int order) {
+  if (!d) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const uint32_t n = numTiles(d);
+  if (n == 0) { cusync::rt::setError("cusync_stage_create: empty grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  std::vector<cusync_dim3> host(n);
+  std::vector<char> taken(n, 0);
+  bool bad = false;
+  for (uint32_t z = 0; z < d->grid.z; z++)
+    for (uint32_t y = 0; y < d->grid.y; y++)
+      for (uint32_t x = 0; x < d->grid.x; x++) {
+        cusync_dim3 b = {x, y, z};
+        const uint32_t id = cusync::dyn::blockIndex(order, d->grid, b);
+        if (id >= n || taken[id]) { bad = true; continue; }
+        taken[id] = 1;
+        host[id] = b;
+      }
+  d->iter = d->iter > 0 ? d->iter : 1;
+  cusync_error e = cusync_stage_alloc(d, host.data());
+  if (e != CUSYNC_SUCCESS) return e;
+  return bad ? CUSYNC_ERROR_INVALID_LINEAR_BLOCK_INDEX : CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc* prod, cusync_stage_desc* cons) {
+  if (!prod || !cons) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
+  if (cons->in.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_CONSUMER;
+  if (prod->tileStatusWrite == nullptr) return CUSYNC_ERROR_NOT_INITIALIZED;
+  cons->prodGrid = prod->grid;
+  cons->tileStatusRead = prod->tileStatusWrite;
+  return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_wait_kernel(uint32_t* semaphore, uint32_t value, void* stream) {
+  if (!semaphore) return CUSYNC_ERROR_NOT_INITIALIZED;
+  hipLaunchKernelGGL(cusync_wait_kernel_impl, dim3(1), dim3(64), 0, (hipStream_t)stream, semaphore, value);
+  if (RT(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc* prod, void* stream) {
+  if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
+  if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
+  return cusync_wait_kernel(prod->kernelExecuted, (uint32_t)prod->iter, stream);
+}
+
+cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems, cusync_dim3* tile_order,
+                                     uint32_t* tile_counter, uint32_t* start_counter,
+                                     uint32_t* kernel_executed, uint32_t* spin_timeouts) {
+  if (!d) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const uint32_t n = numTiles(d);
+  int bad = 0;
+  if (sems) {
+    if (!d->tileStatusWrite) return CUSYNC_ERROR_NOT_PRODUCER;
+    bad |= RT(hipMemcpy(sems, d->tileStatusWrite, sizeof(uint32_t) * n, hipMemcpyDeviceToHost));
+  }
+  if (tile_order) bad |= RT(hipMemcpy(tile_order, d->tileOrder, sizeof(cusync_dim3) * n, hipMemcpyDeviceToHost));
+  if (tile_counter) bad |= RT(hipMemcpy(tile_counter, d->tileCounter, 4, hipMemcpyDeviceToHost));
+  if (start_counter) bad |= RT(hipMemcpy(start_counter, d->startCounter, 4, hipMemcpyDeviceToHost));
+  if (spin_timeouts) bad |= RT(hipMemcpy(spin_timeouts, d->spinTimeouts, 4, hipMemcpyDeviceToHost));
+  if (kernel_executed) {
+    *kernel_executed = 0;
+    if (d->kernelExecuted) bad |= RT(hipMemcpy(kernel_executed, d->kernelExecuted, 4, hipMemcpyDeviceToHost));
+  }
+  return bad ? CUSYNC_ERROR_DEVICE : CUSYNC_SUCCESS;
+}
+
+/* ---- host evaluation of policies -------------------------------------------- */
+
+uint32_t cusync_policy_tile_index(const cusync_policy_desc* p, cusync_dim3 tile, cusync_dim3 grid) {
+  return cusync::dyn::tileIndex(*p, tile, grid);
+}
+uint32_t cusync_policy_wait_value(const cusync_policy_desc* p, cusync_dim3 tile, cusync_dim3 grid) {
+  (void)tile; (void)grid;
+  return cusync::dyn::waitValue(*p);
+}
+uint32_t cusync_policy_post_value(const cusync_policy_desc* p, cusync_dim3 tile, cusync_dim3 grid) {
+  (void)tile; (void)grid;
+  return cusync::dyn::postValue(*p);
+}
+int cusync_policy_is_sync(const cusync_policy_desc* p, cusync_dim3 tile, cusync_dim3 grid) {
+  (void)grid;
+  return cusync::dyn::isSync(*p, tile) ? 1 : 0;
+}
+uint32_t cusync_order_block_index(int order, cusync_dim3 grid, cusync_dim3 block) {
+  return cusync::dyn::blockIndex(order, grid, block);
+}
+cusync_dim3 cusync_order_tile_to_block(int order, cusync_dim3 tile) {
+  return cusync::dyn::tileToBlock(order, tile);
+}
+
+}  // extern "C"

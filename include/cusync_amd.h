@@ -1,0 +1,257 @@
+/*
+ * cusync_amd.h — C ABI of the MI355X-native CuSync library (libcusync_amd.so).
+ *
+ * Plain C types only: pointers, sizes and PODs.  Everything above this line of
+ * the stack (the C++ CuStage API in include/cusync/, the drivers, the Python
+ * test harness) reaches the GPU exclusively through these entry points.
+ *
+ * Each entry point names the interface of the reference (microsoft/cusync) it
+ * stands in for.  Reference paths:
+ *   CS = src/include/cusync
+ *   CC = src/include/cutlass/cusync-cutlass/include/cutlass
+ *   TB = src/ml-bench/transformer     CV = src/ml-bench/volta_conv2d
+ */
+#ifndef CUSYNC_AMD_H
+#define CUSYNC_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* PODs                                                                       */
+/* ------------------------------------------------------------------------- */
+
+typedef struct cusync_dim3 { uint32_t x, y, z; } cusync_dim3;
+
+/* CS/cusync.h:46-53 — same enumerators in the same order; success is 5. */
+typedef enum cusync_error {
+  CUSYNC_ERROR_NOT_PRODUCER = 0,
+  CUSYNC_ERROR_NOT_CONSUMER = 1,
+  CUSYNC_ERROR_NOT_INITIALIZED = 2,
+  CUSYNC_ERROR_INVALID_LINEAR_BLOCK_INDEX = 3,
+  CUSYNC_ERROR_DEVICE = 4,            /* CuSyncErrorCUDAError */
+  CUSYNC_SUCCESS = 5
+} cusync_error;
+
+/* CS/cusync.h:69-75 */
+enum {
+  CUSYNC_OPT_NONE = 0,
+  CUSYNC_OPT_NO_ATOMIC_ADD = 1 << 0,
+  CUSYNC_OPT_AVOID_WAIT_KERNEL = 1 << 1,
+  CUSYNC_OPT_AVOID_CUSTOM_ORDER = 1 << 2,
+  CUSYNC_OPT_REORDER_TILE_LOADS = 1 << 3
+};
+
+/* CS/tile-orders.h:50-76 */
+enum { CUSYNC_ORDER_IDENTITY = 0, CUSYNC_ORDER_TRANSPOSE_XY = 1 };
+
+/* CS/policies.h:18-210; StridedSync TB/mlp.cu:76-101; ConsecutiveSync TB/attention.cu:51-70 */
+enum {
+  CUSYNC_POLICY_NOSYNC = 0,
+  CUSYNC_POLICY_ROWSYNC = 1,
+  CUSYNC_POLICY_TILESYNC = 2,
+  CUSYNC_POLICY_STRIDEDSYNC = 3,
+  CUSYNC_POLICY_CONV2DTILESYNC = 4,
+  CUSYNC_POLICY_CONSECUTIVESYNC = 5
+};
+
+/* Run-time image of a policy type: its template arguments and its two members. */
+typedef struct cusync_policy_desc {
+  int32_t kind;
+  int32_t order;
+  uint32_t tileM, tileN;
+  uint32_t waitValue, postValue;
+  uint32_t gridN, stride;     /* StridedSync<Order, GridN, TileM, TileN, stride> */
+  uint32_t R, S;              /* Conv2DTileSync<Order, R, S, TileM, TileN> */
+  uint32_t H;                 /* ConsecutiveSync<Order, H, TileM, TileN> */
+} cusync_policy_desc;
+
+/* Run-time image of a CuStage object (CS/cusync.h:93-117): what a kernel gets
+ * by value.  Device pointers are owned by whoever called cusync_stage_alloc. */
+typedef struct cusync_stage_desc {
+  cusync_dim3 grid;           /* grid_     : logical tile grid of this stage */
+  cusync_dim3 prodGrid;       /* prodGrid_ : logical tile grid of its producer */
+  cusync_dim3 tileSize;       /* tileSize_ : stored, never read (as in the reference) */
+  int32_t iter;               /* run counter, starts at 1 */
+  int32_t opts;               /* CUSYNC_OPT_* bits */
+  cusync_policy_desc in;      /* inputPolicy_  */
+  cusync_policy_desc out;     /* outputPolicy_ */
+  cusync_dim3 *tileOrder;     /* [numTiles] ticket -> tile */
+  uint32_t *tileCounter;      /* ticket dispenser; 0 between runs */
+  uint32_t *startCounter;     /* counts workgroups that have begun; 0 between runs */
+  uint32_t *kernelExecuted;   /* wait-kernel flag: == iter once every workgroup of the run has begun */
+  uint32_t *spinTimeouts;     /* number of waits of this stage that gave up (0 in a healthy chain) */
+  uint32_t *tileStatusWrite;  /* semaphores this stage posts */
+  uint32_t *tileStatusRead;   /* semaphores this stage waits on (its producer's) */
+} cusync_stage_desc;
+
+/* ------------------------------------------------------------------------- */
+/* Thin runtime layer (replaces the cudaMalloc/Memset/Memcpy/stream/event     */
+/* calls made directly by CS/cusync.h:125-198 and the drivers)                */
+/* ------------------------------------------------------------------------- */
+
+const char *cusync_rt_last_error(void);            /* text of the last failed HIP call, "" if none */
+int cusync_rt_device_count(void);
+int cusync_rt_device_info(int *num_cus, int *clock_khz, size_t *lds_per_cu, size_t *hbm_bytes,
+                          char *name, size_t name_len);
+int cusync_rt_malloc(void **ptr, size_t bytes);     /* 0 on success */
+int cusync_rt_free(void *ptr);
+int cusync_rt_memset(void *ptr, int value, size_t bytes);
+int cusync_rt_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int cusync_rt_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int cusync_rt_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int cusync_rt_stream_create(void **stream);         /* non-blocking stream, default priority */
+int cusync_rt_stream_destroy(void *stream);
+int cusync_rt_stream_sync(void *stream);
+int cusync_rt_device_sync(void);
+int cusync_rt_event_create(void **event);
+int cusync_rt_event_destroy(void *event);
+int cusync_rt_event_record(void *event, void *stream);
+int cusync_rt_event_sync(void *event);
+int cusync_rt_event_elapsed_us(void *start, void *end, double *us);
+int cusync_rt_stream_wait_event(void *stream, void *event);
+
+/* ------------------------------------------------------------------------- */
+/* Stage life cycle                                                           */
+/* ------------------------------------------------------------------------- */
+
+/* Replaces the device half of the CuStage constructor (CS/cusync.h:176-198) and
+ * buildScheduleBuffer (:125-157): uploads host_tile_order[numTiles], zeroes the
+ * ticket and start counters, and for a producer allocates numTiles zeroed
+ * semaphores plus the wait-kernel flag (skipped with AVOID_WAIT_KERNEL).
+ * desc->grid/opts/in/out must be filled in; pointer members are written. */
+cusync_error cusync_stage_alloc(cusync_stage_desc *desc, const cusync_dim3 *host_tile_order);
+/* The reference never frees (no destructor); this does.  Only call on the
+ * descriptor that was passed to cusync_stage_alloc, not on copies. */
+cusync_error cusync_stage_free(cusync_stage_desc *desc);
+/* Same result as cusync_stage_alloc with the tile order generated from
+ * desc->grid for one of the two built-in orders. */
+cusync_error cusync_stage_create(cusync_stage_desc *desc, int order);
+/* CuSync::setProducerConsumerPair (CS/cusync.h:289-298). */
+cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc *prod, cusync_stage_desc *cons);
+/* CuStage::invokeWaitKernel (CS/cusync.h:203-209) + src/cusync.cu:11-25:
+ * enqueues a one-wave kernel on `stream` that returns once the producer's flag
+ * has reached desc->iter.  No-op with AVOID_WAIT_KERNEL. */
+cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc *prod, void *stream);
+/* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
+cusync_error cusync_wait_kernel(uint32_t *semaphore, uint32_t value, void *stream);
+/* Reads back device state for tests (the reference reaches it through the
+ * friend class CuSyncTest, CS/cusync.h:120, tests/cusync-test.h). Any output
+ * pointer may be NULL. sems must hold numTiles entries. */
+cusync_error cusync_stage_read_state(const cusync_stage_desc *desc, uint32_t *sems, cusync_dim3 *tile_order,
+                                     uint32_t *tile_counter, uint32_t *start_counter,
+                                     uint32_t *kernel_executed, uint32_t *spin_timeouts);
+
+/* Host evaluation of a policy / tile order, same arithmetic the device uses. */
+uint32_t cusync_policy_tile_index(const cusync_policy_desc *p, cusync_dim3 tile, cusync_dim3 grid);
+uint32_t cusync_policy_wait_value(const cusync_policy_desc *p, cusync_dim3 tile, cusync_dim3 grid);
+uint32_t cusync_policy_post_value(const cusync_policy_desc *p, cusync_dim3 tile, cusync_dim3 grid);
+int      cusync_policy_is_sync(const cusync_policy_desc *p, cusync_dim3 tile, cusync_dim3 grid);
+uint32_t cusync_order_block_index(int order, cusync_dim3 grid, cusync_dim3 block);
+cusync_dim3 cusync_order_tile_to_block(int order, cusync_dim3 tile);
+
+/* ------------------------------------------------------------------------- */
+/* Sync-aware fp16 GEMM (replaces cutlass::gemm::device::CuSyncGemm,          */
+/* CC/gemm/device/cusyncgemm.h:169-599 and its kernel CC/gemm/kernel/         */
+/* cusyncgemm.h:208-399)                                                      */
+/* ------------------------------------------------------------------------- */
+
+enum { CUSYNC_EPILOGUE_NONE = 0, CUSYNC_EPILOGUE_GELU = 1, CUSYNC_EPILOGUE_RELU = 2 };
+/* How the A operand is formed while it is staged into LDS. */
+enum {
+  CUSYNC_A_PLAIN = 0,
+  CUSYNC_A_SWIGLU = 1          /* A[m,k] = silu(G[m,k]) * G[m,k + K]; G has K*2 valid columns */
+};
+
+/* Tile shapes the library was built with. */
+enum {
+  CUSYNC_TILE_256x256x32 = 0,
+  CUSYNC_TILE_256x128x64 = 1,
+  CUSYNC_TILE_128x128x64 = 2,
+  CUSYNC_TILE_64x128x64 = 3,
+  CUSYNC_TILE_32x128x64 = 4,
+  CUSYNC_TILE_128x256x64 = 5,
+  CUSYNC_TILE_256x64x64 = 6,
+  CUSYNC_TILE_128x64x64 = 7,
+  CUSYNC_TILE_COUNT = 8
+};
+
+typedef struct cusync_gemm_args {
+  cusync_stage_desc stage;     /* Arguments::custage (cusyncgemm.h:293-350) */
+  uint32_t M, N, K;            /* problem_size */
+  const void *A; uint32_t lda; /* fp16 row-major [M,K] (or [M,2K] gate|up for CUSYNC_A_SWIGLU) */
+  const void *B; uint32_t ldb; /* fp16 row-major [K,N] */
+  void *D; uint32_t ldd;       /* fp16 row-major [M,N]; D = epilogue(A*B), alpha = 1, beta = 0 */
+  int32_t epilogue;            /* CUSYNC_EPILOGUE_* */
+  int32_t a_mode;              /* CUSYNC_A_* */
+  int32_t tile;                /* CUSYNC_TILE_* */
+  int32_t split_k;             /* k-slices; > 1 accumulates through `workspace` */
+  void *workspace;             /* split_k > 1: cusync_gemm_workspace_size bytes, zeroed once */
+  int32_t max_workgroups;      /* 0 = as many as stay resident; else cap on launched workgroups */
+} cusync_gemm_args;
+
+/* Tile extents of a CUSYNC_TILE_* id; returns 0 on success. */
+int cusync_gemm_tile_shape(int tile, uint32_t *tileM, uint32_t *tileN, uint32_t *tileK);
+/* Logical grid (n-tiles, m-tiles, k-slices): CuSyncGemmHorizontalThreadblockSwizzle
+ * get_tiled_shape + get_grid_shape (CC/gemm/threadblock/cusync_threadblock_swizzle.h:12-54). */
+cusync_dim3 cusync_gemm_grid(int tile, uint32_t M, uint32_t N, int split_k);
+/* can_implement (cusyncgemm.h:364-386): CUSYNC_SUCCESS or CUSYNC_ERROR_NOT_INITIALIZED
+ * with the reason in cusync_rt_last_error(). */
+cusync_error cusync_gemm_can_implement(const cusync_gemm_args *args);
+/* get_workspace_size (cusyncgemm.h:388-404). */
+size_t cusync_gemm_workspace_size(const cusync_gemm_args *args);
+/* Workgroups of this tile shape that stay resident on the device at once. */
+int cusync_gemm_max_resident(int tile);
+/* run(stream) (cusyncgemm.h:525-563).  args->stage.iter selects the run. */
+cusync_error cusync_gemm_run(const cusync_gemm_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* MLP chain (replaces the extern "C" surface of TB/mlp-lib.cu:555-618 and    */
+/* the hot loops runBaselineGPT3 / runCuSyncGPT3 / runCuSyncLLaMA,            */
+/* TB/mlp.cu:411-491, 645-716, 718-862)                                       */
+/* ------------------------------------------------------------------------- */
+
+enum { CUSYNC_MLP_GPT3 = 0, CUSYNC_MLP_LLAMA = 1 };
+enum { CUSYNC_SYNC_STREAM = 0,     /* kernel-boundary sync: both GEMMs on one stream */
+       CUSYNC_SYNC_ROW = 1, CUSYNC_SYNC_TILE = 2, CUSYNC_SYNC_STRIDED = 3 };
+
+typedef struct cusync_mlp_config {
+  int32_t model;               /* CUSYNC_MLP_* */
+  uint32_t batch;              /* rows of X */
+  uint32_t hidden;             /* H: 12288 (GPT-3) / 8192 (LLaMA) */
+  uint32_t inner;              /* columns of H1: 4H/8 = 6144 (GPT-3); d = 2752 or 2816 (LLaMA) */
+  int32_t sync;                /* CUSYNC_SYNC_* */
+  int32_t tile1, tile2;        /* CUSYNC_TILE_* per GEMM, -1 = pick from the built-in table */
+  int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = the reference's defaults for `sync` */
+  int32_t activation;          /* GPT-3: 1 = GeLU fused in GEMM1, 0 = none.  LLaMA: 1 = silu(g)*u fused
+                                  in GEMM2's A loader, 0 = GEMM2 reads the gate half as is (TB/mlp.cu:785-792) */
+} cusync_mlp_config;
+
+typedef struct cusync_mlp cusync_mlp;   /* opaque */
+
+/* initMLPParams / initCuSyncMLPParams (TB/mlp-lib.cu:555-567, 596-609).
+ * w1: [hidden, inner] (GPT-3) or [hidden, 2*inner] gate|up (LLaMA); w2: [inner, hidden]. */
+cusync_mlp *cusync_mlp_create(const cusync_mlp_config *cfg, const void *w1, const void *w2);
+void cusync_mlp_destroy(cusync_mlp *mlp);
+/* runLLAMA / runCuSyncLLAMA (TB/mlp-lib.cu:569-576, 611-618): `runs` back-to-back
+ * passes x -> h -> y.  h is the intermediate [batch, inner] (GPT-3) or
+ * [batch, 2*inner] (LLaMA).  If times_us != NULL it receives one elapsed time
+ * per run, measured with events start (producer stream) -> end (consumer stream)
+ * exactly as TB/mlp.cu:691-708; each run is then followed by an event wait. */
+cusync_error cusync_mlp_run(cusync_mlp *mlp, const void *x, void *h, void *y, int runs, double *times_us);
+/* Same, but also reports the two kernels' own durations (stream-ordered mode
+ * only; TB/mlp.cu:463-488). */
+cusync_error cusync_mlp_run_split(cusync_mlp *mlp, const void *x, void *h, void *y, int runs,
+                                  double *times_us, double *gemm1_us, double *gemm2_us);
+/* Device state of the two stages for tests (see cusync_stage_read_state). */
+const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer, 1 consumer */);
+int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUSYNC_AMD_H */

@@ -1,0 +1,213 @@
+// GPU test kernels written against the public C++ API (include/cusync/cusync.h),
+// the way a user of the library writes sync-aware kernels.  Built into
+// libcusync_stage_tests.so and driven from pytest through extern "C" entry points.
+//
+// Protocols follow the reference's own tests:
+//   run_simple_test  — tests/simple-test.cu:34-105 (two copy kernels synchronised
+//                      per block; data and semaphore values checked)
+//   run_two_matmuls  — src/examples/twoMatMuls/matrixMul.cu:41-121, 127-272 (two
+//                      chained 32x32-tiled fp32 GEMMs, consumer waits per k-tile)
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <vector>
+
+#include <cusync/cusync.h>
+
+#define HIP_OK(cmd) do { hipError_t e_ = (cmd); if (e_ != hipSuccess) { \
+  printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); return -1; } } while (0)
+
+namespace cusync {
+// Same role as tests/cusync-test.h of the reference: a friend of CuStage that
+// checks, from inside the consumer kernel, that the semaphore a block waited on
+// holds exactly expectedWaitValue * iter.
+class CuSyncTest {
+public:
+  char* semValid;   // device, one flag per stage
+  template<typename Stage>
+  __device__ void setSemValue(uint32_t stageIdx, dim3 tile, Stage& stage) {
+    if (!stage.isConsumer()) return;
+    if (threadIdx.x == 0 && threadIdx.y == 0) {
+      const bool eq = stage.expectedWaitValue(tile) * (uint32_t)stage.iter == stage.waitSemValue(tile);
+      if (!eq) semValid[stageIdx] = 0;
+    }
+  }
+  template<typename Stage> static int iterOf(Stage& s) { return s.iter; }
+};
+}  // namespace cusync
+
+using namespace cusync;
+
+template<typename Stage>
+__global__ void copyKernel(CuSyncTest cutest, Stage stage, int idx, const uint32_t* in, uint32_t* out) {
+  __shared__ int tileSh[3];
+  dim3 tile = stage.tile((dim3*)&tileSh[0]);
+  stage.wait(tile);
+  // The block copies the slice that belongs to the tile it was handed, so the
+  // data check also covers the ticket -> tile mapping.
+  const uint32_t linear = threadIdx.x + tile.x * blockDim.x;
+  out[linear] = in[linear];
+  stage.post(tile);
+  cutest.setSemValue(idx, tile, stage);
+}
+
+struct SimpleResult {
+  int32_t data_ok, sems_ok, prod_status, cons_status, pair_status, wait_status;
+  uint32_t tile_counter_prod, tile_counter_cons, kernel_executed, spin_timeouts;
+};
+
+template<typename Prod, typename Cons, typename Sync>
+static int runSimple(int iters, uint32_t blocks, SimpleResult* res, uint32_t* semsOut, uint32_t* orderOut) {
+  const uint32_t threadsPerBlock = 128;
+  const size_t size = (size_t)blocks * threadsPerBlock;
+  uint32_t *a1, *a2, *a3;
+  HIP_OK(hipMalloc(&a1, size * 4)); HIP_OK(hipMalloc(&a2, size * 4)); HIP_OK(hipMalloc(&a3, size * 4));
+  std::vector<uint32_t> host(size);
+  for (size_t i = 0; i < size; i++) host[i] = (uint32_t)i;
+  HIP_OK(hipMemcpy(a1, host.data(), size * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(a2, 0, size * 4)); HIP_OK(hipMemset(a3, 0, size * 4));
+  hipStream_t prodStream, consStream;
+  HIP_OK(hipStreamCreateWithFlags(&consStream, hipStreamNonBlocking));
+  HIP_OK(hipStreamCreateWithFlags(&prodStream, hipStreamNonBlocking));
+
+  dim3 threads(threadsPerBlock, 1, 1), grid(blocks, 1, 1);
+  Sync sync;
+  Prod prod(grid, threads, NoSync(), sync);
+  Cons cons(grid, threads, sync, NoSync());
+  res->prod_status = prod.status();
+  res->cons_status = cons.status();
+  res->pair_status = CuSync::setProducerConsumerPair(prod, cons);
+
+  CuSyncTest cutest;
+  HIP_OK(hipMalloc(&cutest.semValid, 1));
+  HIP_OK(hipMemset(cutest.semValid, 1, 1));
+
+  res->wait_status = CuSyncSuccess;
+  for (int i = 0; i < iters; i++) {
+    hipLaunchKernelGGL(copyKernel<Prod>, grid, threads, 0, prodStream, cutest, prod, -1, a1, a2);
+    int w = prod.invokeWaitKernel(consStream);
+    if (w != CuSyncSuccess) res->wait_status = w;
+    hipLaunchKernelGGL(copyKernel<Cons>, grid, threads, 0, consStream, cutest, cons, 0, a2, a3);
+    HIP_OK(hipDeviceSynchronize());
+    prod.incrementIter();
+    cons.incrementIter();
+  }
+
+  bool eq = true;
+  HIP_OK(hipMemcpy(host.data(), a2, size * 4, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < size; i++) eq = eq && host[i] == (uint32_t)i;
+  HIP_OK(hipMemcpy(host.data(), a3, size * 4, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < size; i++) eq = eq && host[i] == (uint32_t)i;
+  res->data_ok = eq;
+  char valid = 0;
+  HIP_OK(hipMemcpy(&valid, cutest.semValid, 1, hipMemcpyDeviceToHost));
+  res->sems_ok = valid;
+
+  cusync_stage_desc pd = prod.desc(), cd = cons.desc();
+  uint32_t startCounter = 0;
+  if (cusync_stage_read_state(&pd, semsOut, (cusync_dim3*)orderOut, &res->tile_counter_prod, &startCounter,
+                              &res->kernel_executed, nullptr) != CUSYNC_SUCCESS) return -1;
+  if (cusync_stage_read_state(&cd, nullptr, nullptr, &res->tile_counter_cons, nullptr, nullptr,
+                              &res->spin_timeouts) != CUSYNC_SUCCESS) return -1;
+
+  prod.destroy(); cons.destroy();
+  HIP_OK(hipFree(a1)); HIP_OK(hipFree(a2)); HIP_OK(hipFree(a3)); HIP_OK(hipFree(cutest.semValid));
+  HIP_OK(hipStreamDestroy(prodStream)); HIP_OK(hipStreamDestroy(consStream));
+  return 0;
+}
+
+// ---- two chained fp32 GEMMs on 32x32 tiles (user-written kernel) -------------
+
+const int BLOCK = 32;
+using MMSync = TileSync<IdentityOrder, BLOCK, BLOCK>;
+using MMProd = CuStage<IdentityOrder, NoSync, MMSync>;
+using MMCons = CuStage<IdentityOrder, MMSync, NoSync>;
+
+template<typename Stage>
+__global__ void tiledSgemm(Stage stage, float* C, const float* A, const float* B, int wA, int wB) {
+  __shared__ int tileSh[3];
+  __shared__ float As[BLOCK][BLOCK];
+  __shared__ float Bs[BLOCK][BLOCK];
+  dim3 t = stage.tile((dim3*)&tileSh[0]);
+  const int bx = t.x, by = t.y, tx = threadIdx.x, ty = threadIdx.y;
+  float sum = 0;
+  for (int k0 = 0; k0 < wA; k0 += BLOCK) {
+    // A's tile (columns k0.., rows by*32..) is the producer's output tile {k0/32, by}.
+    dim3 need((uint32_t)k0, (uint32_t)by * BLOCK, 1);
+    stage.wait(need);
+    As[ty][tx] = A[(by * BLOCK + ty) * wA + k0 + tx];
+    Bs[ty][tx] = B[(k0 + ty) * wB + bx * BLOCK + tx];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BLOCK; k++) sum += As[ty][k] * Bs[k][tx];
+    __syncthreads();
+  }
+  C[(by * BLOCK + ty) * wB + bx * BLOCK + tx] = sum;
+  stage.post(dim3((uint32_t)bx * BLOCK, (uint32_t)by * BLOCK, 0));
+}
+
+extern "C" {
+
+// variant: 0 none, 1 NoAtomicAdd, 2 AvoidCustomOrder (tests/simple-test.cu:107-137)
+int run_simple_test(int variant, int iters, uint32_t blocks, SimpleResult* res, uint32_t* semsOut, uint32_t* orderOut) {
+  using Sync = TileSync<IdentityOrder, 1, 1>;
+  if (variant == 0)
+    return runSimple<CuStage<IdentityOrder, NoSync, Sync>, CuStage<IdentityOrder, Sync, NoSync>, Sync>(iters, blocks, res, semsOut, orderOut);
+  if (variant == 1)
+    return runSimple<CuStage<IdentityOrder, NoSync, Sync, NoAtomicAdd>, CuStage<IdentityOrder, Sync, NoSync>, Sync>(iters, blocks, res, semsOut, orderOut);
+  if (variant == 2)
+    return runSimple<CuStage<IdentityOrder, NoSync, Sync, AvoidCustomOrder>, CuStage<IdentityOrder, Sync, NoSync>, Sync>(iters, blocks, res, semsOut, orderOut);
+  return -2;
+}
+
+// C = A*B then E = C*D, all n x n fp32 device pointers supplied by the caller.
+// semsOut receives the (n/32)^2 semaphores of the producer.
+int run_two_matmuls(int n, const float* A, const float* B, const float* D, float* C, float* E,
+                    uint32_t* semsOut, int* statusOut) {
+  if (n % BLOCK) return -2;
+  hipStream_t prodStream, consStream;
+  HIP_OK(hipStreamCreateWithFlags(&consStream, hipStreamNonBlocking));
+  HIP_OK(hipStreamCreateWithFlags(&prodStream, hipStreamNonBlocking));
+  dim3 threads(BLOCK, BLOCK, 1), grid(n / BLOCK, n / BLOCK, 1);
+  MMSync sync;
+  MMProd prod(grid, threads, NoSync(), sync);
+  MMCons cons(grid, threads, sync, NoSync());
+  statusOut[0] = CuSync::setProducerConsumerPair(prod, cons);
+  hipLaunchKernelGGL(tiledSgemm<MMProd>, grid, threads, 0, prodStream, prod, C, A, B, n, n);
+  statusOut[1] = prod.invokeWaitKernel(consStream);
+  hipLaunchKernelGGL(tiledSgemm<MMCons>, grid, threads, 0, consStream, cons, E, (const float*)C, D, n, n);
+  HIP_OK(hipDeviceSynchronize());
+  prod.incrementIter(); cons.incrementIter();
+  cusync_stage_desc pd = prod.desc(), cd = cons.desc();
+  uint32_t timeouts = 0;
+  if (cusync_stage_read_state(&pd, semsOut, nullptr, nullptr, nullptr, nullptr, nullptr) != CUSYNC_SUCCESS) return -1;
+  if (cusync_stage_read_state(&cd, nullptr, nullptr, nullptr, nullptr, nullptr, &timeouts) != CUSYNC_SUCCESS) return -1;
+  statusOut[2] = (int)timeouts;
+  prod.destroy(); cons.destroy();
+  HIP_OK(hipStreamDestroy(prodStream)); HIP_OK(hipStreamDestroy(consStream));
+  return 0;
+}
+
+// Host-only checks of the error paths (no kernel is launched).
+// out[0] pair(consumer-as-producer)  out[1] pair(producer-as-consumer)
+// out[2] invokeWaitKernel on a non-producer  out[3] status() of a valid stage
+// out[4] pair with a default-constructed producer
+int run_error_paths(int* out) {
+  using Sync = TileSync<IdentityOrder, 1, 1>;
+  using P = CuStage<IdentityOrder, NoSync, Sync>;
+  using Cn = CuStage<IdentityOrder, Sync, NoSync>;
+  dim3 grid(4, 1, 1), threads(64, 1, 1);
+  Sync sync;
+  P prod(grid, threads, NoSync(), sync);
+  Cn cons(grid, threads, sync, NoSync());
+  out[0] = CuSync::setProducerConsumerPair(cons, cons);
+  out[1] = CuSync::setProducerConsumerPair(prod, prod);
+  out[2] = cons.invokeWaitKernel(nullptr);
+  out[3] = prod.status();
+  P empty;
+  out[4] = CuSync::setProducerConsumerPair(empty, cons);
+  prod.destroy(); cons.destroy();
+  return 0;
+}
+
+}  // extern "C"

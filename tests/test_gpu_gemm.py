@@ -1,0 +1,180 @@
+"""GPU parity of the sync-aware fp16 GEMM (C ABI: cusync_gemm_run) against the
+CPU oracle, including the chained two-GEMM configuration (M=256, N=K=1024,
+TileSync, producer and consumer on two streams)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from cusync_amd import _lib, api
+from util import assert_close, empty_dev, normal_f16, to_dev, to_host, uniform_f16
+
+pytestmark = pytest.mark.gpu
+
+ALL_TILES = list(range(api.TILE.COUNT))
+
+
+def plain_stage(tile, M, N):
+    return api.Stage(api.gemm_grid(tile, M, N), (1, 1, 1), api.no_sync(), api.no_sync())
+
+
+def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups=0):
+    import torch
+    L = _lib.load()
+    M = a.shape[0]
+    K = K if K is not None else a.shape[1]
+    N = b.shape[1]
+    da, db = to_dev(a), to_dev(b)
+    dd = empty_dev((M, N), fill=float("nan"))
+    torch.cuda.synchronize()
+    st = plain_stage(tile, M, N)
+    rc = api.gemm(st, M, N, K, da.data_ptr(), a.shape[1], db.data_ptr(), N, dd.data_ptr(), N, tile,
+                  epilogue=epilogue, a_mode=a_mode, max_workgroups=max_workgroups)
+    assert rc == api.ERR.SUCCESS, api.last_error()
+    assert L.cusync_rt_device_sync() == 0, api.last_error()
+    state = st.read_state()
+    assert state.tile_counter == 0       # dispenser re-armed
+    st.destroy()
+    return to_host(dd)
+
+
+@pytest.mark.parametrize("tile", ALL_TILES)
+def test_gemm_exact_on_integer_data(tile):
+    # small integers: every product and partial sum is exact in fp32 and fits fp16,
+    # so the result must be bit-identical and any indexing slip shows up exactly
+    print("tile", tile, flush=True)
+    rng = np.random.default_rng(tile)
+    M, N, K = 300, 328, 192
+    a = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    b = rng.integers(-2, 3, (K, N)).astype(np.float16)
+    got = run_gemm(a, b, tile)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, orc.gemm(a, b))
+
+
+@pytest.mark.parametrize("tile", ALL_TILES)
+@pytest.mark.parametrize("shape", [(256, 1024, 1024), (1, 256, 512), (17, 136, 64), (513, 264, 1000)])
+def test_gemm_matches_oracle(tile, shape):
+    print("tile", tile, "shape", shape, flush=True)
+    M, N, K = shape
+    a = uniform_f16((M, K), 1)
+    b = normal_f16((K, N), 2, std=0.05)
+    got = run_gemm(a, b, tile)
+    assert_close(got, orc.gemm(a, b), "gemm tile %d %s" % (tile, shape))
+
+
+@pytest.mark.parametrize("epilogue,orc_epi", [(api.EPI.GELU, orc.EPI_GELU), (api.EPI.RELU, orc.EPI_RELU)])
+def test_gemm_epilogues(epilogue, orc_epi):
+    a = uniform_f16((130, 512), 3)
+    b = normal_f16((512, 256), 4, std=0.1)
+    got = run_gemm(a, b, api.TILE.T128x128x64, epilogue=epilogue)
+    assert_close(got, orc.gemm(a, b, orc_epi), "epilogue %d" % epilogue)
+
+
+@pytest.mark.parametrize("tile", [api.TILE.T128x128x64, api.TILE.T256x128x64, api.TILE.T32x128x64])
+def test_gemm_swiglu_a_operand(tile):
+    # A[m,k] = silu(G[m,k]) * G[m,k+d];  d = 344*8 = 2752 is not a multiple of 128
+    d, M, N = 2752, 70, 256
+    gu = uniform_f16((M, 2 * d), 5) * np.float16(3)
+    w = normal_f16((d, N), 6, std=0.05)
+    got = run_gemm(gu, w, tile, a_mode=1, K=d)
+    want = orc.gemm(orc.swiglu(gu, d), w)
+    assert_close(got, want, "swiglu tile %d" % tile)
+
+
+def test_gemm_persistent_launch_smaller_than_grid():
+    # 4 x 11 = 44 tiles on 5 workgroups: every workgroup loops over several tickets
+    a = uniform_f16((512, 256), 7)
+    b = normal_f16((256, 1400), 8, std=0.05)
+    got = run_gemm(a, b, api.TILE.T128x128x64, max_workgroups=5)
+    assert_close(got, orc.gemm(a, b), "persistent")
+
+
+def test_gemm_can_implement_rejects():
+    L = _lib.load()
+    st = plain_stage(api.TILE.T128x128x64, 64, 64)
+    bad = api.gemm_args(st, 64, 64, 60, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # K % 8 != 0
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "multiples of 8" in api.last_error()
+    bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=2)
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED
+    bad = api.gemm_args(st, 300, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # grid mismatch
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "grid" in api.last_error()
+    st.destroy()
+    # NoAtomicAdd with a counting policy is refused (RowSync counts to gN)
+    g = api.gemm_grid(api.TILE.T128x128x64, 256, 512)
+    rs = api.row_sync(128, g[0])
+    prod = api.Stage(g, (1, 1, 1), api.no_sync(), rs, opts=api.OPT.NO_ATOMIC_ADD)
+    bad = api.gemm_args(prod, 256, 512, 64, 16, 64, 16, 512, 16, 512, api.TILE.T128x128x64)
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "NoAtomicAdd" in api.last_error()
+    prod.destroy()
+
+
+def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10):
+    """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`."""
+    import torch
+    L = _lib.load()
+    a = uniform_f16((M, K), seed)
+    b = uniform_f16((K, N), seed + 1) * np.float16(0.05)
+    d = uniform_f16((N, N), seed + 2) * np.float16(0.05)
+    da, db, dd = to_dev(a), to_dev(b), to_dev(d)
+    dc = empty_dev((M, N), fill=float("nan"))
+    de = empty_dev((M, N), fill=float("nan"))
+    torch.cuda.synchronize()
+    tm, tn, _ = api.tile_shape(tile1)
+    g1, g2 = api.gemm_grid(tile1, M, N), api.gemm_grid(tile2, M, N)
+    if policy_kind == "tile":
+        pol = api.tile_sync(api.ORDER.TRANSPOSE_XY, tm, tn)
+        opol = orc.policy(orc.TILESYNC, orc.ORDER_TRANSPOSE_XY, tm, tn)
+    else:
+        pol = api.row_sync(tm, g1[0])
+        opol = orc.policy(orc.ROWSYNC, tileM=tm, waitValue=g1[0])
+    prod = api.Stage(g1, (1, 1, 1), api.no_sync(), pol, opts=opts)
+    cons = api.Stage(g2, (1, 1, 1), pol, api.no_sync(), opts=opts)
+    assert api.set_producer_consumer_pair(prod, cons) == api.ERR.SUCCESS
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    assert L.cusync_rt_stream_create(C.byref(s1)) == 0 and L.cusync_rt_stream_create(C.byref(s2)) == 0
+    for _ in range(iters):
+        dc.fill_(float("nan")); de.fill_(float("nan"))
+        torch.cuda.synchronize()
+        assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1,
+                        stream=s1, max_workgroups=max_wg) == api.ERR.SUCCESS, api.last_error()
+        assert prod.invokeWaitKernel(s2) == api.ERR.SUCCESS
+        assert api.gemm(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2,
+                        stream=s2, max_workgroups=max_wg) == api.ERR.SUCCESS, api.last_error()
+        assert L.cusync_rt_device_sync() == 0, api.last_error()
+        prod.incrementIter(); cons.incrementIter()
+    ps, cs = prod.read_state(), cons.read_state()
+    want_sems = orc.expected_sems_gemm(opol, g1, tm, tn, iters, opts)
+    L.cusync_rt_stream_destroy(s1); L.cusync_rt_stream_destroy(s2)
+    prod.destroy(); cons.destroy()
+    return a, b, d, to_host(dc), to_host(de), ps, cs, want_sems
+
+
+@pytest.mark.parametrize("policy_kind,opts", [("tile", 0), ("tile", api.OPT.NO_ATOMIC_ADD | api.OPT.REORDER_TILE_LOADS), ("row", 0)])
+@pytest.mark.parametrize("tiles", [(api.TILE.T128x128x64, api.TILE.T128x128x64), (api.TILE.T32x128x64, api.TILE.T64x128x64),
+                                   (api.TILE.T256x128x64, api.TILE.T128x128x64)])
+def test_two_chained_gemms_config1(policy_kind, opts, tiles):
+    # BASELINE config 1: M=256, N=K=1024, fp32 accumulate, inputs uniform from a seed
+    print("chained", policy_kind, opts, tiles, flush=True)
+    M, N, K = 256, 1024, 1024
+    iters = 2
+    a, b, d, c, e, ps, cs, want_sems = chained(M, N, K, tiles[0], tiles[1], policy_kind, iters=iters, opts=opts)
+    c_ref = orc.gemm(a, b)
+    assert_close(c, c_ref, "C")
+    # E's reference multiplies the C the GPU produced (fp16), isolating the second GEMM
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0
+    assert np.array_equal(ps.sems, want_sems)                 # bit-exact semaphore end state
+    assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
+    assert ps.kernel_executed == iters
+
+
+def test_chained_gemms_with_few_workgroups():
+    # both launches hold fewer workgroups than tiles: tickets keep producer rows ahead of consumers
+    a, b, d, c, e, ps, cs, want_sems = chained(512, 1024, 512, api.TILE.T128x128x64, api.TILE.T128x128x64,
+                                               "tile", iters=3, max_wg=6)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3

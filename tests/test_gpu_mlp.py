@@ -1,0 +1,137 @@
+"""GPU parity of the MLP chains (C ABI: cusync_mlp_*) against the CPU oracle:
+GPT-3 175B 1/8 shard (X[B,12288] W1[12288,6144] GeLU W2[6144,12288]) and the
+LLaMA 65B SwiGLU shard (d = 2752 and the reference's d = 2816), stream-ordered
+and under RowSync / TileSync / StridedSync.  The oracle is evaluated on sampled
+rows (each output row depends on one input row only); across sync modes the
+outputs must be bit-identical because synchronisation only changes timing."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from cusync_amd import api
+from util import assert_close, empty_dev, normal_f16, sample_rows, to_dev, to_host, uniform_f16
+
+pytestmark = pytest.mark.gpu
+
+GPT3 = dict(hidden=12288, inner=6144)
+_weights = {}
+
+
+def weights(model, hidden, inner):
+    key = (model, hidden, inner)
+    if key not in _weights:
+        n1 = inner if model == api.MODEL.GPT3 else 2 * inner
+        w1 = normal_f16((hidden, n1), 2)       # seeds: X 1, W1 2, W2 3
+        w2 = normal_f16((inner, hidden), 3)
+        _weights[key] = (w1, w2, to_dev(w1), to_dev(w2))
+    return _weights[key]
+
+
+def run_mlp(model, batch, hidden, inner, sync, runs=2, activation=1, **kw):
+    import torch
+    w1, w2, dw1, dw2 = weights(model, hidden, inner)
+    x = uniform_f16((batch, hidden), 1)
+    dx = to_dev(x)
+    dh = empty_dev((batch, w1.shape[1]), fill=float("nan"))
+    dy = empty_dev((batch, hidden), fill=float("nan"))
+    torch.cuda.synchronize()
+    mlp = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr(), activation=activation, **kw)
+    times = mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=runs)
+    prod, cons = mlp.stage_state(0), mlp.stage_state(1)
+    tiles = mlp.tiles()
+    mlp.destroy()
+    return x, w1, w2, to_host(dh), to_host(dy), prod, cons, tiles, times
+
+
+def check_against_oracle(model, x, w1, w2, h, y, inner, activation=1):
+    rows = sample_rows(x.shape[0])
+    xs = np.ascontiguousarray(x[rows])
+    if model == api.MODEL.GPT3:
+        h_ref = orc.gemm(xs, w1, orc.EPI_GELU if activation else orc.EPI_NONE)
+        assert_close(h[rows], h_ref, "H rows")
+        a2 = np.ascontiguousarray(h[rows])
+    else:
+        h_ref = orc.gemm(xs, w1)
+        assert_close(h[rows], h_ref, "gate|up rows")
+        a2 = orc.swiglu(np.ascontiguousarray(h[rows]), inner) if activation else np.ascontiguousarray(h[rows][:, :inner])
+    # second GEMM is checked on the intermediate the GPU produced
+    assert_close(y[rows], orc.gemm(a2, w2), "Y rows")
+
+
+def expected_sems(prod, tiles, iters):
+    d = prod.desc
+    p = orc.Policy(d.out.kind, d.out.order, d.out.tileM, d.out.tileN, d.out.waitValue, d.out.postValue,
+                   d.out.gridN, d.out.stride, d.out.R, d.out.S, d.out.H)
+    tm, tn, _ = api.tile_shape(tiles[0])
+    return orc.expected_sems_gemm(p, prod.grid, tm, tn, iters, d.opts)
+
+
+@pytest.mark.parametrize("batch", [1, 16, 64, 256, 512])
+def test_gpt3_mlp_all_sync_modes(batch):
+    print("gpt3 batch", batch, flush=True)
+    outs = {}
+    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE):
+        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.GPT3, batch, sync=sync, runs=2, **GPT3)
+        outs[sync] = (h, y)
+        assert cons.spin_timeouts == 0
+        assert prod.tile_counter == 0 and cons.tile_counter == 0 and prod.start_counter == 0
+        if sync != api.SYNC.STREAM:
+            assert np.array_equal(prod.sems, expected_sems(prod, tiles, 2))
+            assert prod.kernel_executed == 2
+        rc, want_order = orc.build_schedule(orc.ORDER_TRANSPOSE_XY, prod.grid)
+        assert np.array_equal(prod.tile_order, want_order)
+    check_against_oracle(api.MODEL.GPT3, x, w1, w2, *outs[api.SYNC.STREAM], inner=6144)
+    for sync in (api.SYNC.ROW, api.SYNC.TILE):
+        assert np.array_equal(outs[sync][0].view(np.uint16), outs[api.SYNC.STREAM][0].view(np.uint16))
+        assert np.array_equal(outs[sync][1].view(np.uint16), outs[api.SYNC.STREAM][1].view(np.uint16))
+
+
+@pytest.mark.parametrize("batch", [1024, 2048])
+def test_gpt3_mlp_full_size(batch):
+    print("gpt3 full batch", batch, flush=True)
+    x, w1, w2, h0, y0, _, _, _, _ = run_mlp(api.MODEL.GPT3, batch, sync=api.SYNC.STREAM, runs=1, **GPT3)
+    check_against_oracle(api.MODEL.GPT3, x, w1, w2, h0, y0, inner=6144)
+    # size-independent property: rows are independent, so a permuted batch permutes the output
+    for sync in (api.SYNC.ROW, api.SYNC.TILE):
+        _, _, _, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.GPT3, batch, sync=sync, runs=3, **GPT3)
+        assert cons.spin_timeouts == 0
+        assert np.array_equal(h.view(np.uint16), h0.view(np.uint16))
+        assert np.array_equal(y.view(np.uint16), y0.view(np.uint16))
+        assert np.array_equal(prod.sems, expected_sems(prod, tiles, 3)) and prod.kernel_executed == 3
+
+
+def test_gpt3_without_activation_matches_reference_check_build():
+    # the reference's --check build has no GeLU (TB/mlp.cu:148-151)
+    x, w1, w2, h, y, _, _, _, _ = run_mlp(api.MODEL.GPT3, 64, sync=api.SYNC.TILE, activation=0, **GPT3)
+    check_against_oracle(api.MODEL.GPT3, x, w1, w2, h, y, inner=6144, activation=0)
+
+
+@pytest.mark.parametrize("inner", [2752, 2816])
+@pytest.mark.parametrize("batch", [1, 64, 256, 1024])
+def test_llama_mlp(inner, batch):
+    print("llama", inner, batch, flush=True)
+    outs = {}
+    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.STRIDED):
+        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2)
+        outs[sync] = (h, y)
+        assert cons.spin_timeouts == 0
+        if sync != api.SYNC.STREAM:
+            assert np.array_equal(prod.sems, expected_sems(prod, tiles, 2))
+    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, *outs[api.SYNC.STREAM], inner=inner)
+    for sync in (api.SYNC.ROW, api.SYNC.STRIDED):
+        assert np.array_equal(outs[sync][1].view(np.uint16), outs[api.SYNC.STREAM][1].view(np.uint16))
+
+
+def test_llama_reference_wiring_no_activation():
+    # the reference's timed path reads the gate half as is (TB/mlp.cu:785-792): TileSync suffices
+    x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, 128, 8192, 2816, api.SYNC.TILE, activation=0)
+    assert cons.spin_timeouts == 0
+    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, h, y, inner=2816, activation=0)
+
+
+def test_strided_sync_rejects_unaligned_split():
+    import torch
+    w = torch.zeros(16, device="cuda", dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="inner % tileN"):
+        api.Mlp(api.MODEL.LLAMA, 256, 8192, 2752, api.SYNC.STRIDED, w.data_ptr(), w.data_ptr(),
+                tile1=api.TILE.T256x128x64)
