@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Benchmark of the CuSync hot path on one MI355X.
+
+Workload: the GPT-3 175B MLP, one GPU's 1/8 shard — X[B,12288] fp16 x
+W1[12288,6144] with GeLU fused -> H[B,6144] x W2[6144,12288] — as two dependent
+GEMMs, stream-ordered (kernel-boundary sync) versus CuSync RowSync / TileSync on
+two streams.  A "step" is one pass of the chain at B = 2048 under the better
+CuSync policy; inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is the step latency in microseconds (lower is
+better); `per_batch` holds the metric proper: latency per B in {1..2048} for the
+three modes, % gain over stream-ordered, TFLOP/s and roofline fraction, measured
+with the reference's protocol (10 warm-up runs, 20 timed, slowest 10 % dropped;
+src/ml-bench/transformer/mlp.cu:954-955, eval_mlp.py:40-50).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HIDDEN, INNER = 12288, 6144
+BATCHES = [1, 16, 64, 256, 512, 1024, 2048]
+PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+
+def trimmed(times):
+    """Mean and stdev after dropping the slowest 10 % (eval_mlp.py:40-50)."""
+    t = sorted(times)
+    keep = t[:max(1, len(t) - len(t) // 10)]
+    return statistics.fmean(keep), (statistics.pstdev(keep) if len(keep) > 1 else 0.0)
+
+
+def mlp_flops(b):
+    return 4.0 * b * HIDDEN * INNER
+
+
+def mlp_bytes(b):
+    # each operand/result once in fp16; the intermediate is written once and read once
+    return 2.0 * (2 * HIDDEN * INNER + b * HIDDEN * 2 + 2 * b * INNER)
+
+
+def ideal_us(b):
+    return max(mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12), mlp_bytes(b) / (PEAK_HBM_GBS * 1e9)) * 1e6
+
+
+def cpu_baseline(x_host, w1_host, w2_host, budget_s=15.0):
+    """Times the CPU oracle (the restatement of the reference's host GEMM,
+    src/ml-bench/transformer/common.h:89-102) on a bounded number of rows of the
+    same workload and scales to the B = 2048 shard."""
+    import numpy as np
+    import oracle as orc
+    t0 = time.perf_counter()
+    h = orc.gemm(x_host[:1], w1_host, orc.EPI_GELU)
+    orc.gemm(h, w2_host)
+    t1 = time.perf_counter() - t0
+    rows = int(max(1, min(64, budget_s / max(t1, 1e-3))))
+    t0 = time.perf_counter()
+    h = orc.gemm(np.ascontiguousarray(x_host[:rows]), w1_host, orc.EPI_GELU)
+    orc.gemm(h, w2_host)
+    t = time.perf_counter() - t0
+    per_row_us = t / rows * 1e6
+    return {
+        "value": per_row_us * 2048, "unit": "us", "cores": orc.num_threads(), "kind": "port",
+        "sample": "%d of 2048 rows of the same MLP (%.1f s of CPU time), scaled linearly; %.2f GFLOP/s" % (
+            rows, t, mlp_flops(rows) / t / 1e9),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=2048, help="B of the timed step")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-batch table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--tile1", type=int, default=-1)
+    ap.add_argument("--tile2", type=int, default=-1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (CuSync is a single-GPU mechanism); "
+                 "run with --gpus 1")
+
+    import numpy as np
+    import torch
+    from cusync_amd import api
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = api.device_info()
+
+    # Synthetic shard: X ~ U[-1,1], W ~ N(0, 0.02), seeds X 1 / W1 2 / W2 3, rounded to fp16.
+    def normal(shape, seed):
+        return (np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * 0.02).astype(np.float16)
+
+    w1_host, w2_host = normal((HIDDEN, INNER), 2), normal((INNER, HIDDEN), 3)
+    x_host = np.random.default_rng(1).uniform(-1, 1, (max(BATCHES), HIDDEN)).astype(np.float32).astype(np.float16)
+    w1, w2, x_all = (torch.from_numpy(a).cuda() for a in (w1_host, w2_host, x_host))
+    torch.cuda.synchronize()
+
+    def make(batch, sync):
+        h = torch.empty((batch, INNER), dtype=torch.float16, device="cuda")
+        y = torch.empty((batch, HIDDEN), dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()
+        m = api.Mlp(api.MODEL.GPT3, batch, HIDDEN, INNER, sync, w1.data_ptr(), w2.data_ptr(),
+                    tile1=args.tile1, tile2=args.tile2)
+        return m, h, y
+
+    def protocol(batch, sync, warm=10, timed=20, split=False):
+        m, h, y = make(batch, sync)
+        x = x_all[:batch]
+        m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=warm)
+        out = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=timed, split=split)
+        timeouts = m.stage_state(1).spin_timeouts
+        tiles = m.tiles()
+        m.destroy()
+        if timeouts:
+            sys.exit("bench.py: %d consumer waits timed out — results invalid" % timeouts)
+        return out, tiles
+
+    per_batch = []
+    if not args.no_sweep:
+        for b in BATCHES:
+            (t_s, g1, g2), tiles = protocol(b, api.SYNC.STREAM, split=True)
+            t_r, _ = protocol(b, api.SYNC.ROW)
+            t_t, _ = protocol(b, api.SYNC.TILE)
+            s, s_sd = trimmed(t_s)
+            r, r_sd = trimmed(t_r)
+            t, t_sd = trimmed(t_t)
+            best = min(r, t)
+            per_batch.append({
+                "B": b, "tiles": list(tiles),
+                "stream_us": round(s, 2), "stream_std": round(s_sd, 2),
+                "gemm1_us": round(trimmed(g1)[0], 2), "gemm2_us": round(trimmed(g2)[0], 2),
+                "rowsync_us": round(r, 2), "rowsync_std": round(r_sd, 2), "rowsync_gain_pct": round(100 - r / s * 100, 2),
+                "tilesync_us": round(t, 2), "tilesync_std": round(t_sd, 2), "tilesync_gain_pct": round(100 - t / s * 100, 2),
+                "best_tflops": round(mlp_flops(b) / best / 1e6, 1),
+                "bound": "mfma" if mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12) > mlp_bytes(b) / (PEAK_HBM_GBS * 1e9) else "hbm",
+                "roofline_frac": round(ideal_us(b) / best, 4),
+            })
+
+    # ---- the timed step: B = args.batch under the better CuSync policy ----------
+    B = args.batch
+    cand = {}
+    for name, sync in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):
+        ts, _ = protocol(B, sync, warm=5, timed=10)
+        cand[name] = (trimmed(ts)[0], sync)
+    policy = min(cand, key=lambda k: cand[k][0])
+    m, h, y = make(B, cand[policy][1])
+    x = x_all[:B]
+    m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step_times = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=args.steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    if m.stage_state(1).spin_timeouts:
+        sys.exit("bench.py: consumer waits timed out — results invalid")
+    tiles = m.tiles()
+    m.destroy()
+    ms_per_step = wall / args.steps * 1e3
+
+    # stream-ordered on the same shape: baseline latency and the kernels' own durations,
+    # taken with HIP events on the stream the kernels run on
+    (t_s, g1, g2), _ = protocol(B, api.SYNC.STREAM, warm=args.warmup, timed=max(10, args.steps), split=True)
+    stream_us = trimmed(t_s)[0]
+    k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
+    flops_per_launch = 2.0 * B * HIDDEN * INNER
+    achieved = flops_per_launch / (k_us * 1e-6) / 1e12
+    tm, tn, tk = api.tile_shape(tiles[0])
+
+    out = {
+        "metric": "GPT-3 MLP shard latency (us) + % gain vs kernel-boundary sync, B=1..2048",
+        "value": round(statistics.fmean(step_times), 2),
+        "unit": "us",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "GPT-3 175B MLP 1/8 shard, B=%d: X[B,12288] x W1[12288,6144] +GeLU -> x W2[6144,12288]" % B,
+                   "policy": policy, "tiles": list(tiles), "device": dev["arch"], "cus": dev["cus"]},
+        "stream_ordered_us": round(stream_us, 2),
+        "gain_pct": round(100 - statistics.fmean(step_times) / stream_us * 100, 2),
+        "tflops": round(mlp_flops(B) / statistics.fmean(step_times) / 1e6, 1),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                     "kernel": "gemmKernel %dx%dx%d (mean of GEMM1 %.1f us and GEMM2 %.1f us, stream-ordered, %.1f GFLOP per launch)" % (
+                         tm, tn, tk, statistics.fmean(g1), statistics.fmean(g2), flops_per_launch / 1e9)},
+        "per_batch": per_batch,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(x_host, w1_host, w2_host)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -23,6 +23,13 @@ namespace cusync {
 
 struct DynStage {
   cusync_stage_desc d;
+  // True when every producer tile starts and ends on a 128-byte line of the
+  // buffer the consumer reads (set by the launcher).  Then a line of that buffer
+  // can only enter this XCD's caches after the semaphore guarding it was seen,
+  // because the kernel began with clean caches and never touches a tile before
+  // its wait; the wait can skip the cache invalidation that would also throw
+  // away the weights the XCD's workgroups share.
+  bool lineAligned;
 
   __device__ __forceinline__ bool isProducer() const { return d.out.kind != CUSYNC_POLICY_NOSYNC; }
   __device__ __forceinline__ bool isConsumer() const { return d.in.kind != CUSYNC_POLICY_NOSYNC; }
@@ -68,16 +75,24 @@ struct DynStage {
     return isConsumer() && dyn::isSync(d.in, tile);
   }
 
+  // Per-run count a semaphore of the input policy must reach.
+  __device__ __forceinline__ uint32_t waitTarget() const { return (uint32_t)d.iter * dyn::waitValue(d.in); }
+
+  // Current value of the semaphore guarding `tile`, without waiting and without
+  // ordering: the caller compares it with waitTarget() later, after other work.
+  __device__ __forceinline__ uint32_t peek(const cusync_dim3& tile) const {
+    return dev::pollOnce(&d.tileStatusRead[dyn::tileIndex(d.in, tile, d.prodGrid)]);
+  }
+
   // Wave-uniform wait: every lane of the calling wave passes the same tile.
   // No barrier; each wave that is going to read the tile calls this itself.
   __device__ __forceinline__ void waitWave(const cusync_dim3& tile) const {
     if (!needsWait(tile)) return;
     const uint32_t idx = dyn::tileIndex(d.in, tile, d.prodGrid);
-    const uint32_t need = (uint32_t)d.iter * dyn::waitValue(d.in);
-    if (!dev::spinUntilAtLeast(&d.tileStatusRead[idx], need)) {
-      if (__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0)
-        dev::ticketAdd(d.spinTimeouts, 1);
-    }
+    const bool ok = lineAligned ? dev::spinUntilAtLeastNoInvalidate(&d.tileStatusRead[idx], waitTarget())
+                                : dev::spinUntilAtLeast(&d.tileStatusRead[idx], waitTarget());
+    if (!ok && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0)
+      dev::ticketAdd(d.spinTimeouts, 1);
   }
 
   // Workgroup-wide post; contains a barrier, call from all threads.

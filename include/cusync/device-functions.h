@@ -34,25 +34,54 @@ CUSYNC_DEVICE void acquireFence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "ag
 // Upper bound on polls of one wait.  A wait that is never satisfied (a lost
 // post, a stage wired to the wrong producer) must not hold the GPU forever:
 // after this many polls the wait gives up and reports failure.  One poll is a
-// trip to the coherent level of the memory system plus a short sleep, i.e. of
-// the order of a microsecond, so the default allows a few seconds.
+// trip to the coherent level of the memory system plus a sleep that grows to
+// about two microseconds, so the default allows a second or two.
 #ifndef CUSYNC_SPIN_LIMIT
-#define CUSYNC_SPIN_LIMIT (1u << 22)
+#define CUSYNC_SPIN_LIMIT (1u << 20)
 #endif
 
-// Spin until *addr >= want; returns false if the poll budget ran out first.
-// Meant to be executed by every lane of a wave with the same arguments (the
-// loads coalesce into one request, the branch is uniform), or by a single lane.
-// s_sleep yields issue slots to the waves that do the producer's work on the
-// same CU.
-CUSYNC_DEVICE bool spinUntilAtLeast(const volatile uint32_t* addr, uint32_t want) {
-  uint32_t polls = 0;
-  bool ok = true;
-  while (loadRelaxed(addr) < want) {
-    if (++polls >= CUSYNC_SPIN_LIMIT) { ok = false; break; }
-    __builtin_amdgcn_s_sleep(2);
+// One poll of a semaphore by a whole wave: only the first active lane touches
+// memory, the value is broadcast to the others.  (Sixty-four lanes loading the
+// same coherent address are sixty-four requests to one memory channel.)
+CUSYNC_DEVICE uint32_t pollOnce(const volatile uint32_t* addr) {
+  uint32_t v = 0;
+  const uint64_t exec = __builtin_amdgcn_read_exec();
+  const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(exec >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)exec, 0u));
+  if (before == 0) v = loadRelaxed(addr);
+  return __builtin_amdgcn_readfirstlane(v);
+}
+
+// Polls *addr until it is >= want; returns false if the poll budget ran out.
+// Sleeps between polls and doubles the sleep up to a few microseconds: a
+// semaphore is one address, and hundreds of waves polling it back to back would
+// saturate the memory channel it lives on and slow the very producer they are
+// waiting for.
+CUSYNC_DEVICE bool pollUntilAtLeast(const volatile uint32_t* addr, uint32_t want) {
+  uint32_t polls = 0, naps = 1;
+  while (pollOnce(addr) < want) {
+    if (++polls >= CUSYNC_SPIN_LIMIT) return false;
+    for (uint32_t i = 0; i < naps; i++) __builtin_amdgcn_s_sleep(16);   // 16 * 64 clocks
+    if (naps < 8) naps <<= 1;
   }
+  return true;
+}
+
+// Spin until *addr >= want, then acquire at agent scope.  Meant to be executed
+// by every lane of a wave with the same arguments (the loads coalesce into one
+// request, the branch is uniform), or by a single lane.
+CUSYNC_DEVICE bool spinUntilAtLeast(const volatile uint32_t* addr, uint32_t want) {
+  const bool ok = pollUntilAtLeast(addr, want);
   acquireFence();
+  return ok;
+}
+
+// Same without the cache invalidation of the acquire.  Only valid when no line
+// of the guarded data can already sit in this XCD's caches (see DynStage).
+// Program order is still kept: the loads that follow are issued after the poll
+// returned.
+CUSYNC_DEVICE bool spinUntilAtLeastNoInvalidate(const volatile uint32_t* addr, uint32_t want) {
+  const bool ok = pollUntilAtLeast(addr, want);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   return ok;
 }
 
