@@ -28,6 +28,9 @@ HIDDEN, INNER = 12288, 6144
 BATCHES = [1, 16, 64, 256, 512, 1024, 2048]
 PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes one GEMM launch of the B = 2048 step moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by
+# a plain copy of known size (profiles/gemm_dma_128x256x32_gpt3_mlp_b2048.md).
+TRAFFIC_BYTES_PER_LAUNCH = 845e6
 
 
 def trimmed(times):
@@ -60,7 +63,7 @@ def cpu_baseline(x_host, w1_host, w2_host, budget_s=15.0):
     h = orc.gemm(x_host[:1], w1_host, orc.EPI_GELU)
     orc.gemm(h, w2_host)
     t1 = time.perf_counter() - t0
-    rows = int(max(1, min(64, budget_s / max(t1, 1e-3))))
+    rows = int(max(1, min(512, budget_s / max(t1, 1e-3))))
     t0 = time.perf_counter()
     h = orc.gemm(np.ascontiguousarray(x_host[:rows]), w1_host, orc.EPI_GELU)
     orc.gemm(h, w2_host)
@@ -81,6 +84,9 @@ def main():
     ap.add_argument("--batch", type=int, default=2048, help="B of the timed step")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-batch table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the leg that times the dominant kernel (stream-ordered GEMM1/GEMM2 at --batch) "
+                         "plus a plain copy of known size; used under rocprofv3 so its per-kernel averages match")
     ap.add_argument("--tile1", type=int, default=-1)
     ap.add_argument("--tile2", type=int, default=-1)
     args = ap.parse_args()
@@ -125,6 +131,32 @@ def main():
             sys.exit("bench.py: %d consumer waits timed out — results invalid" % timeouts)
         return out, tiles
 
+    def roofline_leg(B, warm, timed):
+        """Durations of the two GEMM launches, HIP events on the stream they run on."""
+        (t_s, g1, g2), tiles = protocol(B, api.SYNC.STREAM, warm=warm, timed=timed, split=True)
+        k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
+        flops_per_launch = 2.0 * B * HIDDEN * INNER
+        achieved = flops_per_launch / (k_us * 1e-6) / 1e12
+        tm, tn, tk = api.tile_shape(tiles[0])
+        # plain copy of known size: the scale for the FETCH_SIZE / WRITE_SIZE counters
+        a = torch.zeros(64 << 20, dtype=torch.float16, device="cuda")      # 128 MiB read + 128 MiB written
+        b = torch.empty_like(a)
+        for _ in range(3):
+            torch.add(a, 1, out=b)
+        torch.cuda.synchronize()
+        return {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                "kernel": "gemmDmaKernel/gemmKernel tile %dx%dx%d (mean of GEMM1 %.1f us and GEMM2 %.1f us, stream-ordered, "
+                          "%.1f GFLOP per launch)" % (tm, tn, tk, statistics.fmean(g1), statistics.fmean(g2), flops_per_launch / 1e9),
+                }, trimmed(t_s)[0], tiles
+
+    B = args.batch
+    if args.roofline_only:
+        roof, stream_us, tiles = roofline_leg(B, args.warmup, max(10, args.steps))
+        print(json.dumps({"metric": "dominant kernel only", "roofline": roof, "stream_ordered_us": round(stream_us, 2),
+                          "tiles": list(tiles)}))
+        return
+
     per_batch = []
     if not args.no_sweep:
         for b in BATCHES:
@@ -147,7 +179,6 @@ def main():
             })
 
     # ---- the timed step: B = args.batch under the better CuSync policy ----------
-    B = args.batch
     cand = {}
     for name, sync in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):
         ts, _ = protocol(B, sync, warm=5, timed=10)
@@ -167,14 +198,9 @@ def main():
     m.destroy()
     ms_per_step = wall / args.steps * 1e3
 
-    # stream-ordered on the same shape: baseline latency and the kernels' own durations,
-    # taken with HIP events on the stream the kernels run on
-    (t_s, g1, g2), _ = protocol(B, api.SYNC.STREAM, warm=args.warmup, timed=max(10, args.steps), split=True)
-    stream_us = trimmed(t_s)[0]
-    k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
-    flops_per_launch = 2.0 * B * HIDDEN * INNER
-    achieved = flops_per_launch / (k_us * 1e-6) / 1e12
-    tm, tn, tk = api.tile_shape(tiles[0])
+    # stream-ordered on the same shape: baseline latency and the kernels' own durations
+    roof, stream_us, _ = roofline_leg(B, args.warmup, max(10, args.steps))
+    roof["traffic"] = TRAFFIC_BYTES_PER_LAUNCH
 
     out = {
         "metric": "GPT-3 MLP shard latency (us) + % gain vs kernel-boundary sync, B=1..2048",
@@ -189,10 +215,7 @@ def main():
         "stream_ordered_us": round(stream_us, 2),
         "gain_pct": round(100 - statistics.fmean(step_times) / stream_us * 100, 2),
         "tflops": round(mlp_flops(B) / statistics.fmean(step_times) / 1e6, 1),
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
-                     "kernel": "gemmKernel %dx%dx%d (mean of GEMM1 %.1f us and GEMM2 %.1f us, stream-ordered, %.1f GFLOP per launch)" % (
-                         tm, tn, tk, statistics.fmean(g1), statistics.fmean(g2), flops_per_launch / 1e9)},
+        "roofline": roof,
         "per_batch": per_batch,
     }
     if not args.no_cpu:

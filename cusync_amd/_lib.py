@@ -31,7 +31,7 @@ class PolicyDesc(C.Structure):
 class StageDesc(C.Structure):
     _fields_ = [("grid", Dim3), ("prodGrid", Dim3), ("tileSize", Dim3),
                 ("iter", i32), ("opts", i32), ("in_", PolicyDesc), ("out", PolicyDesc),
-                ("tileOrder", vp), ("tileCounter", vp), ("startCounter", vp),
+                ("tileOrder", vp), ("tileCounter", vp), ("startCounter", vp), ("xcdTickets", vp),
                 ("kernelExecuted", vp), ("spinTimeouts", vp),
                 ("tileStatusWrite", vp), ("tileStatusRead", vp)]
 

@@ -1,0 +1,123 @@
+// Pieces shared by the fp16 GEMM kernels: parameter block, buffer-descriptor
+// loads, epilogue math and the instruction-order directives.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <utility>
+
+#include "../../include/cusync_amd.h"
+#include "stage_device.h"
+
+namespace cusync {
+namespace gemm {
+
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr uint32_t kOutOfRange = 0x80000000u;   // buffer offset beyond any descriptor we build
+
+struct GemmParams {
+  cusync::DynStage stage;
+  uint32_t M, N, K;
+  const half_t* A; uint32_t lda;
+  const half_t* B; uint32_t ldb;
+  half_t* D; uint32_t ldd;
+  int32_t epilogue;
+  int32_t a_mode;
+  uint32_t launched;       // workgroups in this launch
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ uint4v loadChunk(__amdgpu_buffer_rsrc_t r, uint32_t byteOffset) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byteOffset, 0, 0);
+}
+
+// erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7), enough for an fp16 result
+// and a third of the instructions of the library erff.
+__device__ __forceinline__ float fastErf(float x) {
+  const float ax = __builtin_fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * ax);
+  float poly = 1.061405429f;
+  poly = poly * t - 1.453152027f;
+  poly = poly * t + 1.421413741f;
+  poly = poly * t - 0.284496736f;
+  poly = poly * t + 0.254829592f;
+  poly *= t;
+  const float e = __expf(-ax * ax);
+  const float r = 1.0f - poly * e;
+  return __builtin_copysignf(r, x);
+}
+
+__device__ __forceinline__ float applyEpilogue(float v, int epilogue) {
+  if (epilogue == CUSYNC_EPILOGUE_GELU) return 0.5f * v * (1.0f + fastErf(v * 0.70710678118654752f));
+  if (epilogue == CUSYNC_EPILOGUE_RELU) return v > 0.0f ? v : 0.0f;
+  return v;
+}
+
+__device__ __forceinline__ float siluf(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
+// A[m,k] = silu(gate) * up, element-wise on one 16-byte chunk.
+__device__ __forceinline__ uint4v swigluChunk(uint4v gate, uint4v up) {
+  half8 g = __builtin_bit_cast(half8, gate);
+  half8 u = __builtin_bit_cast(half8, up);
+  half8 r;
+#pragma unroll
+  for (int i = 0; i < 8; i++) r[i] = (half_t)(siluf((float)g[i]) * (float)u[i]);
+  return __builtin_bit_cast(uint4v, r);
+}
+
+// Instruction-order directives for the scheduler (groups of one kind of
+// instruction, placed in the order the directives appear).  Without them the
+// compiler serialises "LDS read, wait, two MFMAs", which leaves the matrix
+// pipe idle for the whole LDS latency when only one wavefront runs per SIMD.
+constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
+
+template<int MASK, int SIZE>
+__device__ __forceinline__ void schedGroup() {
+  if constexpr (SIZE > 0) __builtin_amdgcn_sched_group_barrier(MASK, SIZE, 0);
+}
+
+// Share of `total` items that falls to slot `i` of `slots` when spread evenly.
+constexpr int evenShare(int total, int slots, int i) { return (total * (i + 1)) / slots - (total * i) / slots; }
+
+// Order of one pass over an LDS stage: STEPS k-steps of NM MFMAs each.  The R
+// LDS reads that fetch the fragments of k-step s+1 are spread between the
+// MFMAs of k-step s; the W LDS writes that stage the next K chunk are spread
+// over the MFMAs of the second half of the pass, as late as possible so that
+// the global loads feeding them have had time to land.
+template<int STEPS, int NM, int R, int W, int S = 0, int M = 0>
+__device__ __forceinline__ void schedPass() {
+  if constexpr (S == 0 && M == 0) schedGroup<kSchedDsRead, R>();        // fragments of k-step 0
+  if constexpr (S < STEPS) {
+    constexpr int FIRST_W = STEPS / 2;                                  // first k-step that carries writes
+    constexpr int W_SLOTS = (STEPS - FIRST_W) * NM;
+    schedGroup<kSchedMfma, 1>();
+    if constexpr (S + 1 < STEPS) schedGroup<kSchedDsRead, evenShare(R, NM, M)>();
+    if constexpr (S >= FIRST_W) schedGroup<kSchedDsWrite, evenShare(W, W_SLOTS, (S - FIRST_W) * NM + M)>();
+    if constexpr (M + 1 < NM) schedPass<STEPS, NM, R, W, S, M + 1>();
+    else schedPass<STEPS, NM, R, W, S + 1, 0>();
+  }
+}
+
+template<int P> struct Parity { static constexpr int value = P; };
+
+// Calls f(Parity<0>{}), f(Parity<1>{}), ... f(Parity<N-1>{}): a loop whose index
+// is a compile-time constant inside the body.
+template<int N, class F>
+__device__ __forceinline__ void staticFor(F&& f) {
+  [&]<int... I>(std::integer_sequence<int, I...>) { (f(Parity<I>{}), ...); }(std::make_integer_sequence<int, N>{});
+}
+
+}  // namespace gemm
+}  // namespace cusync

@@ -1,0 +1,319 @@
+// fp16 GEMM kernel whose A and B tiles go from global memory straight into LDS
+// (buffer_load ... lds, 16 bytes per lane) without passing through registers.
+//
+// Why: on gfx950 an LDS write issued by a wave (ds_write_b128) costs about 50
+// clocks of that wave's LDS issue time, and with the MFMA rate doubled over
+// CDNA3 the LDS is the scarce unit.  The direct loads take the write half of the
+// LDS traffic off the waves and free the registers a staged copy needs, which
+// is what makes a 256x256 tile (256 accumulator registers per lane) fit.
+//
+// Layout.  A direct load writes one contiguous 1 KiB run of LDS per wave
+// instruction, lane l at byte 16*l, so rows cannot be padded.  Bank conflicts
+// are avoided by permuting WHICH 16-byte chunk of global memory each lane
+// fetches instead (an XOR swizzle):
+//   A stage  [BM rows][BK halfs]:   chunk c of row r lives at slot c ^ swzA(r)
+//   B stage  [BK rows][BN halfs]:   chunk c of row k lives at slot c ^ 4*(k&1)
+// so that the eight lanes the LDS serves together (A fragments: eight rows;
+// B transpose reads: four k rows x 64 bytes) fall on distinct bank groups.
+//
+// Pipeline.  STAGES LDS stages; iteration kt waits for its own chunk
+// (s_waitcnt vmcnt), passes one barrier, issues the loads of chunk kt+STAGES-1
+// into the stage the previous iteration finished with, and runs the MFMAs of
+// chunk kt.  The loads are inline assembly on purpose: the compiler would
+// otherwise wait for every outstanding direct load before any LDS read, which
+// removes the overlap between prefetch and compute.
+#pragma once
+
+#include "gemm_common.h"
+
+namespace cusync {
+namespace gemm {
+
+template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1>
+struct DmaCfg {
+  static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // register budget: 512 / this per lane
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int KS = BK / 16;                        // MFMA k-steps per chunk
+  static constexpr int A_ROW_BYTES = BK * 2, B_ROW_BYTES = BN * 2;
+  static constexpr int A_CPR = A_ROW_BYTES / 16, B_CPR = B_ROW_BYTES / 16;   // 16-byte chunks per row
+  static constexpr int A_STAGE = BM * A_ROW_BYTES, B_STAGE = BK * B_ROW_BYTES;
+  static constexpr int A_LOADS = A_STAGE / 1024 / 4, B_LOADS = B_STAGE / 1024 / 4;   // per wave per chunk
+  static constexpr int LOADS = A_LOADS + B_LOADS;
+  static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES, B_ROWS_PER_LOAD = 1024 / B_ROW_BYTES;
+  static constexpr int LDS_BYTES = STAGES * (A_STAGE + B_STAGE);
+  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile is made of 32x32 MFMA tiles");
+  static_assert(A_CPR == 4 || A_CPR == 8, "BK is 32 or 64");
+  static_assert(B_CPR % 8 == 0, "a B row covers whole 128-byte bank sweeps");
+  static_assert(A_STAGE % 4096 == 0 && B_STAGE % 4096 == 0, "whole 1 KiB loads per wave");
+  static_assert(LDS_BYTES * WAVES_PER_SIMD <= 160 * 1024, "fits the LDS of one CU");
+  static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
+  static_assert(KS >= 2, "the loads of the next chunk ride on the LDS reads of k-step 1");
+};
+
+// One direct load: 64 lanes x 16 bytes from buffer `rsrc` at per-lane byte offset
+// `voff` into LDS at ldsAddr + 16*lane.  ldsAddr must be wave-uniform.
+__device__ __forceinline__ void loadToLds(uint4v rsrc, uint32_t ldsAddr, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(ldsAddr), "v"(voff), "s"(rsrc) : "memory");
+}
+
+template<int N>
+__device__ __forceinline__ void waitVmcnt() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
+__device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  uint4v r;
+  r.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r.z = __builtin_amdgcn_readfirstlane(bytes);
+  r.w = 0x00020000u;
+  return r;
+}
+
+template<class C>
+__global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  __shared__ uint32_t sTicket;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  const cusync::DynStage& stage = p.stage;
+
+  const uint4v rA = rawRsrc(p.A, p.M * p.lda * 2);
+  const uint4v rB = rawRsrc(p.B, p.K * p.ldb * 2);
+  const uint32_t ldsBase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+
+  // ---- direct-load side: which global chunk this lane fetches ---------------
+  // A: load q of this wave fills rows (wave*A_LOADS + q)*A_ROWS_PER_LOAD + lane/A_CPR, slot lane%A_CPR.
+  constexpr int A_SWZ_DIV = 8 / C::A_CPR;                     // rows that share a swizzle value
+  const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + lane / C::A_CPR;
+  const uint32_t aLoadChunk = (lane % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
+  // B: load q fills rows (wave*B_LOADS + q)*B_ROWS_PER_LOAD + lane/B_CPR, slot lane%B_CPR.
+  const uint32_t bLoadRow = wave * C::B_LOADS * C::B_ROWS_PER_LOAD + lane / C::B_CPR;
+  const uint32_t bLoadChunk = (lane % C::B_CPR) ^ (4 * (bLoadRow & 1));
+  static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
+  static_assert(C::B_ROWS_PER_LOAD % 2 == 0, "row parity repeats per load");
+
+  // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
+  // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
+  uint32_t aFrag[C::KS];
+  {
+    const uint32_t row = wm * C::WTM + (lane & 31);
+    const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
+#pragma unroll
+    for (int kk = 0; kk < C::KS; kk++)
+      aFrag[kk] = row * C::A_ROW_BYTES + (((2 * kk + (lane >> 5)) ^ swz) * 16);
+  }
+  // B fragment: transpose read of rows kk*16 + 8*(lane/32) + 4*t + (lane&15)/4,
+  // 4 halfs at column wn*WTN + j*32 + 16*((lane/16)&1) + 4*(lane&3).
+  const uint32_t bFlip = (lane >> 2) & 1;                      // parity of the row this lane reads
+  const uint32_t bRowOff = (8 * (lane >> 5) + ((lane & 15) >> 2)) * C::B_ROW_BYTES;
+  const uint32_t bColOff = (wn * (C::WTN / 8) + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 + (lane & 1) * 8;
+  const uint32_t bFragEven = bRowOff + bColOff + 64 * bFlip;  // MFMA tiles j = 0, 2, ...: slot group j ^ flip
+  const uint32_t bFragOdd = bRowOff + bColOff - 64 * bFlip;   // MFMA tiles j = 1, 3, ...
+
+  if (tid == 0) stage.announceStart(p.launched);
+
+  const uint32_t numTiles = stage.numTiles();
+  const uint32_t nk = (p.K + C::BK - 1) / C::BK;
+  const bool consumer = stage.isConsumer();
+  const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
+  const bool chunkSync = consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
+                         stage.d.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC;
+
+  uint32_t dryXcds = 0;
+  for (uint32_t round = 0;; round++) {
+    if (tid == 0) sTicket = stage.drawTicket(p.launched, round, dryXcds);
+    __syncthreads();
+    const uint32_t ticket = sTicket;
+    if (ticket >= numTiles) break;
+    const cusync_dim3 t = stage.ticketToTile(ticket);
+    const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
+    const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
+
+    floatx16 acc[C::TM][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    // Per-tile byte offsets of this lane's loads at k0 = 0.
+    const uint32_t aVoff0 = ((m0 + aLoadRow) * p.lda + aLoadChunk * 8) * 2;
+    const uint32_t aVstep = C::A_ROWS_PER_LOAD * p.lda * 2;
+    const bool bInRange = n0 + bLoadChunk * 8 < p.N;
+    const uint32_t bVoff0 = (bLoadRow * p.ldb + n0 + bLoadChunk * 8) * 2;
+    const uint32_t bVstep = C::B_ROWS_PER_LOAD * p.ldb * 2;
+
+    // ---- consumer side (same protocol as the staged kernel) ------------------
+    uint32_t nextColTile = 0;
+    const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
+    uint32_t polledTile = 0xffffffffu, polledValue = 0;
+    auto waitRows = [&](uint32_t col, uint32_t z) {
+      for (uint32_t r = m0; r < mEnd; r = (r / tmq + 1) * tmq) {
+        cusync_dim3 w = {r, col, z};
+        stage.waitWave(w);
+      }
+    };
+    auto waitChunk = [&](uint32_t k0) {
+      if (!chunkSync) return;
+      const uint32_t kLast = min(k0 + (uint32_t)C::BK, p.K) - 1;
+      for (; nextColTile <= kLast / tnq; nextColTile++) {
+        if (oneRowBlock && nextColTile == polledTile && cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) continue;
+        waitRows(nextColTile * tnq, 0);
+      }
+    };
+    auto earlyPoll = [&](uint32_t k0) {
+      if (!oneRowBlock || k0 >= p.K) return;
+      const uint32_t ct = k0 / tnq;
+      if (ct < nextColTile || ct == polledTile) return;
+      polledTile = ct;
+      cusync_dim3 w = {m0, ct * tnq, 0};
+      polledValue = stage.peekBegin(w);
+    };
+
+    // Direct load number q (B loads first, then A) of chunk kt into stage S.
+    // Columns / rows outside the operands are redirected out of range and land
+    // in LDS as zeros, so chunks past the end of K may be issued harmlessly.
+    auto issueOne = [&](auto SP, auto QP, uint32_t kt) {
+      constexpr int S = decltype(SP)::value;
+      constexpr int Q = decltype(QP)::value;
+      const uint32_t k0 = kt * C::BK;
+      if constexpr (Q < C::B_LOADS) {
+        const uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
+        loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), bInRange ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange);
+      } else {
+        constexpr int QA = Q - C::B_LOADS;
+        const bool aInRange = k0 + aLoadChunk * 8 < p.K;
+        const uint32_t lds = ldsBase + S * C::A_STAGE + (wave * C::A_LOADS + QA) * 1024;
+        loadToLds(rA, __builtin_amdgcn_readfirstlane(lds), aInRange ? aVoff0 + k0 * 2 + QA * aVstep : kOutOfRange);
+      }
+    };
+    auto issueAll = [&](auto SP, uint32_t kt) {
+      staticFor<C::LOADS>([&](auto QP) { issueOne(SP, QP, kt); });
+    };
+
+    // MFMA pass over stage S.  The direct loads of chunk ktLoad (into stage SL)
+    // are issued one at a time between the LDS reads of the first k-step, so
+    // that they trickle into the memory pipeline under the MFMAs instead of
+    // arriving as one burst that stalls the wave.
+    auto compute = [&](auto SP, auto SLP, uint32_t ktLoad) {
+      constexpr int S = decltype(SP)::value;
+      const char* sa = smem + S * C::A_STAGE;
+      const char* sbE = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE + bFragEven;
+      const char* sbO = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE + bFragOdd;
+      half8 fa[2][C::TM], fb[2][C::TN];
+      constexpr int R = C::TM + C::TN;                 // fragment loads per k-step (a B fragment is two reads)
+      // Fragment f of a k-step: f < TM is A tile f, otherwise B tile f - TM.
+      auto loadFrag = [&](auto FP, int slot, int kk) {
+        constexpr int F = decltype(FP)::value;
+        if constexpr (F < C::TM) {
+          fa[slot][F] = *reinterpret_cast<const half8*>(sa + aFrag[kk] + F * 32 * C::A_ROW_BYTES);
+        } else {
+          constexpr int J = F - C::TM;
+          typedef short4v __attribute__((address_space(3))) * lds_ptr;
+          const char* q = ((J & 1) ? sbO : sbE) + J * 64 + kk * 16 * C::B_ROW_BYTES;
+          short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
+          short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * C::B_ROW_BYTES));
+          half4 l4 = __builtin_bit_cast(half4, lo), h4 = __builtin_bit_cast(half4, hi);
+          fb[slot][J] = __builtin_shufflevector(l4, h4, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      };
+      auto loadFrags = [&](int slot, int kk) {
+        staticFor<R>([&](auto FP) { loadFrag(FP, slot, kk); });
+      };
+      // Fragments of k-step 1 with the direct loads spread between them.
+      auto loadFragsAndIssue = [&](int slot, int kk) {
+        staticFor<R>([&](auto FP) {
+          loadFrag(FP, slot, kk);
+          staticFor<C::LOADS>([&](auto QP) {
+            if constexpr (decltype(QP)::value * R / C::LOADS == decltype(FP)::value) issueOne(SLP, QP, ktLoad);
+          });
+        });
+      };
+      loadFrags(0, 0);
+#pragma unroll
+      for (int kk = 0; kk < C::KS; kk++) {
+        if (kk == 0 && C::KS > 1) loadFragsAndIssue(1, 1);
+        else if (kk + 1 < C::KS) loadFrags((kk + 1) & 1, kk + 1);
+#pragma unroll
+        for (int i = 0; i < C::TM; i++)
+#pragma unroll
+          for (int j = 0; j < C::TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+      }
+      schedPass<C::KS, C::TM * C::TN, C::TM + 2 * C::TN, 0>();
+    };
+
+    // Iteration kt on stage S = kt % STAGES.  Chunks kt+1 .. kt+STAGES-2 are the
+    // ones this wave still has in flight behind chunk kt.
+    auto step = [&](auto SP, uint32_t kt) {
+      constexpr int S = decltype(SP)::value;
+      waitVmcnt<(C::STAGES - 2) * C::LOADS>();
+      __builtin_amdgcn_s_barrier();      // chunk kt is in LDS for everyone; everyone is done with chunk kt-1
+      asm volatile("" ::: "memory");
+      const uint32_t ktLoad = kt + C::STAGES - 1;
+      if (ktLoad < nk) waitChunk(ktLoad * C::BK);
+      earlyPoll((ktLoad + 1) * C::BK);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(SP, Parity<(S + C::STAGES - 1) % C::STAGES>{}, ktLoad);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (consumer) {
+      cusync_dim3 w = {m0, 0, 1};
+      if (stage.needsWait(w)) {
+        if (wave == 0) waitRows(0, 1);
+        __syncthreads();
+      }
+    }
+
+    // Prologue: chunks 0 .. STAGES-2 (chunks past the end of K load zeros).
+    waitChunk(0);
+    issueAll(Parity<0>{}, 0);
+    if constexpr (C::STAGES > 2) { if (nk > 1) waitChunk(C::BK); issueAll(Parity<1>{}, 1); }
+    if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(2 * C::BK); issueAll(Parity<2>{}, 2); }
+    static_assert(C::STAGES >= 2 && C::STAGES <= 4, "prologue written for 2..4 stages");
+    earlyPoll((C::STAGES - 1) * C::BK);
+
+    for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
+      step(Parity<0>{}, kt);
+      if (kt + 1 < nk) step(Parity<1 % C::STAGES>{}, kt + 1);
+      if (C::STAGES > 2 && kt + 2 < nk) step(Parity<2 % C::STAGES>{}, kt + 2);
+      if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
+    }
+
+    // Epilogue (see the staged kernel for the accumulator layout).
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+      const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+          half4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(acc[i][j][g * 4 + e], p.epilogue);
+          if (m < p.M && n < p.N)
+            *reinterpret_cast<half4*>(p.D + (size_t)m * p.ldd + n) = o;
+        }
+      }
+    }
+
+    // All waves must be past their last LDS read before the next tile's loads
+    // land in stage 0; the post (or this barrier) provides that.
+    cusync_dim3 done = {m0, n0, t.z};
+    if (stage.isProducer()) stage.post(done);
+    else __syncthreads();
+  }
+}
+
+}  // namespace gemm
+}  // namespace cusync

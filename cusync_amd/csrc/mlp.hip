@@ -30,22 +30,23 @@ namespace {
 
 using cusync::rt::setError;
 
-// Built-in choice of tile shapes per batch size for 256 CUs.  Rows of the output
-// decide the M extent; the N extent is picked so that the number of tiles of the
-// two GEMMs together stays close to a multiple of what the device holds.
-void pickTiles(const cusync_mlp_config& c, int* t1, int* t2) {
-  int t;
-  if (c.batch <= 32) t = CUSYNC_TILE_32x128x64;
-  else if (c.batch <= 64) t = CUSYNC_TILE_64x128x64;
-  else if (c.batch <= 128) t = CUSYNC_TILE_128x128x64;
-  else t = CUSYNC_TILE_256x128x64;
-  if (c.model == CUSYNC_MLP_LLAMA && c.inner % 128 != 0) {
-    // gate|up split must fall on a tile boundary (2752 = 43 * 64)
-    t = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
-  }
-  *t1 = c.tile1 >= 0 ? c.tile1 : t;
-  *t2 = c.tile2 >= 0 ? c.tile2 : (c.model == CUSYNC_MLP_LLAMA && c.inner % 128 != 0
-                                      ? (c.batch <= 128 ? CUSYNC_TILE_128x128x64 : CUSYNC_TILE_256x128x64) : t);
+// Built-in choice of tile shapes per batch size for 256 CUs.  From 256 rows up
+// the direct-to-LDS 128x256 tile (two workgroups per CU) is the fastest one
+// measured; below that the M extent follows the batch.  A SwiGLU consumer has
+// to use a register-staged tile, and StridedSync needs the gate|up split on a
+// tile boundary (2752 = 43 * 64).
+void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* t2) {
+  int small;
+  if (c.batch <= 32) small = CUSYNC_TILE_32x128x64;
+  else if (c.batch <= 64) small = CUSYNC_TILE_64x128x64;
+  else small = CUSYNC_TILE_128x128x64;
+  const bool big = c.batch > 128;
+  int a = big ? CUSYNC_TILE_128x256x32 : small;
+  int b = big ? (swiglu ? CUSYNC_TILE_256x128x64 : CUSYNC_TILE_128x256x32) : small;
+  if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
+    a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
+  *t1 = c.tile1 >= 0 ? c.tile1 : a;
+  *t2 = c.tile2 >= 0 ? c.tile2 : b;
 }
 
 cusync_policy_desc noSync() {
@@ -101,8 +102,10 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->ldh = m->n1;
   m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : CUSYNC_EPILOGUE_NONE;
   m->aMode2 = (llama && cfg->activation) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
-  pickTiles(*cfg, &m->tile1, &m->tile2);
 
+  int sync = cfg->sync;
+  if (llama && sync == CUSYNC_SYNC_TILE && m->aMode2 == CUSYNC_A_SWIGLU && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
+  pickTiles(*cfg, sync, m->aMode2 == CUSYNC_A_SWIGLU, &m->tile1, &m->tile2);
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
     setError("mlp: unknown tile id");
@@ -110,8 +113,6 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     return nullptr;
   }
 
-  int sync = cfg->sync;
-  if (llama && sync == CUSYNC_SYNC_TILE && m->aMode2 == CUSYNC_A_SWIGLU) sync = CUSYNC_SYNC_STRIDED;
   cusync_policy_desc pol = noSync();
   int opts = 0;
   const cusync_dim3 g1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, 1);

@@ -95,17 +95,18 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   if (!d || !host_tile_order) return CUSYNC_ERROR_NOT_INITIALIZED;
   const uint32_t n = numTiles(d);
   if (n == 0) { cusync::rt::setError("cusync_stage_alloc: empty grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr;
+  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr; d->xcdTickets = nullptr;
   d->kernelExecuted = nullptr; d->spinTimeouts = nullptr; d->tileStatusWrite = nullptr;
-  // The three small counters share one allocation: [tileCounter, startCounter, spinTimeouts, kernelExecuted]
-  // each on its own 128-byte line so that polling one does not disturb the others.
+  // The small counters share one allocation: [tileCounter, startCounter, spinTimeouts, kernelExecuted,
+  // xcdTickets[9]], each on its own 128-byte line so that polling one does not disturb the others.
   const size_t line = 128;
   char* counters = nullptr;
-  if (RT(hipMalloc((void**)&counters, 4 * line))) return CUSYNC_ERROR_DEVICE;
-  if (RT(hipMemset(counters, 0, 4 * line))) return CUSYNC_ERROR_DEVICE;
+  if (RT(hipMalloc((void**)&counters, 13 * line))) return CUSYNC_ERROR_DEVICE;
+  if (RT(hipMemset(counters, 0, 13 * line))) return CUSYNC_ERROR_DEVICE;
   d->tileCounter = (uint32_t*)(counters);
   d->startCounter = (uint32_t*)(counters + line);
   d->spinTimeouts = (uint32_t*)(counters + 2 * line);
+  d->xcdTickets = (uint32_t*)(counters + 4 * line);
   const bool producer = d->out.kind != CUSYNC_POLICY_NOSYNC;
   if (producer && !(d->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) d->kernelExecuted = (uint32_t*)(counters + 3 * line);
   if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return CUSYNC_ERROR_DEVICE;
@@ -123,7 +124,7 @@ cusync_error cusync_stage_free(cusync_stage_desc* d) {
   if (d->tileCounter) bad |= RT(hipFree(d->tileCounter));       // base of the counters block
   if (d->tileOrder) bad |= RT(hipFree(d->tileOrder));
   if (d->tileStatusWrite) bad |= RT(hipFree(d->tileStatusWrite));
-  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr;
+  d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr; d->xcdTickets = nullptr;
   d->kernelExecuted = nullptr; d->spinTimeouts = nullptr; d->tileStatusWrite = nullptr;
   return bad ? CUSYNC_ERROR_DEVICE : CUSYNC_SUCCESS;
 }
@@ -185,7 +186,14 @@ cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems,
     bad |= RT(hipMemcpy(sems, d->tileStatusWrite, sizeof(uint32_t) * n, hipMemcpyDeviceToHost));
   }
   if (tile_order) bad |= RT(hipMemcpy(tile_order, d->tileOrder, sizeof(cusync_dim3) * n, hipMemcpyDeviceToHost));
-  if (tile_counter) bad |= RT(hipMemcpy(tile_counter, d->tileCounter, 4, hipMemcpyDeviceToHost));
+  if (tile_counter) {
+    // the plain dispenser plus the nine per-XCD counters: all must be back at 0 between runs
+    uint32_t block[13 * 32];
+    bad |= RT(hipMemcpy(block, d->tileCounter, sizeof block, hipMemcpyDeviceToHost));
+    uint32_t sum = block[0];
+    for (int i = 0; i < 9; i++) sum += block[(4 + i) * 32];
+    *tile_counter = sum;
+  }
   if (start_counter) bad |= RT(hipMemcpy(start_counter, d->startCounter, 4, hipMemcpyDeviceToHost));
   if (spin_timeouts) bad |= RT(hipMemcpy(spin_timeouts, d->spinTimeouts, 4, hipMemcpyDeviceToHost));
   if (kernel_executed) {

@@ -47,19 +47,52 @@ struct DynStage {
     }
   }
 
+  // Id of the XCD (accelerator die) this wave runs on, 0..7.
+  static __device__ __forceinline__ uint32_t xcdId() {
+    uint32_t x;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+    return x & 7u;
+  }
+
   // Draws the next ticket for this workgroup (first thread only).  `round` is
-  // how many tickets this workgroup has already drawn.  Returns numTiles() or
-  // more when the tiles have run out.
-  __device__ __forceinline__ uint32_t drawTicket(uint32_t launched, uint32_t round) const {
+  // how many tickets this workgroup has already drawn, `dry` a bit mask the
+  // caller keeps across rounds (start it at 0).  Returns numTiles() or more
+  // when the tiles have run out.
+  //
+  // Each of the eight XCDs has its own L2, so which workgroup gets which tile
+  // decides how much of the operands is re-fetched from memory.  The tiles are
+  // therefore dealt per XCD: XCD x owns the column tiles [x*gx/8, (x+1)*gx/8) of
+  // every row, in row-major order, and a workgroup draws from the dispenser of
+  // the XCD it runs on.  The workgroups of one XCD thus share the same few B
+  // column panels (and, row by row, the same A panels) in their L2.  A
+  // workgroup whose own dispenser is empty helps the next XCD, so the end of the
+  // launch stays balanced.  The ticket returned is the tile's position in the
+  // row-major schedule; it still goes through the stage's ticket -> tile table.
+  __device__ __forceinline__ uint32_t drawTicket(uint32_t launched, uint32_t round, uint32_t& dry) const {
     if (!customOrder()) {
       const uint32_t wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
       return wg + round * launched;
     }
-    const uint32_t t = dev::ticketAdd(d.tileCounter, 1);
-    // Every workgroup draws exactly one ticket past the end; the last of those
-    // re-arms the dispenser for the next run.
-    if (t == numTiles() + launched - 1) dev::storeRelaxed(d.tileCounter, 0);
-    return t;
+    constexpr uint32_t kLine = 32;          // counters are 128 bytes apart
+    const uint32_t mine = xcdId();
+    for (uint32_t s = 0; s < 8; s++) {
+      const uint32_t x = (mine + s) & 7u;
+      if (dry & (1u << x)) continue;
+      const uint32_t lo = x * d.grid.x / 8, cols = (x + 1) * d.grid.x / 8 - lo;
+      const uint32_t count = cols * d.grid.y * d.grid.z;
+      if (count != 0) {
+        const uint32_t l = dev::ticketAdd(&d.xcdTickets[x * kLine], 1);
+        if (l < count) return lo + l % cols + (l / cols) * d.grid.x;
+      }
+      dry |= 1u << x;
+    }
+    // Nothing left anywhere.  The last workgroup to find that out re-arms the
+    // dispensers for the next run.
+    const uint32_t finished = dev::ticketAdd(&d.xcdTickets[8 * kLine], 1);
+    if (finished == launched - 1) {
+      for (uint32_t x = 0; x < 9; x++) dev::storeRelaxed(&d.xcdTickets[x * kLine], 0);
+    }
+    return 0xffffffffu;
   }
 
   __device__ __forceinline__ cusync_dim3 ticketToTile(uint32_t ticket) const {
@@ -78,10 +111,11 @@ struct DynStage {
   // Per-run count a semaphore of the input policy must reach.
   __device__ __forceinline__ uint32_t waitTarget() const { return (uint32_t)d.iter * dyn::waitValue(d.in); }
 
-  // Current value of the semaphore guarding `tile`, without waiting and without
-  // ordering: the caller compares it with waitTarget() later, after other work.
-  __device__ __forceinline__ uint32_t peek(const cusync_dim3& tile) const {
-    return dev::pollOnce(&d.tileStatusRead[dyn::tileIndex(d.in, tile, d.prodGrid)]);
+  // Starts a read of the semaphore guarding `tile` without waiting for it and
+  // without ordering; dev::pollFinish() on the result, after other work, gives
+  // the value to compare with waitTarget().
+  __device__ __forceinline__ uint32_t peekBegin(const cusync_dim3& tile) const {
+    return dev::pollBegin(&d.tileStatusRead[dyn::tileIndex(d.in, tile, d.prodGrid)]);
   }
 
   // Wave-uniform wait: every lane of the calling wave passes the same tile.

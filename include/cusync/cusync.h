@@ -78,6 +78,7 @@ private:
   dim3* tileOrder;                  // device: ticket -> tile
   uint32_t* tileCounter;            // device: ticket dispenser
   uint32_t* startCounter_;          // device: used by the prebuilt persistent kernels
+  uint32_t* xcdTickets_;            // device: per-XCD ticket dispensers of the prebuilt kernels
   uint32_t* kernelExecuted_;        // device: wait-kernel flag
   uint32_t* spinTimeouts_;          // device: waits that gave up
   volatile uint32_t* tileStatusWrite_;
@@ -112,6 +113,7 @@ private:
     tileOrder = (dim3*)d.tileOrder;
     tileCounter = d.tileCounter;
     startCounter_ = d.startCounter;
+    xcdTickets_ = d.xcdTickets;
     kernelExecuted_ = d.kernelExecuted;
     spinTimeouts_ = d.spinTimeouts;
     tileStatusWrite_ = d.tileStatusWrite;
@@ -131,7 +133,7 @@ public:
   CuStage(dim3 grid, dim3 tileSize, InputSyncPolicy inputPolicy, OutputSyncPolicy outputPolicy)
       : grid_(grid), prodGrid_(0, 0, 0), tileSize_(tileSize), iter(1),
         inputPolicy_(inputPolicy), outputPolicy_(outputPolicy),
-        tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
+        tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), xcdTickets_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
         tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncSuccess) {
     static_assert(!((Opts & NoAtomicAdd) && std::is_same<OutputSyncPolicy, NoSync>::value &&
                     std::is_same<InputSyncPolicy, NoSync>::value), "NoAtomicAdd on a stage that never syncs");
@@ -140,7 +142,7 @@ public:
 
   CUSYNC_DEVICE_HOST CuStage()
       : grid_(0, 0, 0), prodGrid_(0, 0, 0), tileSize_(0, 0, 0), iter(1),
-        tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
+        tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), xcdTickets_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
         tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncErrorNotInitialized) {}
 
   // Outcome of construction: CuSyncSuccess, or CuSyncErrorInvalidLinearBlockIndex
@@ -166,7 +168,7 @@ public:
   void destroy() {
     cusync_stage_desc d = desc();
     cusync_stage_free(&d);
-    tileOrder = nullptr; tileCounter = nullptr; startCounter_ = nullptr;
+    tileOrder = nullptr; tileCounter = nullptr; startCounter_ = nullptr; xcdTickets_ = nullptr;
     kernelExecuted_ = nullptr; spinTimeouts_ = nullptr; tileStatusWrite_ = nullptr;
   }
 
@@ -193,6 +195,7 @@ public:
     d.tileOrder = (cusync_dim3*)tileOrder;
     d.tileCounter = tileCounter;
     d.startCounter = startCounter_;
+    d.xcdTickets = xcdTickets_;
     d.kernelExecuted = kernelExecuted_;
     d.spinTimeouts = spinTimeouts_;
     d.tileStatusWrite = (uint32_t*)tileStatusWrite_;

@@ -40,16 +40,19 @@ CUSYNC_DEVICE void acquireFence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "ag
 #define CUSYNC_SPIN_LIMIT (1u << 20)
 #endif
 
-// One poll of a semaphore by a whole wave: only the first active lane touches
-// memory, the value is broadcast to the others.  (Sixty-four lanes loading the
-// same coherent address are sixty-four requests to one memory channel.)
-CUSYNC_DEVICE uint32_t pollOnce(const volatile uint32_t* addr) {
+// First half of a poll by a whole wave: only the first active lane touches
+// memory (sixty-four lanes loading the same coherent address are sixty-four
+// requests to one memory channel).  The result stays in that lane's register so
+// the wave need not wait for it yet; pollFinish() broadcasts it.
+CUSYNC_DEVICE uint32_t pollBegin(const volatile uint32_t* addr) {
   uint32_t v = 0;
   const uint64_t exec = __builtin_amdgcn_read_exec();
   const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(exec >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)exec, 0u));
   if (before == 0) v = loadRelaxed(addr);
-  return __builtin_amdgcn_readfirstlane(v);
+  return v;
 }
+CUSYNC_DEVICE uint32_t pollFinish(uint32_t begun) { return __builtin_amdgcn_readfirstlane(begun); }
+CUSYNC_DEVICE uint32_t pollOnce(const volatile uint32_t* addr) { return pollFinish(pollBegin(addr)); }
 
 // Polls *addr until it is >= want; returns false if the poll budget ran out.
 // Sleeps between polls and doubles the sleep up to a few microseconds: a

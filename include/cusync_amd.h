@@ -83,6 +83,8 @@ typedef struct cusync_stage_desc {
   cusync_dim3 *tileOrder;     /* [numTiles] ticket -> tile */
   uint32_t *tileCounter;      /* ticket dispenser; 0 between runs */
   uint32_t *startCounter;     /* counts workgroups that have begun; 0 between runs */
+  uint32_t *xcdTickets;       /* 9 counters, 128 bytes apart: one ticket dispenser per XCD for the prebuilt
+                                 kernels plus a count of workgroups that ran dry; all 0 between runs */
   uint32_t *kernelExecuted;   /* wait-kernel flag: == iter once every workgroup of the run has begun */
   uint32_t *spinTimeouts;     /* number of waits of this stage that gave up (0 in a healthy chain) */
   uint32_t *tileStatusWrite;  /* semaphores this stage posts */
@@ -167,7 +169,9 @@ enum {
   CUSYNC_A_SWIGLU = 1          /* A[m,k] = silu(G[m,k]) * G[m,k + K]; G has K*2 valid columns */
 };
 
-/* Tile shapes the library was built with. */
+/* Tile shapes the library was built with.  256x256x32, 256x128x32, 128x256x32 and
+ * 128x128x32 move their operands from global memory straight into LDS and have no SwiGLU
+ * variant; the others stage them through registers. */
 enum {
   CUSYNC_TILE_256x256x32 = 0,
   CUSYNC_TILE_256x128x64 = 1,
@@ -177,7 +181,10 @@ enum {
   CUSYNC_TILE_128x256x64 = 5,
   CUSYNC_TILE_256x64x64 = 6,
   CUSYNC_TILE_128x64x64 = 7,
-  CUSYNC_TILE_COUNT = 8
+  CUSYNC_TILE_256x128x32 = 8,
+  CUSYNC_TILE_128x256x32 = 9,
+  CUSYNC_TILE_128x128x32 = 10,
+  CUSYNC_TILE_COUNT = 11
 };
 
 typedef struct cusync_gemm_args {
