@@ -45,7 +45,8 @@ class GemmArgs(C.Structure):
 
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
-                ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32)]
+                ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
+                ("split_k1", i32), ("split_k2", i32)]
 
 
 # every symbol include/cusync_amd.h declares: name -> (restype, argtypes)
@@ -94,6 +95,7 @@ SIGNATURES = {
     "cusync_mlp_run_split": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_mlp_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
     "cusync_mlp_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "cusync_mlp_splits": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
 }
 
 _lib = None

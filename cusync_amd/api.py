@@ -178,13 +178,13 @@ def gemm_grid(tile, M, N, split_k=1):
 
 
 def gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, epilogue=EPI.NONE, a_mode=0, split_k=1,
-              max_workgroups=0):
+              max_workgroups=0, workspace=None):
     a = GemmArgs()
     a.stage = stage.desc
     a.M, a.N, a.K = M, N, K
     a.A, a.lda, a.B, a.ldb, a.D, a.ldd = A, lda, B, ldb, D, ldd
     a.epilogue, a.a_mode, a.tile, a.split_k = epilogue, a_mode, tile, split_k
-    a.workspace = None
+    a.workspace = workspace
     a.max_workgroups = max_workgroups
     return a
 
@@ -200,9 +200,10 @@ def gemm(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, stream=None, **kw):
 class Mlp:
     """Handle over cusync_mlp_* (the reference's libmlp C surface, src/ml-bench/transformer/mlp-lib.cu:555-618)."""
 
-    def __init__(self, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=-1, tile2=-1, opts=-1, activation=1):
+    def __init__(self, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=-1, tile2=-1, opts=-1, activation=1,
+                 split_k1=0, split_k2=0):
         self.L = _lib.load()
-        self.cfg = MlpConfig(model, batch, hidden, inner, sync, tile1, tile2, opts, activation)
+        self.cfg = MlpConfig(model, batch, hidden, inner, sync, tile1, tile2, opts, activation, split_k1, split_k2)
         self.h = self.L.cusync_mlp_create(C.byref(self.cfg), w1_ptr, w2_ptr)
         if not self.h:
             raise RuntimeError("cusync_mlp_create failed: " + last_error())
@@ -220,6 +221,11 @@ class Mlp:
     def tiles(self):
         a, b = C.c_int(0), C.c_int(0)
         self.L.cusync_mlp_tiles(self.h, C.byref(a), C.byref(b))
+        return a.value, b.value
+
+    def splits(self):
+        a, b = C.c_int(0), C.c_int(0)
+        self.L.cusync_mlp_splits(self.h, C.byref(a), C.byref(b))
         return a.value, b.value
 
     def stage_state(self, which):

@@ -20,6 +20,7 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr uint32_t kOutOfRange = 0x80000000u;   // buffer offset beyond any descriptor we build
@@ -33,6 +34,11 @@ struct GemmParams {
   int32_t epilogue;
   int32_t a_mode;
   uint32_t launched;       // workgroups in this launch
+  // split-K: slice z of a tile covers K columns [z*kPerSlice, (z+1)*kPerSlice)
+  uint32_t splitK, kPerSlice;
+  float* partials;         // [splitK][mPad][N] fp32 partial sums
+  uint32_t* arrivals;      // [m-tiles * n-tiles] slices finished per output tile; 0 between launches
+  uint32_t mPad;           // m-tiles * BM
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void* base, uint32_t bytes) {
@@ -108,6 +114,83 @@ __device__ __forceinline__ void schedPass() {
     if constexpr (M + 1 < NM) schedPass<STEPS, NM, R, W, S, M + 1>();
     else schedPass<STEPS, NM, R, W, S + 1, 0>();
   }
+}
+
+// Writes the accumulators of one output tile and tells the caller whether this
+// workgroup completed the tile (and therefore posts it).
+//
+// acc[i][j][r] of lane l is output row  m0 + wm*WTM + i*32 + (l & 31)  and column
+// n0 + wn*WTN + j*32 + 8*(r/4) + 4*(l/32) + r%4.
+//
+// Without split-K the epilogue is applied and the fp16 result stored.  With
+// split-K the slice's fp32 partial sums go to the workspace; the slice that
+// arrives last (per-tile counter, release/acquire at agent scope because the
+// slices ran on different XCDs) adds the slices in index order — so the result
+// does not depend on arrival order — applies the epilogue, stores, re-arms the
+// counter and posts.  Must be called by all threads of the workgroup.
+template<class C>
+__device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
+                                           const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast) {
+  const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
+  auto storeFinal = [&](auto&& value) {
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+      const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+          if (m < p.M && n < p.N) {
+            const floatx4 v = value(i, j, g, m, n);
+            half4 o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
+            *reinterpret_cast<half4*>(p.D + (size_t)m * p.ldd + n) = o;
+          }
+        }
+      }
+    }
+  };
+  if (p.splitK <= 1) {
+    storeFinal([&](int i, int j, int g, uint32_t, uint32_t) {
+      return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+    });
+    return true;
+  }
+  const size_t sliceStride = (size_t)p.mPad * p.N;
+#pragma unroll
+  for (int i = 0; i < C::TM; i++) {
+    const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+        if (m < p.M && n < p.N)
+          *reinterpret_cast<floatx4*>(p.partials + t.z * sliceStride + (size_t)m * p.N + n) =
+              floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t* counter = p.arrivals + t.y * p.stage.d.grid.x + t.x;
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = before == p.splitK - 1;
+    if (last) dev::storeRelaxed(counter, 0);
+    *sLast = last;
+  }
+  __syncthreads();
+  if (!*sLast) return false;
+  dev::acquireFence();
+  storeFinal([&](int, int, int, uint32_t m, uint32_t n) {
+    floatx4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t z = 0; z < p.splitK; z++)
+      sum += *reinterpret_cast<const floatx4*>(p.partials + z * sliceStride + (size_t)m * p.N + n);
+    return sum;
+  });
+  return true;
 }
 
 template<int P> struct Parity { static constexpr int value = P; };

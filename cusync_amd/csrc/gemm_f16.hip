@@ -146,7 +146,12 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   }
   if (((uintptr_t)a->A | (uintptr_t)a->B) % 16 || (uintptr_t)a->D % 8) { setError("gemm: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->a_mode == CUSYNC_A_SWIGLU && !ti->kernel[1]) { setError("gemm: this tile shape has no SwiGLU variant"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if (a->split_k > 1) { setError("gemm: split_k > 1 is not built"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->split_k < 1) { setError("gemm: split_k must be at least 1"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->split_k > 1) {
+    if ((uint32_t)a->split_k > (a->K + ti->bk - 1) / ti->bk) { setError("gemm: more k-slices than K chunks"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (!a->workspace || (uintptr_t)a->workspace % 16) { setError("gemm: split_k > 1 needs a 16-byte aligned workspace of cusync_gemm_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  }
   if (a->a_mode != CUSYNC_A_PLAIN && a->a_mode != CUSYNC_A_SWIGLU) { setError("gemm: unknown a_mode"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_RELU) { setError("gemm: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
@@ -169,9 +174,17 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   return CUSYNC_SUCCESS;
 }
 
+// [split_k][m-tiles*BM][N] fp32 partial sums, then one arrival counter per output tile.
+static size_t partialBytes(const cusync_gemm_args* a, const TileInfo* ti) {
+  const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
+  return (size_t)a->split_k * g.y * ti->bm * a->N * sizeof(float);
+}
+
 size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {
-  (void)a;
-  return 0;
+  TileInfo* ti = a ? tileInfo(a->tile) : nullptr;
+  if (!ti || a->split_k <= 1) return 0;
+  const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
+  return partialBytes(a, ti) + (size_t)g.x * g.y * sizeof(uint32_t);
 }
 
 cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
@@ -198,6 +211,12 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   p.epilogue = a->epilogue;
   p.a_mode = a->a_mode;
   p.launched = launched;
+  p.splitK = (uint32_t)a->split_k;
+  const uint32_t chunks = (a->K + ti->bk - 1) / ti->bk;
+  p.kPerSlice = (chunks + p.splitK - 1) / p.splitK * ti->bk;
+  p.mPad = s.grid.y * ti->bm;
+  p.partials = (float*)a->workspace;
+  p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
   hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(kThreads), ti->lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;

@@ -76,7 +76,7 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
 template<class C>
 __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  __shared__ uint32_t sTicket;
+  __shared__ uint32_t sTicket, sLast;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -120,7 +120,6 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   if (tid == 0) stage.announceStart(p.launched);
 
   const uint32_t numTiles = stage.numTiles();
-  const uint32_t nk = (p.K + C::BK - 1) / C::BK;
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
   const bool chunkSync = consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
@@ -135,6 +134,8 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     const cusync_dim3 t = stage.ticketToTile(ticket);
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
+    const uint32_t kBegin = t.z * p.kPerSlice, kEnd = min(p.K, kBegin + p.kPerSlice);
+    const uint32_t nk = (kEnd - kBegin + C::BK - 1) / C::BK;
 
     floatx16 acc[C::TM][C::TN];
 #pragma unroll
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     const uint32_t bVstep = C::B_ROWS_PER_LOAD * p.ldb * 2;
 
     // ---- consumer side (same protocol as the staged kernel) ------------------
-    uint32_t nextColTile = 0;
+    uint32_t nextColTile = kBegin / tnq;
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
     uint32_t polledTile = 0xffffffffu, polledValue = 0;
     auto waitRows = [&](uint32_t col, uint32_t z) {
@@ -163,14 +164,14 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     };
     auto waitChunk = [&](uint32_t k0) {
       if (!chunkSync) return;
-      const uint32_t kLast = min(k0 + (uint32_t)C::BK, p.K) - 1;
+      const uint32_t kLast = min(k0 + (uint32_t)C::BK, kEnd) - 1;
       for (; nextColTile <= kLast / tnq; nextColTile++) {
         if (oneRowBlock && nextColTile == polledTile && cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) continue;
         waitRows(nextColTile * tnq, 0);
       }
     };
     auto earlyPoll = [&](uint32_t k0) {
-      if (!oneRowBlock || k0 >= p.K) return;
+      if (!oneRowBlock || k0 >= kEnd) return;
       const uint32_t ct = k0 / tnq;
       if (ct < nextColTile || ct == polledTile) return;
       polledTile = ct;
@@ -179,18 +180,19 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     };
 
     // Direct load number q (B loads first, then A) of chunk kt into stage S.
-    // Columns / rows outside the operands are redirected out of range and land
-    // in LDS as zeros, so chunks past the end of K may be issued harmlessly.
+    // Columns / rows outside the operands or past the end of this K slice are
+    // redirected out of range and land in LDS as zeros, so chunks past the end
+    // may be issued harmlessly.
     auto issueOne = [&](auto SP, auto QP, uint32_t kt) {
       constexpr int S = decltype(SP)::value;
       constexpr int Q = decltype(QP)::value;
-      const uint32_t k0 = kt * C::BK;
+      const uint32_t k0 = kBegin + kt * C::BK;
       if constexpr (Q < C::B_LOADS) {
         const uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
-        loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), bInRange ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange);
+        loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), (bInRange && k0 < kEnd) ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange);
       } else {
         constexpr int QA = Q - C::B_LOADS;
-        const bool aInRange = k0 + aLoadChunk * 8 < p.K;
+        const bool aInRange = k0 + aLoadChunk * 8 < kEnd;   // never touch columns the slice has not waited for
         const uint32_t lds = ldsBase + S * C::A_STAGE + (wave * C::A_LOADS + QA) * 1024;
         loadToLds(rA, __builtin_amdgcn_readfirstlane(lds), aInRange ? aVoff0 + k0 * 2 + QA * aVstep : kOutOfRange);
       }
@@ -259,8 +261,8 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       __builtin_amdgcn_s_barrier();      // chunk kt is in LDS for everyone; everyone is done with chunk kt-1
       asm volatile("" ::: "memory");
       const uint32_t ktLoad = kt + C::STAGES - 1;
-      if (ktLoad < nk) waitChunk(ktLoad * C::BK);
-      earlyPoll((ktLoad + 1) * C::BK);
+      if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
+      earlyPoll(kBegin + (ktLoad + 1) * C::BK);
       __builtin_amdgcn_sched_barrier(0);
       compute(SP, Parity<(S + C::STAGES - 1) % C::STAGES>{}, ktLoad);
       __builtin_amdgcn_sched_barrier(0);
@@ -275,12 +277,12 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     }
 
     // Prologue: chunks 0 .. STAGES-2 (chunks past the end of K load zeros).
-    waitChunk(0);
+    waitChunk(kBegin);
     issueAll(Parity<0>{}, 0);
-    if constexpr (C::STAGES > 2) { if (nk > 1) waitChunk(C::BK); issueAll(Parity<1>{}, 1); }
-    if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(2 * C::BK); issueAll(Parity<2>{}, 2); }
+    if constexpr (C::STAGES > 2) { if (nk > 1) waitChunk(kBegin + C::BK); issueAll(Parity<1>{}, 1); }
+    if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); issueAll(Parity<2>{}, 2); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 4, "prologue written for 2..4 stages");
-    earlyPoll((C::STAGES - 1) * C::BK);
+    earlyPoll(kBegin + (C::STAGES - 1) * C::BK);
 
     for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
       step(Parity<0>{}, kt);
@@ -289,28 +291,12 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
     }
 
-    // Epilogue (see the staged kernel for the accumulator layout).
-#pragma unroll
-    for (int i = 0; i < C::TM; i++) {
-      const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
-#pragma unroll
-      for (int j = 0; j < C::TN; j++) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
-          half4 o;
-#pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(acc[i][j][g * 4 + e], p.epilogue);
-          if (m < p.M && n < p.N)
-            *reinterpret_cast<half4*>(p.D + (size_t)m * p.ldd + n) = o;
-        }
-      }
-    }
+    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
 
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
     cusync_dim3 done = {m0, n0, t.z};
-    if (stage.isProducer()) stage.post(done);
+    if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();
   }
 }

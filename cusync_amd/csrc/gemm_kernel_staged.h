@@ -37,7 +37,7 @@ struct TileCfg {
 template<class C, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  __shared__ uint32_t sTicket;
+  __shared__ uint32_t sTicket, sLast;
   half_t* const sA = reinterpret_cast<half_t*>(smem);
   half_t* const sB = sA + 2 * C::A_HALFS;
 
@@ -66,7 +66,6 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   if (tid == 0) stage.announceStart(p.launched);
 
   const uint32_t numTiles = stage.numTiles();
-  const uint32_t nk = (p.K + C::BK - 1) / C::BK;
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
   // Policies that synchronise once per row of tiles (RowSync, ConsecutiveSync) are
@@ -83,6 +82,9 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     const cusync_dim3 t = stage.ticketToTile(ticket);      // x = column tile, y = row tile
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
+    // K range of this slice, in chunks of BK counted from kBegin
+    const uint32_t kBegin = t.z * p.kPerSlice, kEnd = min(p.K, kBegin + p.kPerSlice);
+    const uint32_t nk = (kEnd - kBegin + C::BK - 1) / C::BK;
 
     floatx16 acc[C::TM][C::TN];
 #pragma unroll
@@ -107,8 +109,8 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     // The semaphore of the next column tile is polled one iteration early (the
     // load returns while MFMAs run), so in steady state no wave ever stalls on a
     // poll; only a tile that is really not there yet makes the wave spin.
-    uint32_t nextColTile = 0;        // producer column tiles below this one have been waited for
-    uint32_t nextColTileUp = swiglu ? p.K / tnq : 0;
+    uint32_t nextColTile = kBegin / tnq;   // producer column tiles below this one have been waited for (or are not needed)
+    uint32_t nextColTileUp = swiglu ? (p.K + kBegin) / tnq : 0;
     (void)nextColTileUp;
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
     uint32_t polledTile = 0xffffffffu, polledValue = 0;
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     };
     auto waitChunk = [&](uint32_t k0) {
       if (!chunkSync) return;
-      const uint32_t kLast = min(k0 + (uint32_t)C::BK, p.K) - 1;
+      const uint32_t kLast = min(k0 + (uint32_t)C::BK, kEnd) - 1;
       for (; nextColTile <= kLast / tnq; nextColTile++) waitColTile(nextColTile);
       if constexpr (swiglu) {
         // The up half lies K columns to the right.  StridedSync folds it onto the
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
       }
     };
     auto earlyPoll = [&](uint32_t k0) {      // k0: first column of a chunk whose loads come one iteration later
-      if (!oneRowBlock || k0 >= p.K) return;
+      if (!oneRowBlock || k0 >= kEnd) return;
       const uint32_t ct = k0 / tnq;
       if (ct < nextColTile || ct == polledTile) return;
       cusync_dim3 w = {m0, ct * tnq, 0};
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
 
     auto issue = [&](auto P, uint32_t kt) {
       constexpr int S = decltype(P)::value;
-      const uint32_t k0 = kt * C::BK;
+      const uint32_t k0 = kBegin + kt * C::BK;
       // weights first: they need no wait
 #pragma unroll
       for (int i = 0; i < C::CB; i++) {
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     };
     auto step = [&](auto P, uint32_t kt) {
       if (kt + 2 < nk) issue(P, kt + 2);
-      earlyPoll((kt + 3) * C::BK);
+      earlyPoll(kBegin + (kt + 3) * C::BK);
       __builtin_amdgcn_sched_barrier(0);
       computeAndStash(P);
       __builtin_amdgcn_sched_barrier(0);
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
 
     issue(Parity<0>{}, 0);
     if (nk > 1) issue(Parity<1>{}, 1);
-    earlyPoll(2 * C::BK);
+    earlyPoll(kBegin + 2 * C::BK);
     stash(Parity<0>{});
     __syncthreads();
 
@@ -247,27 +249,9 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
       if (kt + 1 < nk) step(Parity<1>{}, kt + 1);
     }
 
-    // Epilogue.  acc[i][j][r] of lane l is output row  m = .. + (l & 31)  and
-    // column  n = .. + 8*(r/4) + 4*(l/32) + r%4.
-#pragma unroll
-    for (int i = 0; i < C::TM; i++) {
-      const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
-#pragma unroll
-      for (int j = 0; j < C::TN; j++) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
-          half4 o;
-#pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(acc[i][j][g * 4 + e], p.epilogue);
-          if (m < p.M && n < p.N)
-            *reinterpret_cast<half4*>(p.D + (size_t)m * p.ldd + n) = o;
-        }
-      }
-    }
-
+    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
     cusync_dim3 done = {m0, n0, t.z};
-    stage.post(done);    // barrier inside when the stage is a producer
+    if (completed) stage.post(done);    // barrier inside when the stage is a producer (the decision is workgroup-uniform)
   }
 }
 

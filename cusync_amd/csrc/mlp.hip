@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <string.h>
+#include <algorithm>
 #include <string>
 
 #include "../../include/cusync_amd.h"
@@ -18,6 +19,9 @@ struct cusync_mlp {
   const void* w1;
   const void* w2;
   int tile1, tile2;
+  int split1, split2;
+  void* ws1;
+  void* ws2;
   uint32_t n1, k1, n2, k2;          // GEMM1 is [batch,k1]x[k1,n1], GEMM2 is [batch,k2]x[k2,n2]
   uint32_t ldh;                      // row pitch of the intermediate
   int epilogue1, aMode2;
@@ -30,9 +34,8 @@ namespace {
 
 using cusync::rt::setError;
 
-// Built-in choice of tile shapes per batch size for 256 CUs.  From 256 rows up
-// the direct-to-LDS 128x256 tile (two workgroups per CU) is the fastest one
-// measured; below that the M extent follows the batch.  A SwiGLU consumer has
+// Built-in choice of tile shapes per batch size for 256 CUs.  Above 128 rows the
+// direct-to-LDS tiles are used; below that the M extent follows the batch.  A SwiGLU consumer has
 // to use a register-staged tile, and StridedSync needs the gate|up split on a
 // tile boundary (2752 = 43 * 64).
 void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* t2) {
@@ -41,12 +44,27 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   else if (c.batch <= 64) small = CUSYNC_TILE_64x128x64;
   else small = CUSYNC_TILE_128x128x64;
   const bool big = c.batch > 128;
-  int a = big ? CUSYNC_TILE_128x256x32 : small;
-  int b = big ? (swiglu ? CUSYNC_TILE_256x128x64 : CUSYNC_TILE_128x256x32) : small;
+  // measured on the GPT-3 shard: 128x128 wins up to 512 rows (more tiles to spread), 128x256 from 2048 on
+  int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
+  int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
   *t2 = c.tile2 >= 0 ? c.tile2 : b;
+}
+
+// k-slices for a GEMM of `tiles` output tiles: double while the launch stays
+// within one and a half workgroups per CU and every slice keeps at least eight
+// K chunks.  Small batches are bound by streaming the weights, and without
+// slices a 32-row problem occupies 48 workgroups on 256 CUs; beyond about 384
+// workgroups the cost of adding the slices' partial sums outweighs the gain
+// (measured: M=16, N=6144, K=12288 takes 121 / 49 / 52 / 72 us with 1 / 4 / 8 / 16 slices).
+int pickSplit(int requested, uint32_t tiles, uint32_t K, uint32_t bk, int resident) {
+  if (requested > 0) return requested;
+  const uint32_t target = (uint32_t)std::min(resident, 384);
+  int s = 1;
+  while (tiles * (uint32_t)s * 2 <= target && K / ((uint32_t)s * 2) >= 8 * bk) s *= 2;
+  return s;
 }
 
 cusync_policy_desc noSync() {
@@ -61,7 +79,8 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
   cusync_gemm_args a;
   memset(&a, 0, sizeof a);
   a.M = m->cfg.batch;
-  a.split_k = 1;
+  a.split_k = which == 0 ? m->split1 : m->split2;
+  a.workspace = which == 0 ? m->ws1 : m->ws2;
   if (which == 0) {
     a.stage = m->prod;
     a.N = m->n1; a.K = m->k1;
@@ -115,8 +134,16 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
 
   cusync_policy_desc pol = noSync();
   int opts = 0;
-  const cusync_dim3 g1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, 1);
-  const cusync_dim3 g2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, 1);
+  uint32_t bk1 = 0, bk2 = 0;
+  cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk1);
+  cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, &bk2);
+  const cusync_dim3 flat1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, 1);
+  const cusync_dim3 flat2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, 1);
+  m->split1 = pickSplit(cfg->split_k1, flat1.x * flat1.y, m->k1, bk1, cusync_gemm_max_resident(m->tile1));
+  m->split2 = pickSplit(cfg->split_k2, flat2.x * flat2.y, m->k2, bk2, cusync_gemm_max_resident(m->tile2));
+  m->ws1 = m->ws2 = nullptr;
+  const cusync_dim3 g1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, m->split1);
+  const cusync_dim3 g2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, m->split2);
   switch (sync) {
     case CUSYNC_SYNC_STREAM:
       break;
@@ -161,6 +188,14 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     delete m;
     return nullptr;
   }
+  for (int which = 0; which < 2; which++) {
+    cusync_gemm_args a = gemmArgs(m, which, nullptr, nullptr, nullptr);
+    const size_t bytes = cusync_gemm_workspace_size(&a);
+    if (bytes == 0) continue;
+    void* ws = nullptr;
+    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { delete m; return nullptr; }
+    (which == 0 ? m->ws1 : m->ws2) = ws;
+  }
   if (CUSYNC_HIP(hipStreamCreateWithFlags(&m->sProd, hipStreamNonBlocking)) ||
       CUSYNC_HIP(hipStreamCreateWithFlags(&m->sCons, hipStreamNonBlocking)) ||
       CUSYNC_HIP(hipEventCreate(&m->eStart)) || CUSYNC_HIP(hipEventCreate(&m->eMid)) ||
@@ -177,6 +212,8 @@ void cusync_mlp_destroy(cusync_mlp* m) {
   (void)hipStreamSynchronize(m->sCons);
   cusync_stage_free(&m->prod);
   cusync_stage_free(&m->cons);
+  if (m->ws1) (void)hipFree(m->ws1);
+  if (m->ws2) (void)hipFree(m->ws2);
   (void)hipEventDestroy(m->eStart); (void)hipEventDestroy(m->eMid); (void)hipEventDestroy(m->eEnd);
   (void)hipStreamDestroy(m->sProd); (void)hipStreamDestroy(m->sCons);
   delete m;
@@ -231,6 +268,13 @@ cusync_error cusync_mlp_run(cusync_mlp* m, const void* x, void* h, void* y, int 
 const cusync_stage_desc* cusync_mlp_stage(const cusync_mlp* m, int which) {
   if (!m) return nullptr;
   return which == 0 ? &m->prod : &m->cons;
+}
+
+int cusync_mlp_splits(const cusync_mlp* m, int* split_k1, int* split_k2) {
+  if (!m) return 1;
+  if (split_k1) *split_k1 = m->split1;
+  if (split_k2) *split_k2 = m->split2;
+  return 0;
 }
 
 int cusync_mlp_tiles(const cusync_mlp* m, int* tile1, int* tile2) {

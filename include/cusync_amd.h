@@ -196,8 +196,8 @@ typedef struct cusync_gemm_args {
   int32_t epilogue;            /* CUSYNC_EPILOGUE_* */
   int32_t a_mode;              /* CUSYNC_A_* */
   int32_t tile;                /* CUSYNC_TILE_* */
-  int32_t split_k;             /* k-slices; > 1 accumulates through `workspace` */
-  void *workspace;             /* split_k > 1: cusync_gemm_workspace_size bytes, zeroed once */
+  int32_t split_k;             /* k-slices (grid z); > 1 adds the slices' fp32 partial sums through `workspace` */
+  void *workspace;             /* split_k > 1: cusync_gemm_workspace_size bytes, zeroed once by the caller */
   int32_t max_workgroups;      /* 0 = as many as stay resident; else cap on launched workgroups */
 } cusync_gemm_args;
 
@@ -236,6 +236,8 @@ typedef struct cusync_mlp_config {
   int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = the reference's defaults for `sync` */
   int32_t activation;          /* GPT-3: 1 = GeLU fused in GEMM1, 0 = none.  LLaMA: 1 = silu(g)*u fused
                                   in GEMM2's A loader, 0 = GEMM2 reads the gate half as is (TB/mlp.cu:785-792) */
+  int32_t split_k1, split_k2;  /* k-slices per GEMM (--split-k1/--split-k2, TB/mlp.cu:880-931); 0 = pick so that
+                                  the launch fills the device */
 } cusync_mlp_config;
 
 typedef struct cusync_mlp cusync_mlp;   /* opaque */
@@ -257,6 +259,7 @@ cusync_error cusync_mlp_run_split(cusync_mlp *mlp, const void *x, void *h, void 
 /* Device state of the two stages for tests (see cusync_stage_read_state). */
 const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer, 1 consumer */);
 int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
+int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 
 #ifdef __cplusplus
 }

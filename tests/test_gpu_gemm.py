@@ -15,11 +15,11 @@ pytestmark = pytest.mark.gpu
 ALL_TILES = list(range(api.TILE.COUNT))
 
 
-def plain_stage(tile, M, N):
-    return api.Stage(api.gemm_grid(tile, M, N), (1, 1, 1), api.no_sync(), api.no_sync())
+def plain_stage(tile, M, N, split_k=1):
+    return api.Stage(api.gemm_grid(tile, M, N, split_k), (1, 1, 1), api.no_sync(), api.no_sync())
 
 
-def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups=0):
+def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups=0, split_k=1, launches=1):
     import torch
     L = _lib.load()
     M = a.shape[0]
@@ -28,11 +28,20 @@ def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups
     da, db = to_dev(a), to_dev(b)
     dd = empty_dev((M, N), fill=float("nan"))
     torch.cuda.synchronize()
-    st = plain_stage(tile, M, N)
-    rc = api.gemm(st, M, N, K, da.data_ptr(), a.shape[1], db.data_ptr(), N, dd.data_ptr(), N, tile,
-                  epilogue=epilogue, a_mode=a_mode, max_workgroups=max_workgroups)
-    assert rc == api.ERR.SUCCESS, api.last_error()
-    assert L.cusync_rt_device_sync() == 0, api.last_error()
+    st = plain_stage(tile, M, N, split_k)
+    args = api.gemm_args(st, M, N, K, da.data_ptr(), a.shape[1], db.data_ptr(), N, dd.data_ptr(), N, tile,
+                         epilogue=epilogue, a_mode=a_mode, max_workgroups=max_workgroups, split_k=split_k)
+    ws = None
+    if split_k > 1:
+        ws = torch.zeros(L.cusync_gemm_workspace_size(C.byref(args)), dtype=torch.uint8, device="cuda")   # zeroed once
+        torch.cuda.synchronize()
+        args.workspace = ws.data_ptr()
+    for _ in range(launches):          # a second launch checks that the arrival counters re-armed themselves
+        dd.fill_(float("nan"))
+        torch.cuda.synchronize()
+        rc = L.cusync_gemm_run(C.byref(args), None)
+        assert rc == api.ERR.SUCCESS, api.last_error()
+        assert L.cusync_rt_device_sync() == 0, api.last_error()
     state = st.read_state()
     assert state.tile_counter == 0       # dispenser re-armed
     st.destroy()
@@ -92,12 +101,40 @@ def test_gemm_persistent_launch_smaller_than_grid():
     assert_close(got, orc.gemm(a, b), "persistent")
 
 
+@pytest.mark.parametrize("tile", [api.TILE.T128x128x64, api.TILE.T32x128x64, api.TILE.T128x256x32, api.TILE.T256x256x32,
+                                  api.TILE.T128x128x32])
+@pytest.mark.parametrize("split", [2, 3, 8])
+def test_gemm_split_k(tile, split):
+    print("split-k tile", tile, "slices", split, flush=True)
+    rng = np.random.default_rng(tile * 10 + split)
+    M, N, K = 200, 392, 1024
+    a = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    b = rng.integers(-2, 3, (K, N)).astype(np.float16)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float16)
+    assert np.array_equal(run_gemm(a, b, tile, split_k=split, launches=2), want)
+    # random data, GeLU applied after the slices are added
+    a = uniform_f16((M, K), 21)
+    b = normal_f16((K, N), 22, std=0.05)
+    got = run_gemm(a, b, tile, split_k=split, epilogue=api.EPI.GELU)
+    assert_close(got, orc.gemm(a, b, orc.EPI_GELU), "split-k %d tile %d" % (split, tile))
+
+
+def test_gemm_split_k_is_deterministic():
+    a = uniform_f16((64, 4096), 23)
+    b = normal_f16((4096, 256), 24, std=0.05)
+    first = run_gemm(a, b, api.TILE.T64x128x64, split_k=16)
+    for _ in range(3):
+        assert np.array_equal(run_gemm(a, b, api.TILE.T64x128x64, split_k=16).view(np.uint16), first.view(np.uint16))
+
+
 def test_gemm_can_implement_rejects():
     L = _lib.load()
     st = plain_stage(api.TILE.T128x128x64, 64, 64)
     bad = api.gemm_args(st, 64, 64, 60, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # K % 8 != 0
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "multiples of 8" in api.last_error()
-    bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=2)
+    bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=2)   # more slices than K chunks
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "k-slices" in api.last_error()
+    bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=0)
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED
     bad = api.gemm_args(st, 300, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # grid mismatch
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "grid" in api.last_error()
@@ -111,7 +148,7 @@ def test_gemm_can_implement_rejects():
     prod.destroy()
 
 
-def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10):
+def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1)):
     """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`."""
     import torch
     L = _lib.load()
@@ -123,7 +160,7 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
     de = empty_dev((M, N), fill=float("nan"))
     torch.cuda.synchronize()
     tm, tn, _ = api.tile_shape(tile1)
-    g1, g2 = api.gemm_grid(tile1, M, N), api.gemm_grid(tile2, M, N)
+    g1, g2 = api.gemm_grid(tile1, M, N, split[0]), api.gemm_grid(tile2, M, N, split[1])
     if policy_kind == "tile":
         pol = api.tile_sync(api.ORDER.TRANSPOSE_XY, tm, tn)
         opol = orc.policy(orc.TILESYNC, orc.ORDER_TRANSPOSE_XY, tm, tn)
@@ -135,14 +172,18 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
     assert api.set_producer_consumer_pair(prod, cons) == api.ERR.SUCCESS
     s1, s2 = C.c_void_p(), C.c_void_p()
     assert L.cusync_rt_stream_create(C.byref(s1)) == 0 and L.cusync_rt_stream_create(C.byref(s2)) == 0
+    a1 = api.gemm_args(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1, split_k=split[0], max_workgroups=max_wg)
+    a2 = api.gemm_args(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2, split_k=split[1], max_workgroups=max_wg)
+    ws = [torch.zeros(max(16, L.cusync_gemm_workspace_size(C.byref(x))), dtype=torch.uint8, device="cuda") for x in (a1, a2)]
+    torch.cuda.synchronize()
     for _ in range(iters):
         dc.fill_(float("nan")); de.fill_(float("nan"))
         torch.cuda.synchronize()
-        assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1,
-                        stream=s1, max_workgroups=max_wg) == api.ERR.SUCCESS, api.last_error()
+        assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1, stream=s1,
+                        max_workgroups=max_wg, split_k=split[0], workspace=ws[0].data_ptr()) == api.ERR.SUCCESS, api.last_error()
         assert prod.invokeWaitKernel(s2) == api.ERR.SUCCESS
-        assert api.gemm(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2,
-                        stream=s2, max_workgroups=max_wg) == api.ERR.SUCCESS, api.last_error()
+        assert api.gemm(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2, stream=s2,
+                        max_workgroups=max_wg, split_k=split[1], workspace=ws[1].data_ptr()) == api.ERR.SUCCESS, api.last_error()
         assert L.cusync_rt_device_sync() == 0, api.last_error()
         prod.incrementIter(); cons.incrementIter()
     ps, cs = prod.read_state(), cons.read_state()
@@ -178,3 +219,16 @@ def test_chained_gemms_with_few_workgroups():
     assert_close(c, orc.gemm(a, b), "C")
     assert_close(e, orc.gemm(c, d), "E")
     assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3
+
+
+@pytest.mark.parametrize("policy_kind,opts", [("tile", api.OPT.NO_ATOMIC_ADD), ("row", 0)])
+def test_chained_gemms_with_split_k(policy_kind, opts):
+    # split-K on both sides: only the slice that completes a tile posts it, and a consumer slice waits
+    # for the producer tiles of its own K range only (CC/gemm/kernel/cusyncgemm.h:374-398)
+    a, b, d, c, e, ps, cs, want_sems = chained(256, 1024, 1024, api.TILE.T64x128x64, api.TILE.T128x128x32,
+                                               policy_kind, iters=2, opts=opts, split=(4, 2))
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0
+    assert np.array_equal(ps.sems, want_sems)      # entries of the k-slices beyond the first stay 0
+    assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.kernel_executed == 2

@@ -38,7 +38,7 @@ def run_mlp(model, batch, hidden, inner, sync, runs=2, activation=1, **kw):
     mlp = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr(), activation=activation, **kw)
     times = mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=runs)
     prod, cons = mlp.stage_state(0), mlp.stage_state(1)
-    tiles = mlp.tiles()
+    tiles = mlp.tiles() + mlp.splits()
     mlp.destroy()
     return x, w1, w2, to_host(dh), to_host(dy), prod, cons, tiles, times
 
@@ -111,8 +111,12 @@ def test_gpt3_without_activation_matches_reference_check_build():
 def test_llama_mlp(inner, batch):
     print("llama", inner, batch, flush=True)
     outs = {}
-    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.STRIDED):
-        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2)
+    # StridedSync constrains the tile width (gate|up split on a tile boundary); the other modes are run with
+    # the same tiles and k-slices so that all three execute the same kernels and must agree bit for bit
+    same = {}
+    for sync in (api.SYNC.STRIDED, api.SYNC.STREAM, api.SYNC.ROW):
+        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2, **same)
+        same = dict(tile1=tiles[0], tile2=tiles[1], split_k1=tiles[2], split_k2=tiles[3])
         outs[sync] = (h, y)
         assert cons.spin_timeouts == 0
         if sync != api.SYNC.STREAM:
