@@ -43,6 +43,12 @@ class GemmArgs(C.Structure):
                 ("workspace", vp), ("max_workgroups", i32)]
 
 
+class Conv2dArgs(C.Structure):
+    _fields_ = [("stage", StageDesc), ("N", u32), ("H", u32), ("W", u32), ("C", u32), ("K", u32), ("R", u32), ("S", u32),
+                ("pad", u32), ("stride", u32), ("x", vp), ("w", vp), ("y", vp),
+                ("epilogue", i32), ("tile", i32), ("max_workgroups", i32)]
+
+
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
                 ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
@@ -89,6 +95,11 @@ SIGNATURES = {
     "cusync_gemm_workspace_size": (sz, [C.POINTER(GemmArgs)]),
     "cusync_gemm_max_resident": (C.c_int, [C.c_int]),
     "cusync_gemm_run": (C.c_int, [C.POINTER(GemmArgs), vp]),
+    "cusync_conv2d_tile_shape": (C.c_int, [C.c_int, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
+    "cusync_conv2d_grid": (Dim3, [C.c_int, u32, u32, u32, u32, u32, u32, u32, u32]),
+    "cusync_conv2d_can_implement": (C.c_int, [C.POINTER(Conv2dArgs)]),
+    "cusync_conv2d_max_resident": (C.c_int, [C.c_int]),
+    "cusync_conv2d_run": (C.c_int, [C.POINTER(Conv2dArgs), vp]),
     "cusync_mlp_create": (vp, [C.POINTER(MlpConfig), vp, vp]),
     "cusync_mlp_destroy": (None, [vp]),
     "cusync_mlp_run": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double)]),

@@ -9,7 +9,7 @@ import ctypes as C
 from types import SimpleNamespace
 
 from . import _lib
-from ._lib import Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
+from ._lib import Conv2dArgs, Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
 
 ERR = SimpleNamespace(NOT_PRODUCER=0, NOT_CONSUMER=1, NOT_INITIALIZED=2,
                       INVALID_LINEAR_BLOCK_INDEX=3, DEVICE=4, SUCCESS=5)
@@ -19,6 +19,7 @@ POLICY = SimpleNamespace(NOSYNC=0, ROWSYNC=1, TILESYNC=2, STRIDEDSYNC=3, CONV2DT
 EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2)
 TILE = SimpleNamespace(T256x256x32=0, T256x128x64=1, T128x128x64=2, T64x128x64=3, T32x128x64=4,
                        T128x256x64=5, T256x64x64=6, T128x64x64=7, T256x128x32=8, T128x256x32=9, T128x128x32=10, COUNT=11)
+CONV_TILE = SimpleNamespace(T128x64x32=0, T128x128x32=1, T256x64x32=2, COUNT=3)
 SYNC = SimpleNamespace(STREAM=0, ROW=1, TILE=2, STRIDED=3)
 MODEL = SimpleNamespace(GPT3=0, LLAMA=1)
 
@@ -193,6 +194,33 @@ def gemm(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, stream=None, **kw):
     """Launch one sync-aware GEMM; pointers are raw device addresses."""
     a = gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, **kw)
     return _lib.load().cusync_gemm_run(C.byref(a), stream)
+
+
+# ---- convolution -------------------------------------------------------------------
+
+def conv2d_tile_shape(tile):
+    m, n, k = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    if _lib.load().cusync_conv2d_tile_shape(tile, C.byref(m), C.byref(n), C.byref(k)):
+        raise ValueError("unknown conv tile id %r" % (tile,))
+    return m.value, n.value, k.value
+
+
+def conv2d_grid(tile, N, H, W, K, R=3, S=3, pad=1, stride=1):
+    return _lib.load().cusync_conv2d_grid(tile, N, H, W, K, R, S, pad, stride).tup()
+
+
+def conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, R=3, S=3, pad=1, stride=1, epilogue=EPI.NONE, max_workgroups=0):
+    a = Conv2dArgs()
+    a.stage = stage.desc
+    a.N, a.H, a.W, a.C, a.K, a.R, a.S, a.pad, a.stride = N, H, W, Cc, K, R, S, pad, stride
+    a.x, a.w, a.y = x, w, y
+    a.epilogue, a.tile, a.max_workgroups = epilogue, tile, max_workgroups
+    return a
+
+
+def conv2d(stage, N, H, W, Cc, K, x, w, y, tile, stream=None, **kw):
+    a = conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, **kw)
+    return _lib.load().cusync_conv2d_run(C.byref(a), stream)
 
 
 # ---- MLP chain -------------------------------------------------------------------

@@ -39,7 +39,11 @@ struct GemmParams {
   float* partials;         // [splitK][mPad][N] fp32 partial sums
   uint32_t* arrivals;      // [m-tiles * n-tiles] slices finished per output tile; 0 between launches
   uint32_t mPad;           // m-tiles * BM
+  // implicit-GEMM convolution (A is gathered from an NHWC tensor): M = n*P*Q, K = R*S*C, k = (r*S + s)*C + c
+  uint32_t cvN, cvH, cvW, cvC, cvP, cvQ, cvR, cvS, cvPad, cvStride;
 };
+
+enum { kAPlain = 0, kAConv = 1 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

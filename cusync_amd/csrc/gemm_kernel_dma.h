@@ -29,16 +29,18 @@
 namespace cusync {
 namespace gemm {
 
-template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1>
+template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false>
 struct DmaCfg {
+  static constexpr bool BT = BT_;                          // B given as [N][K] (k contiguous), e.g. KRSC filters
   static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // register budget: 512 / this per lane
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int KS = BK / 16;                        // MFMA k-steps per chunk
-  static constexpr int A_ROW_BYTES = BK * 2, B_ROW_BYTES = BN * 2;
+  static constexpr int A_ROW_BYTES = BK * 2, B_ROW_BYTES = BT ? BK * 2 : BN * 2;
+  static constexpr int B_ROWS = BT ? BN : BK;
   static constexpr int A_CPR = A_ROW_BYTES / 16, B_CPR = B_ROW_BYTES / 16;   // 16-byte chunks per row
-  static constexpr int A_STAGE = BM * A_ROW_BYTES, B_STAGE = BK * B_ROW_BYTES;
+  static constexpr int A_STAGE = BM * A_ROW_BYTES, B_STAGE = B_ROWS * B_ROW_BYTES;
   static constexpr int A_LOADS = A_STAGE / 1024 / 4, B_LOADS = B_STAGE / 1024 / 4;   // per wave per chunk
   static constexpr int LOADS = A_LOADS + B_LOADS;
   static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES, B_ROWS_PER_LOAD = 1024 / B_ROW_BYTES;
@@ -46,7 +48,7 @@ struct DmaCfg {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile is made of 32x32 MFMA tiles");
   static_assert(A_CPR == 4 || A_CPR == 8, "BK is 32 or 64");
-  static_assert(B_CPR % 8 == 0, "a B row covers whole 128-byte bank sweeps");
+  static_assert(BT || B_CPR % 8 == 0, "a B row covers whole 128-byte bank sweeps");
   static_assert(A_STAGE % 4096 == 0 && B_STAGE % 4096 == 0, "whole 1 KiB loads per wave");
   static_assert(LDS_BYTES * WAVES_PER_SIMD <= 160 * 1024, "fits the LDS of one CU");
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
@@ -73,8 +75,9 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
   return r;
 }
 
-template<class C>
+template<class C, int AMODE = kAPlain>
 __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
+  constexpr bool conv = AMODE == kAConv;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   __shared__ uint32_t sTicket, sLast;
 
@@ -84,8 +87,8 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   const int wm = wave / C::WN, wn = wave % C::WN;
   const cusync::DynStage& stage = p.stage;
 
-  const uint4v rA = rawRsrc(p.A, p.M * p.lda * 2);
-  const uint4v rB = rawRsrc(p.B, p.K * p.ldb * 2);
+  const uint4v rA = rawRsrc(p.A, conv ? p.cvN * p.cvH * p.cvW * p.cvC * 2 : p.M * p.lda * 2);
+  const uint4v rB = rawRsrc(p.B, (C::BT ? p.N : p.K) * p.ldb * 2);
   const uint32_t ldsBase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
   // ---- direct-load side: which global chunk this lane fetches ---------------
@@ -94,10 +97,12 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + lane / C::A_CPR;
   const uint32_t aLoadChunk = (lane % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
   // B: load q fills rows (wave*B_LOADS + q)*B_ROWS_PER_LOAD + lane/B_CPR, slot lane%B_CPR.
+  // With B given k-contiguous ([N][K]) its stage is laid out and swizzled exactly like A's.
   const uint32_t bLoadRow = wave * C::B_LOADS * C::B_ROWS_PER_LOAD + lane / C::B_CPR;
-  const uint32_t bLoadChunk = (lane % C::B_CPR) ^ (4 * (bLoadRow & 1));
+  const uint32_t bLoadChunk = C::BT ? (lane % C::B_CPR) ^ ((bLoadRow / A_SWZ_DIV) & (C::B_CPR - 1))
+                                    : (lane % C::B_CPR) ^ (4 * (bLoadRow & 1));
   static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
-  static_assert(C::B_ROWS_PER_LOAD % 2 == 0, "row parity repeats per load");
+  static_assert(C::B_ROWS_PER_LOAD % (C::BT ? A_SWZ_DIV * C::A_CPR : 2) == 0, "swizzle repeats per load");
 
   // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
   // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
@@ -116,6 +121,15 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   const uint32_t bColOff = (wn * (C::WTN / 8) + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 + (lane & 1) * 8;
   const uint32_t bFragEven = bRowOff + bColOff + 64 * bFlip;  // MFMA tiles j = 0, 2, ...: slot group j ^ flip
   const uint32_t bFragOdd = bRowOff + bColOff - 64 * bFlip;   // MFMA tiles j = 1, 3, ...
+  // k-contiguous B: same addressing as the A fragment, rows are output columns.
+  uint32_t bFragT[C::KS];
+  {
+    const uint32_t row = wn * C::WTN + (lane & 31);
+    const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
+#pragma unroll
+    for (int kk = 0; kk < C::KS; kk++)
+      bFragT[kk] = row * C::A_ROW_BYTES + (((2 * kk + (lane >> 5)) ^ swz) * 16);
+  }
 
   if (tid == 0) stage.announceStart(p.launched);
 
@@ -148,9 +162,24 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     // Per-tile byte offsets of this lane's loads at k0 = 0.
     const uint32_t aVoff0 = ((m0 + aLoadRow) * p.lda + aLoadChunk * 8) * 2;
     const uint32_t aVstep = C::A_ROWS_PER_LOAD * p.lda * 2;
-    const bool bInRange = n0 + bLoadChunk * 8 < p.N;
-    const uint32_t bVoff0 = (bLoadRow * p.ldb + n0 + bLoadChunk * 8) * 2;
+    const bool bInRange = C::BT ? true : n0 + bLoadChunk * 8 < p.N;
+    const uint32_t bVoff0 = C::BT ? ((n0 + bLoadRow) * p.ldb + bLoadChunk * 8) * 2     // rows past N fall outside the buffer
+                                  : (bLoadRow * p.ldb + n0 + bLoadChunk * 8) * 2;
     const uint32_t bVstep = C::B_ROWS_PER_LOAD * p.ldb * 2;
+
+    // Convolution: the pixel each of this lane's A rows stands for.
+    int32_t cvIh0[C::A_LOADS], cvIw0[C::A_LOADS];
+    uint32_t cvBase[C::A_LOADS];
+    if constexpr (conv) {
+#pragma unroll
+      for (int q = 0; q < C::A_LOADS; q++) {
+        const uint32_t m = m0 + aLoadRow + q * C::A_ROWS_PER_LOAD;
+        const uint32_t img = m / (p.cvP * p.cvQ), rem = m % (p.cvP * p.cvQ);
+        cvIh0[q] = (int32_t)((rem / p.cvQ) * p.cvStride) - (int32_t)p.cvPad;
+        cvIw0[q] = (int32_t)((rem % p.cvQ) * p.cvStride) - (int32_t)p.cvPad;
+        cvBase[q] = m < p.M ? img * p.cvH * p.cvW * p.cvC : kOutOfRange / 2;
+      }
+    }
 
     // ---- consumer side (same protocol as the staged kernel) ------------------
     uint32_t nextColTile = kBegin / tnq;
@@ -162,8 +191,39 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
         stage.waitWave(w);
       }
     };
+    // Convolution fed by another convolution: the rows of the producer's output
+    // this tile reads are its own pixels plus the filter's halo, and a K chunk
+    // (r, s, c0..) lies in the producer's column tile c0 / tileN.  Each column
+    // tile is waited for once, for the whole halo range.
+    uint32_t cvSeen = 0;
+    auto cvRowRange = [&](uint32_t& lo, uint32_t& hi) {
+      auto pixelRow = [&](uint32_t m) {
+        const uint32_t img = m / (p.cvP * p.cvQ), rem = m % (p.cvP * p.cvQ);
+        return (img * p.cvH + (rem / p.cvQ) * p.cvStride) * p.cvW + (rem % p.cvQ) * p.cvStride;
+      };
+      const uint32_t before = p.cvPad * p.cvW + p.cvPad, after = (p.cvR - 1 - p.cvPad) * p.cvW + (p.cvS - 1 - p.cvPad);
+      const uint32_t first = pixelRow(m0), last = pixelRow(mEnd - 1) + after;
+      lo = first > before ? first - before : 0;
+      hi = min(last, p.cvN * p.cvH * p.cvW - 1);
+    };
+    auto cvWaitRows = [&](uint32_t policyCol, uint32_t z) {
+      uint32_t lo, hi;
+      cvRowRange(lo, hi);
+      for (uint32_t r = lo; r <= hi; r = (r / tmq + 1) * tmq) {
+        cusync_dim3 w = {r, policyCol, z};
+        stage.waitWave(w);
+      }
+    };
     auto waitChunk = [&](uint32_t k0) {
       if (!chunkSync) return;
+      if constexpr (conv) {
+        const uint32_t ct = (k0 % p.cvC) / tnq;
+        if (cvSeen & (1u << ct)) return;
+        cvSeen |= 1u << ct;
+        // Conv2DTileSync divides the K tile index by R*S to get the channel tile
+        cvWaitRows(stage.d.in.kind == CUSYNC_POLICY_CONV2DTILESYNC ? ct * p.cvR * p.cvS * tnq : ct * tnq, 0);
+        return;
+      }
       const uint32_t kLast = min(k0 + (uint32_t)C::BK, kEnd) - 1;
       for (; nextColTile <= kLast / tnq; nextColTile++) {
         if (oneRowBlock && nextColTile == polledTile && cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) continue;
@@ -171,7 +231,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       }
     };
     auto earlyPoll = [&](uint32_t k0) {
-      if (!oneRowBlock || k0 >= kEnd) return;
+      if (conv || !oneRowBlock || k0 >= kEnd) return;
       const uint32_t ct = k0 / tnq;
       if (ct < nextColTile || ct == polledTile) return;
       polledTile = ct;
@@ -189,12 +249,22 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       const uint32_t k0 = kBegin + kt * C::BK;
       if constexpr (Q < C::B_LOADS) {
         const uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
-        loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), (bInRange && k0 < kEnd) ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange);
+        uint32_t off;
+        if constexpr (C::BT) off = k0 + bLoadChunk * 8 < kEnd ? bVoff0 + k0 * 2 + Q * bVstep : kOutOfRange;
+        else off = (bInRange && k0 < kEnd) ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange;
+        loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), off);
       } else {
         constexpr int QA = Q - C::B_LOADS;
         const bool aInRange = k0 + aLoadChunk * 8 < kEnd;   // never touch columns the slice has not waited for
         const uint32_t lds = ldsBase + S * C::A_STAGE + (wave * C::A_LOADS + QA) * 1024;
-        loadToLds(rA, __builtin_amdgcn_readfirstlane(lds), aInRange ? aVoff0 + k0 * 2 + QA * aVstep : kOutOfRange);
+        uint32_t off = aInRange ? aVoff0 + k0 * 2 + QA * aVstep : kOutOfRange;
+        if constexpr (conv) {
+          const uint32_t rs = k0 / p.cvC, c0 = k0 % p.cvC;
+          const int32_t ih = cvIh0[QA] + (int32_t)(rs / p.cvS), iw = cvIw0[QA] + (int32_t)(rs % p.cvS);
+          const bool inside = aInRange && cvBase[QA] != kOutOfRange / 2 && ih >= 0 && ih < (int32_t)p.cvH && iw >= 0 && iw < (int32_t)p.cvW;
+          off = inside ? (cvBase[QA] + ((uint32_t)ih * p.cvW + (uint32_t)iw) * p.cvC + c0 + aLoadChunk * 8) * 2 : kOutOfRange;
+        }
+        loadToLds(rA, __builtin_amdgcn_readfirstlane(lds), off);
       }
     };
     auto issueAll = [&](auto SP, uint32_t kt) {
@@ -219,6 +289,10 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
           fa[slot][F] = *reinterpret_cast<const half8*>(sa + aFrag[kk] + F * 32 * C::A_ROW_BYTES);
         } else {
           constexpr int J = F - C::TM;
+          if constexpr (C::BT) {
+            fb[slot][J] = *reinterpret_cast<const half8*>(smem + C::STAGES * C::A_STAGE + S * C::B_STAGE + bFragT[kk] + J * 32 * C::B_ROW_BYTES);
+            return;
+          }
           typedef short4v __attribute__((address_space(3))) * lds_ptr;
           const char* q = ((J & 1) ? sbO : sbE) + J * 64 + kk * 16 * C::B_ROW_BYTES;
           short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
@@ -250,7 +324,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
           for (int j = 0; j < C::TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
       }
-      schedPass<C::KS, C::TM * C::TN, C::TM + 2 * C::TN, 0>();
+      schedPass<C::KS, C::TM * C::TN, C::TM + (C::BT ? 1 : 2) * C::TN, 0>();
     };
 
     // Iteration kt on stage S = kt % STAGES.  Chunks kt+1 .. kt+STAGES-2 are the
@@ -271,7 +345,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     if (consumer) {
       cusync_dim3 w = {m0, 0, 1};
       if (stage.needsWait(w)) {
-        if (wave == 0) waitRows(0, 1);
+        if (wave == 0) { if constexpr (conv) cvWaitRows(0, 1); else waitRows(0, 1); }
         __syncthreads();
       }
     }

@@ -217,6 +217,44 @@ int cusync_gemm_max_resident(int tile);
 cusync_error cusync_gemm_run(const cusync_gemm_args *args, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Sync-aware NHWC forward convolution as an implicit GEMM (replaces           */
+/* cutlass::conv::device::CuSyncImplicitGemmConvolution,                       */
+/* CC/conv/device/cusyncimplicit_gemm_convolution.h:226-298, and its kernel    */
+/* CC/conv/kernel/implicit_cusyncgemm_convolution.h:287-477)                   */
+/* ------------------------------------------------------------------------- */
+
+enum {
+  CUSYNC_CONV_TILE_128x64x32 = 0,    /* M x K_out x K chunk */
+  CUSYNC_CONV_TILE_128x128x32 = 1,
+  CUSYNC_CONV_TILE_256x64x32 = 2,
+  CUSYNC_CONV_TILE_COUNT = 3
+};
+
+typedef struct cusync_conv2d_args {
+  cusync_stage_desc stage;     /* Arguments::custage; grid = cusync_conv2d_grid(...) */
+  uint32_t N, H, W, C;         /* input  x[N,H,W,C]  fp16 NHWC */
+  uint32_t K, R, S;            /* filter w[K,R,S,C]  fp16 KRSC, cross-correlation (CV/resnet.cu:678) */
+  uint32_t pad, stride;        /* same in both directions; output y[N,P,Q,K], P = (H+2*pad-R)/stride+1 */
+  const void *x;
+  const void *w;
+  void *y;
+  int32_t epilogue;            /* CUSYNC_EPILOGUE_* (the ResNet pair uses RELU after the first convolution) */
+  int32_t tile;                /* CUSYNC_CONV_TILE_* */
+  int32_t max_workgroups;      /* 0 = as many as stay resident */
+} cusync_conv2d_args;
+
+int cusync_conv2d_tile_shape(int tile, uint32_t *tileM, uint32_t *tileN, uint32_t *tileK);
+/* Logical grid (K_out tiles, N*P*Q tiles, 1): the implicit-GEMM form of get_tiled_shape
+ * (CC/gemm/threadblock/cusync_threadblock_swizzle.h:34-44). */
+cusync_dim3 cusync_conv2d_grid(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
+                               uint32_t pad, uint32_t stride);
+cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args *args);
+int cusync_conv2d_max_resident(int tile);
+/* operator()(stream) (cusyncimplicit_gemm_convolution.h:283-298).  A consumer stage waits, per producer
+ * channel tile, for every producer row block reached by the filter window of its rows. */
+cusync_error cusync_conv2d_run(const cusync_conv2d_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* MLP chain (replaces the extern "C" surface of TB/mlp-lib.cu:555-618 and    */
 /* the hot loops runBaselineGPT3 / runCuSyncGPT3 / runCuSyncLLaMA,            */
 /* TB/mlp.cu:411-491, 645-716, 718-862)                                       */
