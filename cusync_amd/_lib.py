@@ -49,6 +49,16 @@ class Conv2dArgs(C.Structure):
                 ("epilogue", i32), ("tile", i32), ("max_workgroups", i32)]
 
 
+class AttentionArgs(C.Structure):
+    _fields_ = [("stage", StageDesc), ("seq", u32), ("heads", u32), ("head_dim", u32), ("qkv", vp), ("ldqkv", u32),
+                ("out", vp), ("ldo", u32), ("scale", C.c_float), ("causal", i32), ("max_workgroups", i32)]
+
+
+class AttnLayerConfig(C.Structure):
+    _fields_ = [("seq", u32), ("hidden", u32), ("heads", u32), ("head_dim", u32), ("sync", i32),
+                ("tile1", i32), ("tile3", i32), ("opts", i32), ("causal", i32)]
+
+
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
                 ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
@@ -100,6 +110,16 @@ SIGNATURES = {
     "cusync_conv2d_can_implement": (C.c_int, [C.POINTER(Conv2dArgs)]),
     "cusync_conv2d_max_resident": (C.c_int, [C.c_int]),
     "cusync_conv2d_run": (C.c_int, [C.POINTER(Conv2dArgs), vp]),
+    "cusync_attention_tile_shape": (C.c_int, [C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
+    "cusync_attention_grid": (Dim3, [u32, u32]),
+    "cusync_attention_can_implement": (C.c_int, [C.POINTER(AttentionArgs)]),
+    "cusync_attention_max_resident": (C.c_int, []),
+    "cusync_attention_run": (C.c_int, [C.POINTER(AttentionArgs), vp]),
+    "cusync_attn_layer_create": (vp, [C.POINTER(AttnLayerConfig), vp, vp]),
+    "cusync_attn_layer_destroy": (None, [vp]),
+    "cusync_attn_layer_run": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "cusync_attn_layer_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
+    "cusync_attn_layer_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cusync_mlp_create": (vp, [C.POINTER(MlpConfig), vp, vp]),
     "cusync_mlp_destroy": (None, [vp]),
     "cusync_mlp_run": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double)]),

@@ -9,7 +9,7 @@ import ctypes as C
 from types import SimpleNamespace
 
 from . import _lib
-from ._lib import Conv2dArgs, Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
+from ._lib import AttentionArgs, AttnLayerConfig, Conv2dArgs, Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
 
 ERR = SimpleNamespace(NOT_PRODUCER=0, NOT_CONSUMER=1, NOT_INITIALIZED=2,
                       INVALID_LINEAR_BLOCK_INDEX=3, DEVICE=4, SUCCESS=5)
@@ -221,6 +221,80 @@ def conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, R=3, S=3, pad=1, stride=1,
 def conv2d(stage, N, H, W, Cc, K, x, w, y, tile, stream=None, **kw):
     a = conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, **kw)
     return _lib.load().cusync_conv2d_run(C.byref(a), stream)
+
+
+# ---- attention -------------------------------------------------------------------
+
+def attention_tile_shape():
+    m, n, k = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    _lib.load().cusync_attention_tile_shape(C.byref(m), C.byref(n), C.byref(k))
+    return m.value, n.value, k.value
+
+
+def attention_grid(seq, heads):
+    return _lib.load().cusync_attention_grid(seq, heads).tup()
+
+
+def attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, head_dim=128, scale=0.0, causal=True, max_workgroups=0):
+    a = AttentionArgs()
+    a.stage = stage.desc
+    a.seq, a.heads, a.head_dim = seq, heads, head_dim
+    a.qkv, a.ldqkv, a.out, a.ldo = qkv, ldqkv, out, ldo
+    a.scale, a.causal, a.max_workgroups = scale, int(causal), max_workgroups
+    return a
+
+
+def attention(stage, seq, heads, qkv, ldqkv, out, ldo, stream=None, **kw):
+    a = attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, **kw)
+    return _lib.load().cusync_attention_run(C.byref(a), stream)
+
+
+def _read_stage(L, d):
+    import numpy as np
+    g = d.grid
+    n = g.x * g.y * g.z
+    sems = np.zeros(n, np.uint32)
+    order = np.zeros((n, 3), np.uint32)
+    tc, sc, ke, to = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    producer = d.out.kind != POLICY.NOSYNC
+    check(L.cusync_stage_read_state(C.byref(d), sems.ctypes.data_as(C.c_void_p) if producer else None,
+                                    order.ctypes.data_as(C.c_void_p), C.byref(tc), C.byref(sc),
+                                    C.byref(ke), C.byref(to)), "read_state")
+    return SimpleNamespace(desc=d, grid=g.tup(), sems=sems, tile_order=order, tile_counter=tc.value,
+                           start_counter=sc.value, kernel_executed=ke.value, spin_timeouts=to.value)
+
+
+class AttnLayer:
+    """Handle over cusync_attn_layer_*: X Wqkv -> fused attention -> O Wo, stream-ordered or as three
+    CuSync stages (the chain of src/ml-bench/transformer/attention.cu:702-830)."""
+
+    def __init__(self, seq, hidden, heads, sync, wqkv_ptr, wo_ptr, head_dim=128, tile1=-1, tile3=-1, opts=-1, causal=True):
+        self.L = _lib.load()
+        self.cfg = AttnLayerConfig(seq, hidden, heads, head_dim, sync, tile1, tile3, opts, int(causal))
+        self.h = self.L.cusync_attn_layer_create(C.byref(self.cfg), wqkv_ptr, wo_ptr)
+        if not self.h:
+            raise RuntimeError("cusync_attn_layer_create failed: " + last_error())
+
+    def run(self, x_ptr, qkv_ptr, o_ptr, y_ptr, runs=1, stages=False):
+        times = (C.c_double * runs)()
+        per_stage = (C.c_double * (3 * runs))()
+        check(self.L.cusync_attn_layer_run(self.h, x_ptr, qkv_ptr, o_ptr, y_ptr, runs, times, per_stage), "cusync_attn_layer_run")
+        if stages:
+            return list(times), [list(per_stage[3 * r:3 * r + 3]) for r in range(runs)]
+        return list(times)
+
+    def tiles(self):
+        a, b = C.c_int(0), C.c_int(0)
+        self.L.cusync_attn_layer_tiles(self.h, C.byref(a), C.byref(b))
+        return a.value, b.value
+
+    def stage_state(self, which):
+        return _read_stage(self.L, self.L.cusync_attn_layer_stage(self.h, which).contents)
+
+    def destroy(self):
+        if self.h:
+            self.L.cusync_attn_layer_destroy(self.h)
+            self.h = None
 
 
 # ---- MLP chain -------------------------------------------------------------------

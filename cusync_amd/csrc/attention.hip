@@ -1,0 +1,289 @@
+// Fused attention stage and the self-attention chain
+//   QKV = X Wqkv  ->  O = softmax(mask(Q K^T / sqrt(128))) V per head  ->  Y = O Wo
+// run stream-ordered or as three CuSync stages on three streams.  Stands in for
+// the reference's attention driver (src/ml-bench/transformer/attention.cu:84-110
+// stage wiring, :560-700 baseline, :702-830 overlapped run), which builds the
+// same dependency chain out of four CUTLASS GEMMs; here the two inner products
+// are one fused kernel that is consumer and producer at once (the role of
+// SCuStage / OCuStage, attention.cu:101-104).
+#include <hip/hip_runtime.h>
+
+#include <math.h>
+#include <string.h>
+#include <algorithm>
+#include <mutex>
+
+#include "../../include/cusync_amd.h"
+#include "rt_internal.h"
+#include "attention_kernel.h"
+
+namespace {
+
+using cusync::rt::setError;
+using namespace cusync::attn;
+
+std::mutex g_attnMutex;
+int g_attnResidentPerCU = -1;
+
+int residentAttention() {
+  std::lock_guard<std::mutex> lock(g_attnMutex);
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
+  if (g_attnResidentPerCU < 0) {
+    if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attentionKernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes))) return 0;
+    int n = 0;
+    if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attentionKernel, kThreads, kLdsBytes))) return 0;
+    g_attnResidentPerCU = n;
+  }
+  return g_attnResidentPerCU * prop.multiProcessorCount;
+}
+
+cusync_policy_desc noSync() {
+  cusync_policy_desc p;
+  memset(&p, 0, sizeof p);
+  p.kind = CUSYNC_POLICY_NOSYNC;
+  p.tileM = p.tileN = 1; p.R = p.S = 1;
+  return p;
+}
+
+}  // namespace
+
+struct cusync_attn_layer {
+  cusync_attn_layer_config cfg;
+  const void* wqkv;
+  const void* wo;
+  uint32_t E;                      // heads * head_dim
+  int tile1, tile3;
+  cusync_stage_desc st[3];         // QKV projection, attention, output projection
+  hipStream_t stream[3];
+  hipEvent_t eStart, eMid1, eMid2, eEnd;
+};
+
+extern "C" {
+
+int cusync_attention_tile_shape(uint32_t* tileM, uint32_t* tileN, uint32_t* blockKV) {
+  if (tileM) *tileM = kBQ;
+  if (tileN) *tileN = kHD;
+  if (blockKV) *blockKV = kBKV;
+  return 0;
+}
+
+cusync_dim3 cusync_attention_grid(uint32_t seq, uint32_t heads) {
+  cusync_dim3 g = {heads, (seq + kBQ - 1) / kBQ, 1};
+  return g;
+}
+
+cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
+  if (!a) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (!a->seq || !a->heads) { setError("attention: empty problem"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->head_dim != (uint32_t)kHD) { setError("attention: head width must be 128"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  const uint32_t E = a->heads * kHD;
+  if (a->ldqkv < 3 * E || a->ldqkv % 8 || a->ldo < E || a->ldo % 4) { setError("attention: row pitch too small or misaligned"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if ((uint64_t)a->seq * a->ldqkv * 2 >= 0x80000000ull) { setError("attention: QKV larger than 2 GiB is not addressable by one buffer descriptor"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if ((uintptr_t)a->qkv % 16 || (uintptr_t)a->out % 8 || !a->qkv || !a->out) { setError("attention: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  const cusync_dim3 g = cusync_attention_grid(a->seq, a->heads);
+  const cusync_stage_desc& s = a->stage;
+  if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("attention: stage grid does not match cusync_attention_grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (!s.tileOrder || !s.tileCounter || !s.startCounter || !s.spinTimeouts || !s.xcdTickets) { setError("attention: stage not allocated"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (s.out.kind != CUSYNC_POLICY_NOSYNC && !s.tileStatusWrite) { setError("attention: producer stage without semaphores"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (s.in.kind != CUSYNC_POLICY_NOSYNC) {
+    if (!s.tileStatusRead) { setError("attention: consumer stage not paired with a producer"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (s.in.kind != CUSYNC_POLICY_ROWSYNC && s.in.kind != CUSYNC_POLICY_TILESYNC && s.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC) {
+      setError("attention: input policy must be RowSync, TileSync or ConsecutiveSync");
+      return CUSYNC_ERROR_NOT_INITIALIZED;
+    }
+    if (s.in.tileM == 0 || s.in.tileN == 0) { setError("attention: input policy with zero tile extent"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (s.in.kind == CUSYNC_POLICY_CONSECUTIVESYNC && (s.in.H / 8 != E || E % s.in.tileN)) {
+      setError("attention: ConsecutiveSync must group exactly the Q, K and V column tiles (H/8 == heads*128)");
+      return CUSYNC_ERROR_NOT_INITIALIZED;
+    }
+  }
+  if ((s.opts & CUSYNC_OPT_NO_ATOMIC_ADD) && s.out.kind != CUSYNC_POLICY_NOSYNC &&
+      cusync::dyn::waitValue(s.out) != cusync::dyn::postValue(s.out)) {
+    setError("attention: NoAtomicAdd needs a policy whose wait value equals its post value");
+    return CUSYNC_ERROR_NOT_INITIALIZED;
+  }
+  return CUSYNC_SUCCESS;
+}
+
+int cusync_attention_max_resident(void) { return residentAttention(); }
+
+cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) {
+  cusync_error e = cusync_attention_can_implement(a);
+  if (e != CUSYNC_SUCCESS) return e;
+  const int resident = residentAttention();
+  if (resident <= 0) { setError("attention: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
+  const cusync_stage_desc& s = a->stage;
+  uint32_t launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)resident);
+  if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
+
+  AttnParams p = {};
+  p.stage.d = s;
+  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->qkv % 128 == 0 && (a->ldqkv * 2) % 128 == 0 &&
+                        (s.in.kind != CUSYNC_POLICY_TILESYNC || (s.in.tileN * 2) % 128 == 0);
+  p.S = a->seq; p.heads = a->heads;
+  p.qkv = (const half_t*)a->qkv; p.ldq = a->ldqkv;
+  p.out = (half_t*)a->out; p.ldo = a->ldo;
+  const float scale = a->scale > 0.0f ? a->scale : 1.0f / sqrtf((float)kHD);
+  p.scaleLog2 = scale * 1.4426950408889634f;
+  p.causal = a->causal ? 1 : 0;
+  p.launched = launched;
+  hipLaunchKernelGGL(attentionKernel, dim3(launched), dim3(kThreads), kLdsBytes, (hipStream_t)stream, p);
+  if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  return CUSYNC_SUCCESS;
+}
+
+/* ---- the chain ---------------------------------------------------------------- */
+
+cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg, const void* wqkv, const void* wo) {
+  if (!cfg || !wqkv || !wo) { setError("attn layer: null argument"); return nullptr; }
+  if (!cfg->seq || !cfg->hidden || !cfg->heads) { setError("attn layer: empty shape"); return nullptr; }
+  if (cfg->head_dim != (uint32_t)kHD) { setError("attn layer: head width must be 128"); return nullptr; }
+  cusync_attn_layer* L = new cusync_attn_layer();
+  L->cfg = *cfg;
+  L->wqkv = wqkv; L->wo = wo;
+  L->E = cfg->heads * kHD;
+  // Same per-row-count choice as the MLP chain: 128x128 tiles while the grid would otherwise not
+  // cover the device, 128x256 from 2048 rows on.
+  const int small = cfg->seq <= 32 ? CUSYNC_TILE_32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
+  const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
+  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : dflt;
+  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : dflt;
+  uint32_t tm1 = 0, tn1 = 0;
+  if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
+    setError("attn layer: unknown tile id");
+    delete L;
+    return nullptr;
+  }
+  const cusync_dim3 g1 = cusync_gemm_grid(L->tile1, cfg->seq, 3 * L->E, 1);
+  const cusync_dim3 g2 = cusync_attention_grid(cfg->seq, cfg->heads);
+  const cusync_dim3 g3 = cusync_gemm_grid(L->tile3, cfg->seq, cfg->hidden, 1);
+
+  cusync_policy_desc sync1 = noSync(), sync2 = noSync();
+  int opts = 0;
+  switch (cfg->sync) {
+    case CUSYNC_SYNC_STREAM:
+      break;
+    case CUSYNC_SYNC_ROW:       // RowSync<kM> on both edges, attention.cu:84-90
+      sync1.kind = CUSYNC_POLICY_ROWSYNC; sync1.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      sync1.tileM = tm1; sync1.tileN = 1; sync1.waitValue = g1.x; sync1.postValue = 1;
+      sync2 = sync1;
+      sync2.tileM = kBQ; sync2.waitValue = g2.x;
+      break;
+    case CUSYNC_SYNC_TILE:      // TileSync on both edges, attention.cu:91-97
+      sync1.kind = CUSYNC_POLICY_TILESYNC; sync1.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      sync1.tileM = tm1; sync1.tileN = tn1; sync1.waitValue = 1; sync1.postValue = 1;
+      sync2 = sync1;
+      sync2.tileM = kBQ; sync2.tileN = kHD;
+      opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
+      break;
+    case CUSYNC_SYNC_STRIDED:   // ConsecutiveSync into the attention, RowSync out of it, attention.cu:98-110
+      if (L->E % tn1) { setError("attn layer: ConsecutiveSync needs heads*128 % tileN == 0"); delete L; return nullptr; }
+      sync1.kind = CUSYNC_POLICY_CONSECUTIVESYNC; sync1.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      sync1.tileM = tm1; sync1.tileN = tn1; sync1.H = 8 * L->E;
+      sync1.waitValue = L->E / tn1; sync1.postValue = 1;
+      sync2.kind = CUSYNC_POLICY_ROWSYNC; sync2.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      sync2.tileM = kBQ; sync2.tileN = 1; sync2.waitValue = g2.x; sync2.postValue = 1;
+      break;
+    default:
+      setError("attn layer: unknown sync mode");
+      delete L;
+      return nullptr;
+  }
+  if (cfg->opts >= 0) opts |= cfg->opts;
+
+  const cusync_dim3 grids[3] = {g1, g2, g3};
+  const cusync_policy_desc ins[3] = {noSync(), sync1, sync2}, outs[3] = {sync1, sync2, noSync()};
+  for (int i = 0; i < 3; i++) {
+    memset(&L->st[i], 0, sizeof L->st[i]);
+    L->st[i].grid = grids[i]; L->st[i].tileSize = {1, 1, 1}; L->st[i].iter = 1; L->st[i].opts = opts;
+    L->st[i].in = ins[i]; L->st[i].out = outs[i];
+    if (cusync_stage_create(&L->st[i], CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) { delete L; return nullptr; }
+  }
+  if (cfg->sync != CUSYNC_SYNC_STREAM &&
+      (cusync_set_producer_consumer_pair(&L->st[0], &L->st[1]) != CUSYNC_SUCCESS ||
+       cusync_set_producer_consumer_pair(&L->st[1], &L->st[2]) != CUSYNC_SUCCESS)) {
+    setError("attn layer: pairing the stages failed");
+    delete L;
+    return nullptr;
+  }
+  for (int i = 0; i < 3; i++)
+    if (CUSYNC_HIP(hipStreamCreateWithFlags(&L->stream[i], hipStreamNonBlocking))) { delete L; return nullptr; }
+  if (CUSYNC_HIP(hipEventCreate(&L->eStart)) || CUSYNC_HIP(hipEventCreate(&L->eMid1)) ||
+      CUSYNC_HIP(hipEventCreate(&L->eMid2)) || CUSYNC_HIP(hipEventCreate(&L->eEnd))) { delete L; return nullptr; }
+  return L;
+}
+
+void cusync_attn_layer_destroy(cusync_attn_layer* L) {
+  if (!L) return;
+  for (int i = 0; i < 3; i++) (void)hipStreamSynchronize(L->stream[i]);
+  for (int i = 0; i < 3; i++) cusync_stage_free(&L->st[i]);
+  (void)hipEventDestroy(L->eStart); (void)hipEventDestroy(L->eMid1); (void)hipEventDestroy(L->eMid2); (void)hipEventDestroy(L->eEnd);
+  for (int i = 0; i < 3; i++) (void)hipStreamDestroy(L->stream[i]);
+  delete L;
+}
+
+cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qkv, void* o, void* y, int runs,
+                                   double* times_us, double* stage_us) {
+  if (!L || !x || !qkv || !o || !y) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const bool overlapped = L->cfg.sync != CUSYNC_SYNC_STREAM;
+  const uint32_t S = L->cfg.seq, E = L->E, H = L->cfg.hidden;
+  for (int r = 0; r < runs; r++) {
+    cusync_gemm_args a1, a3;
+    memset(&a1, 0, sizeof a1); memset(&a3, 0, sizeof a3);
+    a1.stage = L->st[0]; a1.M = S; a1.N = 3 * E; a1.K = H;
+    a1.A = x; a1.lda = H; a1.B = L->wqkv; a1.ldb = 3 * E; a1.D = qkv; a1.ldd = 3 * E;
+    a1.tile = L->tile1; a1.split_k = 1;
+    cusync_attention_args a2;
+    memset(&a2, 0, sizeof a2);
+    a2.stage = L->st[1]; a2.seq = S; a2.heads = L->cfg.heads; a2.head_dim = kHD;
+    a2.qkv = qkv; a2.ldqkv = 3 * E; a2.out = o; a2.ldo = E; a2.scale = 0.0f; a2.causal = L->cfg.causal;
+    a3.stage = L->st[2]; a3.M = S; a3.N = H; a3.K = E;
+    a3.A = o; a3.lda = E; a3.B = L->wo; a3.ldb = H; a3.D = y; a3.ldd = H;
+    a3.tile = L->tile3; a3.split_k = 1;
+
+    hipStream_t s0 = L->stream[0], s1 = overlapped ? L->stream[1] : s0, s2 = overlapped ? L->stream[2] : s0;
+    cusync_error e;
+    if (CUSYNC_HIP(hipEventRecord(L->eStart, s0))) return CUSYNC_ERROR_DEVICE;
+    if ((e = cusync_gemm_run(&a1, s0)) != CUSYNC_SUCCESS) return e;
+    if (overlapped) { if ((e = cusync_invoke_wait_kernel(&L->st[0], s1)) != CUSYNC_SUCCESS) return e; }
+    else if (CUSYNC_HIP(hipEventRecord(L->eMid1, s0))) return CUSYNC_ERROR_DEVICE;
+    if ((e = cusync_attention_run(&a2, s1)) != CUSYNC_SUCCESS) return e;
+    if (overlapped) { if ((e = cusync_invoke_wait_kernel(&L->st[1], s2)) != CUSYNC_SUCCESS) return e; }
+    else if (CUSYNC_HIP(hipEventRecord(L->eMid2, s0))) return CUSYNC_ERROR_DEVICE;
+    if ((e = cusync_gemm_run(&a3, s2)) != CUSYNC_SUCCESS) return e;
+    if (CUSYNC_HIP(hipEventRecord(L->eEnd, s2))) return CUSYNC_ERROR_DEVICE;
+    if (CUSYNC_HIP(hipEventSynchronize(L->eEnd))) return CUSYNC_ERROR_DEVICE;
+    if (overlapped && (CUSYNC_HIP(hipStreamSynchronize(s0)) || CUSYNC_HIP(hipStreamSynchronize(s1)))) return CUSYNC_ERROR_DEVICE;
+    float ms = 0;
+    if (times_us) {
+      if (CUSYNC_HIP(hipEventElapsedTime(&ms, L->eStart, L->eEnd))) return CUSYNC_ERROR_DEVICE;
+      times_us[r] = (double)ms * 1000.0;
+    }
+    if (!overlapped && stage_us) {
+      hipEvent_t ev[4] = {L->eStart, L->eMid1, L->eMid2, L->eEnd};
+      for (int i = 0; i < 3; i++) {
+        if (CUSYNC_HIP(hipEventElapsedTime(&ms, ev[i], ev[i + 1]))) return CUSYNC_ERROR_DEVICE;
+        stage_us[3 * r + i] = (double)ms * 1000.0;
+      }
+    }
+    for (int i = 0; i < 3; i++) L->st[i].iter += 1;
+  }
+  return CUSYNC_SUCCESS;
+}
+
+const cusync_stage_desc* cusync_attn_layer_stage(const cusync_attn_layer* L, int which) {
+  if (!L || which < 0 || which > 2) return nullptr;
+  return &L->st[which];
+}
+
+int cusync_attn_layer_tiles(const cusync_attn_layer* L, int* tile1, int* tile3) {
+  if (!L) return 1;
+  if (tile1) *tile1 = L->tile1;
+  if (tile3) *tile3 = L->tile3;
+  return 0;
+}
+
+}  // extern "C"

@@ -255,6 +255,61 @@ int cusync_conv2d_max_resident(int tile);
 cusync_error cusync_conv2d_run(const cusync_conv2d_args *args, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Fused multi-head attention stage: O = softmax(mask(Q K^T * scale)) V per    */
+/* head, fp16 in/out, fp32 accumulate.  Takes the place of the two inner GEMM  */
+/* stages S = Q K^T and O = P V of the reference's attention chain (gemm_op2 / */
+/* gemm_op3 with SCuStage / OCuStage, TB/attention.cu:101-104, 797-803): it is */
+/* a consumer of the QKV projection and a producer for the output projection.  */
+/* ------------------------------------------------------------------------- */
+
+typedef struct cusync_attention_args {
+  cusync_stage_desc stage;     /* grid = cusync_attention_grid(seq, heads) */
+  uint32_t seq, heads, head_dim;   /* head_dim must be 128 */
+  const void *qkv;             /* [seq][ldqkv] fp16: Q at column 0, K at heads*head_dim, V at 2*heads*head_dim */
+  uint32_t ldqkv;
+  void *out;                   /* [seq][ldo] fp16, head h in columns h*head_dim .. */
+  uint32_t ldo;
+  float scale;                 /* softmax scale; 0 selects 1/sqrt(head_dim) */
+  int32_t causal;              /* 1: query i sees keys 0..i */
+  int32_t max_workgroups;      /* 0 = as many as stay resident */
+} cusync_attention_args;
+
+/* Rows per output tile (128), columns per output tile (= head_dim) and key/value rows per inner step. */
+int cusync_attention_tile_shape(uint32_t *tileM, uint32_t *tileN, uint32_t *blockKV);
+/* Logical grid (heads, row tiles, 1); an output tile is posted as {row, head*head_dim, 0}. */
+cusync_dim3 cusync_attention_grid(uint32_t seq, uint32_t heads);
+cusync_error cusync_attention_can_implement(const cusync_attention_args *args);
+int cusync_attention_max_resident(void);
+/* As a consumer (input policy RowSync, TileSync or ConsecutiveSync over the QKV projection's tiles) the
+ * kernel waits for the producer tiles holding its Q rows, and for those of each K / V block right
+ * before loading it; as a producer it posts each finished output tile. */
+cusync_error cusync_attention_run(const cusync_attention_args *args, void *stream);
+
+/* Self-attention chain X Wqkv -> attention -> O Wo (TB/attention.cu:560-830 runBaseline / runCuSync). */
+typedef struct cusync_attn_layer_config {
+  uint32_t seq;                /* rows of X */
+  uint32_t hidden;             /* columns of X and of Y (12288 for the GPT-3 shard) */
+  uint32_t heads, head_dim;    /* 12 x 128 per GPU */
+  int32_t sync;                /* CUSYNC_SYNC_*; STRIDED = ConsecutiveSync into the attention, RowSync out of it */
+  int32_t tile1, tile3;        /* GEMM tile ids, -1 = built-in choice */
+  int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = none */
+  int32_t causal;
+} cusync_attn_layer_config;
+
+typedef struct cusync_attn_layer cusync_attn_layer;
+
+/* wqkv: [hidden][3*heads*head_dim], wo: [heads*head_dim][hidden], both fp16 row-major device pointers. */
+cusync_attn_layer *cusync_attn_layer_create(const cusync_attn_layer_config *cfg, const void *wqkv, const void *wo);
+void cusync_attn_layer_destroy(cusync_attn_layer *layer);
+/* x: [seq][hidden]; qkv: [seq][3*heads*head_dim]; o: [seq][heads*head_dim]; y: [seq][hidden].  Runs `runs`
+ * times, synchronising after each; times_us[r] = start of the first kernel to end of the last.  For the
+ * stream-ordered mode stage_us[3*r + i] receives the time of stage i. */
+cusync_error cusync_attn_layer_run(cusync_attn_layer *layer, const void *x, void *qkv, void *o, void *y, int runs,
+                                   double *times_us, double *stage_us);
+const cusync_stage_desc *cusync_attn_layer_stage(const cusync_attn_layer *layer, int which);
+int cusync_attn_layer_tiles(const cusync_attn_layer *layer, int *tile1, int *tile3);
+
+/* ------------------------------------------------------------------------- */
 /* MLP chain (replaces the extern "C" surface of TB/mlp-lib.cu:555-618 and    */
 /* the hot loops runBaselineGPT3 / runCuSyncGPT3 / runCuSyncLLaMA,            */
 /* TB/mlp.cu:411-491, 645-716, 718-862)                                       */

@@ -1,0 +1,174 @@
+"""GPU parity of the fused attention stage (cusync_attention_*) and of the self-attention chain
+X Wqkv -> softmax(mask(Q K^T / sqrt(128))) V -> O Wo (cusync_attn_layer_*) against the CPU oracle,
+stream-ordered and under RowSync / TileSync / ConsecutiveSync (the wiring of
+src/ml-bench/transformer/attention.cu:84-110).  Shapes of the benchmark: 12 heads x 128 per GPU,
+hidden 12288, sequence 256..2048."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from cusync_amd import _lib, api
+from util import assert_close, empty_dev, normal_f16, sample_rows, to_dev, to_host, uniform_f16
+
+pytestmark = pytest.mark.gpu
+
+
+def run_attention(qkv, heads, causal=True, max_workgroups=0, launches=1):
+    import torch
+    L = _lib.load()
+    S = qkv.shape[0]
+    dq = to_dev(qkv)
+    do = empty_dev((S, heads * 128), fill=float("nan"))
+    torch.cuda.synchronize()
+    st = api.Stage(api.attention_grid(S, heads), (1, 1, 1), api.no_sync(), api.no_sync())
+    for _ in range(launches):
+        do.fill_(float("nan"))
+        torch.cuda.synchronize()
+        rc = api.attention(st, S, heads, dq.data_ptr(), qkv.shape[1], do.data_ptr(), heads * 128, causal=causal,
+                           max_workgroups=max_workgroups)
+        assert rc == api.ERR.SUCCESS, api.last_error()
+        assert L.cusync_rt_device_sync() == 0, api.last_error()
+    assert st.read_state().tile_counter == 0
+    st.destroy()
+    return to_host(do)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("S,heads", [(1, 1), (64, 1), (100, 2), (128, 1), (129, 1), (200, 3), (256, 12), (448, 2), (1000, 1)])
+def test_attention_matches_oracle(S, heads, causal):
+    print("attention", S, heads, causal, flush=True)
+    qkv = normal_f16((S, 3 * heads * 128), 11, std=1.0)
+    got = run_attention(qkv, heads, causal)
+    assert_close(got, orc.attention(qkv, heads, 128, causal), "O")
+
+
+def test_attention_closed_forms():
+    S, heads = 300, 2
+    E = heads * 128
+    rng = np.random.default_rng(5)
+    qkv = normal_f16((S, 3 * E), 12, std=1.0)
+    # Q = 0: every visible key weighs the same, row i of O is the mean of V rows 0..i
+    qkv[:, :E] = 0
+    v = rng.integers(-4, 5, (S, E)).astype(np.float16)
+    qkv[:, 2 * E:] = v
+    got = run_attention(qkv, heads, True).astype(np.float32)
+    want = np.cumsum(v.astype(np.float64), axis=0) / np.arange(1, S + 1)[:, None]
+    assert np.array_equal(got[0], v[0].astype(np.float32))          # first row sees only itself
+    assert np.max(np.abs(got - want)) < 4e-3
+    # all V rows equal: the weights sum to one, so O repeats that row whatever Q and K are
+    qkv = normal_f16((S, 3 * E), 13, std=1.0)
+    qkv[:, 2 * E:] = v[7]
+    got = run_attention(qkv, heads, False).astype(np.float32)
+    assert np.max(np.abs(got - v[7].astype(np.float32)[None, :])) < 4e-3
+    # a key that dominates: K row 5 = 16 * Q direction for every query, so O is V row 5 for rows >= 5
+    qkv = np.zeros((S, 3 * E), np.float16)
+    qkv[:, :E] = 1.0
+    qkv[5, E:2 * E] = 16.0
+    qkv[:, 2 * E:] = v
+    got = run_attention(qkv, heads, True).astype(np.float32)
+    assert np.array_equal(got[5:], np.broadcast_to(v[5].astype(np.float32), got[5:].shape))
+
+
+def test_attention_persistent_launch_and_relaunch():
+    qkv = normal_f16((512, 3 * 4 * 128), 14, std=1.0)
+    got = run_attention(qkv, 4, True, max_workgroups=3, launches=2)
+    assert_close(got, orc.attention(qkv, 4, 128, True), "O")
+
+
+def test_attention_can_implement_rejects():
+    import torch
+    L = _lib.load()
+    buf = torch.zeros(1 << 20, dtype=torch.float16, device="cuda")
+    st = api.Stage(api.attention_grid(256, 2), (1, 1, 1), api.no_sync(), api.no_sync())
+
+    def rc(seq=256, heads=2, ldqkv=768, ldo=256, **kw):
+        a = api.attention_args(st, seq, heads, buf.data_ptr(), ldqkv, buf.data_ptr(), ldo, **kw)
+        return L.cusync_attention_can_implement(C.byref(a))
+
+    assert rc() == api.ERR.SUCCESS
+    assert rc(head_dim=64) != api.ERR.SUCCESS
+    assert rc(ldqkv=512) != api.ERR.SUCCESS          # narrower than Q|K|V
+    assert rc(ldo=128) != api.ERR.SUCCESS
+    assert rc(seq=512) != api.ERR.SUCCESS            # stage grid no longer matches
+    assert rc(heads=3, ldqkv=1152, ldo=384) != api.ERR.SUCCESS
+    assert "attention" in api.last_error()
+    cons = api.Stage(api.attention_grid(256, 2), (1, 1, 1), api.strided_sync(api.ORDER.TRANSPOSE_XY, 256, 128, 128, 2), api.no_sync())
+    a = api.attention_args(cons, 256, 2, buf.data_ptr(), 768, buf.data_ptr(), 256)
+    assert L.cusync_attention_can_implement(C.byref(a)) != api.ERR.SUCCESS   # unpaired, and not a supported policy
+    st.destroy(); cons.destroy()
+
+
+_weights = {}
+
+
+def layer_weights(hidden, heads):
+    key = (hidden, heads)
+    if key not in _weights:
+        E = heads * 128
+        wqkv = normal_f16((hidden, 3 * E), 2)
+        wo = normal_f16((E, hidden), 3)
+        _weights[key] = (wqkv, wo, to_dev(wqkv), to_dev(wo))
+    return _weights[key]
+
+
+def run_layer(S, hidden, heads, sync, runs=2, **kw):
+    import torch
+    wqkv, wo, dwqkv, dwo = layer_weights(hidden, heads)
+    E = heads * 128
+    x = uniform_f16((S, hidden), 1)
+    dx = to_dev(x)
+    dqkv = empty_dev((S, 3 * E), fill=float("nan"))
+    do = empty_dev((S, E), fill=float("nan"))
+    dy = empty_dev((S, hidden), fill=float("nan"))
+    torch.cuda.synchronize()
+    layer = api.AttnLayer(S, hidden, heads, sync, dwqkv.data_ptr(), dwo.data_ptr(), **kw)
+    times = layer.run(dx.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=runs)
+    states = [layer.stage_state(i) for i in range(3)]
+    tiles = layer.tiles()
+    layer.destroy()
+    return x, wqkv, wo, to_host(dqkv), to_host(do), to_host(dy), states, tiles, times
+
+
+def expected_sems(state, tile_m, tile_n, iters):
+    d = state.desc
+    p = orc.Policy(d.out.kind, d.out.order, d.out.tileM, d.out.tileN, d.out.waitValue, d.out.postValue,
+                   d.out.gridN, d.out.stride, d.out.R, d.out.S, d.out.H)
+    return orc.expected_sems_gemm(p, state.grid, tile_m, tile_n, iters, d.opts)
+
+
+def check_layer(S, hidden, heads, sampled, **kw):
+    outs = {}
+    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE, api.SYNC.STRIDED):
+        print("  sync", sync, flush=True)
+        x, wqkv, wo, qkv, o, y, states, tiles, _ = run_layer(S, hidden, heads, sync, runs=2, **kw)
+        outs[sync] = (qkv, o, y)
+        for st in states:
+            assert st.spin_timeouts == 0 and st.tile_counter == 0 and st.start_counter == 0
+        if sync != api.SYNC.STREAM:
+            tm, tn, _ = api.tile_shape(tiles[0])
+            assert np.array_equal(states[0].sems, expected_sems(states[0], tm, tn, 2))
+            assert np.array_equal(states[1].sems, expected_sems(states[1], 128, 128, 2))
+            assert states[0].kernel_executed == 2 and states[1].kernel_executed == 2
+    qkv, o, y = outs[api.SYNC.STREAM]
+    rows = sample_rows(S) if sampled else list(range(S))
+    assert_close(qkv[rows], orc.gemm(np.ascontiguousarray(x[rows]), wqkv), "QKV rows")
+    # later stages are checked on the intermediates the GPU produced
+    assert_close(o, orc.attention(qkv, heads, 128, True), "O")
+    assert_close(y[rows], orc.gemm(np.ascontiguousarray(o[rows]), wo), "Y rows")
+    for sync in (api.SYNC.ROW, api.SYNC.TILE, api.SYNC.STRIDED):       # synchronisation only changes timing
+        for got, want, name in zip(outs[sync], outs[api.SYNC.STREAM], ("QKV", "O", "Y")):
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (sync, name)
+
+
+@pytest.mark.parametrize("S,tile", [(256, api.TILE.T128x128x64), (200, api.TILE.T64x128x64), (384, api.TILE.T128x256x32)])
+def test_attention_layer_small(S, tile):
+    print("attn layer small", S, tile, flush=True)
+    check_layer(S, 512, 2, sampled=False, tile1=tile, tile3=tile)
+
+
+@pytest.mark.parametrize("S", [256, 512, 1024, 2048])
+def test_attention_layer_gpt3_shard(S):
+    print("attn layer gpt3", S, flush=True)
+    check_layer(S, 12288, 12, sampled=True)
