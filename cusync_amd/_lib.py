@@ -30,7 +30,7 @@ class PolicyDesc(C.Structure):
 
 class StageDesc(C.Structure):
     _fields_ = [("grid", Dim3), ("prodGrid", Dim3), ("tileSize", Dim3),
-                ("iter", i32), ("opts", i32), ("in_", PolicyDesc), ("out", PolicyDesc),
+                ("iter", i32), ("opts", i32), ("flags", u32), ("reserved", u32), ("in_", PolicyDesc), ("out", PolicyDesc),
                 ("tileOrder", vp), ("tileCounter", vp), ("startCounter", vp), ("xcdTickets", vp),
                 ("kernelExecuted", vp), ("spinTimeouts", vp),
                 ("tileStatusWrite", vp), ("tileStatusRead", vp)]
@@ -47,6 +47,11 @@ class Conv2dArgs(C.Structure):
     _fields_ = [("stage", StageDesc), ("N", u32), ("H", u32), ("W", u32), ("C", u32), ("K", u32), ("R", u32), ("S", u32),
                 ("pad", u32), ("stride", u32), ("x", vp), ("w", vp), ("y", vp),
                 ("epilogue", i32), ("tile", i32), ("max_workgroups", i32)]
+
+
+class ConvChainConfig(C.Structure):
+    _fields_ = [("N", u32), ("H", u32), ("W", u32), ("C", u32), ("layers", u32), ("sync", i32), ("tile", i32),
+                ("opts", i32), ("relu", i32)]
 
 
 class AttentionArgs(C.Structure):
@@ -110,6 +115,11 @@ SIGNATURES = {
     "cusync_conv2d_can_implement": (C.c_int, [C.POINTER(Conv2dArgs)]),
     "cusync_conv2d_max_resident": (C.c_int, [C.c_int]),
     "cusync_conv2d_run": (C.c_int, [C.POINTER(Conv2dArgs), vp]),
+    "cusync_conv_chain_create": (vp, [C.POINTER(ConvChainConfig), C.POINTER(vp)]),
+    "cusync_conv_chain_destroy": (None, [vp]),
+    "cusync_conv_chain_run": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "cusync_conv_chain_stage": (C.POINTER(StageDesc), [vp, u32]),
+    "cusync_conv_chain_tile": (C.c_int, [vp]),
     "cusync_attention_tile_shape": (C.c_int, [C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_attention_grid": (Dim3, [u32, u32]),
     "cusync_attention_can_implement": (C.c_int, [C.POINTER(AttentionArgs)]),

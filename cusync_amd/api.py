@@ -9,7 +9,7 @@ import ctypes as C
 from types import SimpleNamespace
 
 from . import _lib
-from ._lib import AttentionArgs, AttnLayerConfig, Conv2dArgs, Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
+from ._lib import AttentionArgs, AttnLayerConfig, Conv2dArgs, ConvChainConfig, Dim3, GemmArgs, MlpConfig, PolicyDesc, StageDesc
 
 ERR = SimpleNamespace(NOT_PRODUCER=0, NOT_CONSUMER=1, NOT_INITIALIZED=2,
                       INVALID_LINEAR_BLOCK_INDEX=3, DEVICE=4, SUCCESS=5)
@@ -223,6 +223,40 @@ def conv2d(stage, N, H, W, Cc, K, x, w, y, tile, stream=None, **kw):
     return _lib.load().cusync_conv2d_run(C.byref(a), stream)
 
 
+class ConvChain:
+    """Handle over cusync_conv_chain_*: `layers` dependent 3x3 convolutions, stream-ordered or one CuSync
+    stage per layer (src/ml-bench/volta_conv2d/resnet.cu, vgg.cu)."""
+
+    def __init__(self, N, H, W, Cc, weight_ptrs, sync, tile=-1, opts=-1, relu=True):
+        self.L = _lib.load()
+        self.layers = len(weight_ptrs)
+        self.cfg = ConvChainConfig(N, H, W, Cc, self.layers, sync, tile, opts, int(relu))
+        arr = (C.c_void_p * self.layers)(*weight_ptrs)
+        self.h = self.L.cusync_conv_chain_create(C.byref(self.cfg), arr)
+        if not self.h:
+            raise RuntimeError("cusync_conv_chain_create failed: " + last_error())
+
+    def run(self, x_ptr, y_ptrs, runs=1, layers=False):
+        times = (C.c_double * runs)()
+        per = (C.c_double * (runs * self.layers))()
+        ys = (C.c_void_p * self.layers)(*y_ptrs)
+        check(self.L.cusync_conv_chain_run(self.h, x_ptr, ys, runs, times, per), "cusync_conv_chain_run")
+        if layers:
+            return list(times), [list(per[r * self.layers:(r + 1) * self.layers]) for r in range(runs)]
+        return list(times)
+
+    def tile(self):
+        return self.L.cusync_conv_chain_tile(self.h)
+
+    def stage_state(self, which):
+        return _read_stage(self.L, self.L.cusync_conv_chain_stage(self.h, which).contents)
+
+    def destroy(self):
+        if self.h:
+            self.L.cusync_conv_chain_destroy(self.h)
+            self.h = None
+
+
 # ---- attention -------------------------------------------------------------------
 
 def attention_tile_shape():
@@ -331,19 +365,7 @@ class Mlp:
         return a.value, b.value
 
     def stage_state(self, which):
-        import numpy as np
-        d = self.L.cusync_mlp_stage(self.h, which).contents
-        g = d.grid
-        n = g.x * g.y * g.z
-        sems = np.zeros(n, np.uint32)
-        order = np.zeros((n, 3), np.uint32)
-        tc, sc, ke, to = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
-        producer = d.out.kind != POLICY.NOSYNC
-        check(self.L.cusync_stage_read_state(C.byref(d), sems.ctypes.data_as(C.c_void_p) if producer else None,
-                                             order.ctypes.data_as(C.c_void_p), C.byref(tc), C.byref(sc),
-                                             C.byref(ke), C.byref(to)), "read_state")
-        return SimpleNamespace(desc=d, grid=g.tup(), sems=sems, tile_order=order, tile_counter=tc.value,
-                               start_counter=sc.value, kernel_executed=ke.value, spin_timeouts=to.value)
+        return _read_stage(self.L, self.L.cusync_mlp_stage(self.h, which).contents)
 
     def destroy(self):
         if self.h:

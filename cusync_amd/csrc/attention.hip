@@ -25,19 +25,22 @@ using namespace cusync::attn;
 std::mutex g_attnMutex;
 int g_attnResidentPerCU = -1;
 
+int g_attnNumCUs = 0;
+
 int residentAttention() {
   std::lock_guard<std::mutex> lock(g_attnMutex);
-  int dev = 0;
-  hipDeviceProp_t prop;
-  if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
   if (g_attnResidentPerCU < 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
+    g_attnNumCUs = prop.multiProcessorCount;
     if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attentionKernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes))) return 0;
     int n = 0;
     if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attentionKernel, kThreads, kLdsBytes))) return 0;
     g_attnResidentPerCU = n;
   }
-  return g_attnResidentPerCU * prop.multiProcessorCount;
+  return g_attnResidentPerCU * g_attnNumCUs;
 }
 
 cusync_policy_desc noSync() {

@@ -85,8 +85,6 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   const uint32_t vEven = vRowOff + vColOff + 64 * flip;          // tiles t = 0, 2: + 64 t
   const uint32_t vOdd = vRowOff + vColOff + 64 - 64 * flip;      // tiles t = 1, 3: + 64 (t - 1)
 
-  if (tid == 0) stage.announceStart(p.launched);
-
   const uint32_t numTiles = stage.numTiles();
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
@@ -103,12 +101,19 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     }
   };
 
-  uint32_t dryXcds = 0;
+  // Thread 0 keeps the ticket state: the start count is issued first and settled after the
+  // first tile's loads are under way; the draw of the next ticket is issued while a tile is
+  // being computed and settled when the tile is done.
+  uint32_t dryXcds = 0, nextRaw = 0;
+  const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = stage.drawTicket(p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
     __syncthreads();
     const uint32_t ticket = sTicket;
-    if (ticket >= numTiles) break;
+    if (ticket >= numTiles) {
+      if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+      break;
+    }
     const cusync_dim3 t = stage.ticketToTile(ticket);
     const uint32_t head = t.x, q0 = t.y * kBQ;
     const uint32_t qEnd = min(q0 + (uint32_t)kBQ, p.S);
@@ -147,6 +152,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
 
     waitKV(0);
     issue(0, 0);
+    if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
 
     float rowMax = kMasked, rowSum = 0.0f;      // rowSum: this half-wave's share
     floatx16 o[4];
@@ -232,6 +238,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
         }
     }
 
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
     // Normalise and store: register r of tile tt is head-dim 32tt + 8(r/4) + 4hi + r%4 of query myq.
     rowSum += __shfl_xor(rowSum, 32);
     const float inv = 1.0f / rowSum;

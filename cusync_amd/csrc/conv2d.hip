@@ -14,8 +14,10 @@
 // halo reaches, not only for the block of its own rows.
 #include <hip/hip_runtime.h>
 
+#include <string.h>
 #include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "../../include/cusync_amd.h"
 #include "rt_internal.h"
@@ -49,19 +51,22 @@ ConvTile* convTile(int tile) {
   return &g_convTiles[tile];
 }
 
+int g_convNumCUs = 0;
+
 int residentConv(ConvTile* ti) {
   std::lock_guard<std::mutex> lock(g_convMutex);
-  int dev = 0;
-  hipDeviceProp_t prop;
-  if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
   if (ti->residentPerCU < 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
+    g_convNumCUs = prop.multiProcessorCount;
     if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds))) return 0;
     int n = 0;
     if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel, kThreads, ti->lds))) return 0;
     ti->residentPerCU = n;
   }
-  return ti->residentPerCU * prop.multiProcessorCount;
+  return ti->residentPerCU * g_convNumCUs;
 }
 
 uint32_t outExtent(uint32_t in, uint32_t filter, uint32_t pad, uint32_t stride) { return (in + 2 * pad - filter) / stride + 1; }
@@ -166,5 +171,157 @@ cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }
+
+}  // extern "C"
+
+/* ---- chain of same-shape 3x3 convolutions ------------------------------------------ */
+
+struct cusync_conv_chain {
+  cusync_conv_chain_config cfg;
+  std::vector<const void*> w;
+  std::vector<cusync_stage_desc> st;
+  std::vector<hipStream_t> stream;
+  std::vector<hipEvent_t> ev;        // layers + 1 events: start, after each layer
+};
+
+namespace {
+
+cusync_policy_desc noSyncDesc() {
+  cusync_policy_desc p;
+  memset(&p, 0, sizeof p);
+  p.kind = CUSYNC_POLICY_NOSYNC;
+  p.tileM = p.tileN = 1; p.R = p.S = 1;
+  return p;
+}
+
+void freeChain(cusync_conv_chain* c) {
+  for (auto s : c->stream) (void)hipStreamSynchronize(s);
+  for (auto& d : c->st) cusync_stage_free(&d);
+  for (auto e : c->ev) (void)hipEventDestroy(e);
+  for (auto s : c->stream) (void)hipStreamDestroy(s);
+  delete c;
+}
+
+}  // namespace
+
+extern "C" {
+
+cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg, const void* const* weights) {
+  using cusync::rt::setError;
+  if (!cfg || !weights) { setError("conv chain: null argument"); return nullptr; }
+  if (cfg->layers < 1 || cfg->layers > 16) { setError("conv chain: 1 to 16 layers"); return nullptr; }
+  cusync_conv_chain* c = new cusync_conv_chain();
+  c->cfg = *cfg;
+  if (c->cfg.tile < 0) c->cfg.tile = cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_128x64x32;
+  uint32_t tm = 0, tn = 0;
+  if (cusync_conv2d_tile_shape(c->cfg.tile, &tm, &tn, nullptr)) { setError("conv chain: unknown tile id"); delete c; return nullptr; }
+  const cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);
+  if (g.x == 0 || g.y == 0) { setError("conv chain: empty shape"); delete c; return nullptr; }
+
+  // Edge policies: what a layer posts and what the next one waits on
+  // (src/ml-bench/volta_conv2d/resnet.cu:107-116; in vgg.cu the middle layers are consumer and producer at once).
+  cusync_policy_desc post = noSyncDesc(), wait = noSyncDesc();
+  int opts = 0;
+  switch (cfg->sync) {
+    case CUSYNC_SYNC_STREAM:
+      break;
+    case CUSYNC_SYNC_ROW:
+      post.kind = CUSYNC_POLICY_ROWSYNC; post.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      post.tileM = tm; post.tileN = 1; post.waitValue = g.x; post.postValue = 1;
+      wait = post;
+      break;
+    case CUSYNC_SYNC_TILE:
+      post.kind = CUSYNC_POLICY_TILESYNC; post.order = CUSYNC_ORDER_TRANSPOSE_XY;
+      post.tileM = tm; post.tileN = tn; post.waitValue = 1; post.postValue = 1;
+      wait = post;
+      wait.kind = CUSYNC_POLICY_CONV2DTILESYNC; wait.R = 3; wait.S = 3;
+      opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
+      break;
+    default:
+      setError("conv chain: sync must be STREAM, ROW or TILE");
+      delete c;
+      return nullptr;
+  }
+  if (cfg->opts >= 0) opts |= cfg->opts;
+  c->st.resize(cfg->layers);
+  for (uint32_t i = 0; i < cfg->layers; i++) memset(&c->st[i], 0, sizeof c->st[i]);
+  for (uint32_t i = 0; i < cfg->layers; i++) {
+    c->w.push_back(weights[i]);
+    cusync_stage_desc& d = c->st[i];
+    d.grid = g; d.tileSize = {1, 1, 1}; d.iter = 1; d.opts = opts;
+    d.in = i == 0 ? noSyncDesc() : wait;
+    d.out = i + 1 == cfg->layers ? noSyncDesc() : post;
+    if (!weights[i] || cusync_stage_create(&d, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) { freeChain(c); return nullptr; }
+  }
+  if (cfg->sync != CUSYNC_SYNC_STREAM)
+    for (uint32_t i = 0; i + 1 < cfg->layers; i++)
+      if (cusync_set_producer_consumer_pair(&c->st[i], &c->st[i + 1]) != CUSYNC_SUCCESS) { freeChain(c); return nullptr; }
+  const uint32_t streams = cfg->sync == CUSYNC_SYNC_STREAM ? 1 : cfg->layers;
+  for (uint32_t i = 0; i < streams; i++) {
+    hipStream_t s;
+    if (CUSYNC_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking))) { freeChain(c); return nullptr; }
+    c->stream.push_back(s);
+  }
+  for (uint32_t i = 0; i <= cfg->layers; i++) {
+    hipEvent_t e;
+    if (CUSYNC_HIP(hipEventCreate(&e))) { freeChain(c); return nullptr; }
+    c->ev.push_back(e);
+  }
+  return c;
+}
+
+void cusync_conv_chain_destroy(cusync_conv_chain* c) {
+  if (c) freeChain(c);
+}
+
+cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* const* ys, int runs,
+                                   double* times_us, double* layer_us) {
+  if (!c || !x || !ys) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const uint32_t n = c->cfg.layers;
+  const bool overlapped = c->cfg.sync != CUSYNC_SYNC_STREAM;
+  for (int r = 0; r < runs; r++) {
+    if (CUSYNC_HIP(hipEventRecord(c->ev[0], c->stream[0]))) return CUSYNC_ERROR_DEVICE;
+    for (uint32_t i = 0; i < n; i++) {
+      hipStream_t s = c->stream[overlapped ? i : 0];
+      cusync_conv2d_args a;
+      memset(&a, 0, sizeof a);
+      a.stage = c->st[i];
+      a.N = c->cfg.N; a.H = c->cfg.H; a.W = c->cfg.W; a.C = c->cfg.C; a.K = c->cfg.C;
+      a.R = a.S = 3; a.pad = 1; a.stride = 1;
+      a.x = i == 0 ? x : ys[i - 1];
+      a.w = c->w[i];
+      a.y = ys[i];
+      a.epilogue = (c->cfg.relu && i + 1 < n) ? CUSYNC_EPILOGUE_RELU : CUSYNC_EPILOGUE_NONE;
+      a.tile = c->cfg.tile;
+      cusync_error e;
+      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
+      if ((e = cusync_conv2d_run(&a, s)) != CUSYNC_SUCCESS) return e;
+      if ((!overlapped || i + 1 == n) && CUSYNC_HIP(hipEventRecord(c->ev[i + 1], s))) return CUSYNC_ERROR_DEVICE;
+    }
+    if (CUSYNC_HIP(hipEventSynchronize(c->ev[n]))) return CUSYNC_ERROR_DEVICE;
+    if (overlapped)
+      for (uint32_t i = 0; i + 1 < n; i++)
+        if (CUSYNC_HIP(hipStreamSynchronize(c->stream[i]))) return CUSYNC_ERROR_DEVICE;
+    float ms = 0;
+    if (times_us) {
+      if (CUSYNC_HIP(hipEventElapsedTime(&ms, c->ev[0], c->ev[n]))) return CUSYNC_ERROR_DEVICE;
+      times_us[r] = (double)ms * 1000.0;
+    }
+    if (!overlapped && layer_us)
+      for (uint32_t i = 0; i < n; i++) {
+        if (CUSYNC_HIP(hipEventElapsedTime(&ms, c->ev[i], c->ev[i + 1]))) return CUSYNC_ERROR_DEVICE;
+        layer_us[(size_t)r * n + i] = (double)ms * 1000.0;
+      }
+    for (uint32_t i = 0; i < n; i++) c->st[i].iter += 1;
+  }
+  return CUSYNC_SUCCESS;
+}
+
+const cusync_stage_desc* cusync_conv_chain_stage(const cusync_conv_chain* c, uint32_t which) {
+  if (!c || which >= c->cfg.layers) return nullptr;
+  return &c->st[which];
+}
+
+int cusync_conv_chain_tile(const cusync_conv_chain* c) { return c ? c->cfg.tile : -1; }
 
 }  // extern "C"

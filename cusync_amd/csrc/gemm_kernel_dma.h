@@ -131,20 +131,25 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       bFragT[kk] = row * C::A_ROW_BYTES + (((2 * kk + (lane >> 5)) ^ swz) * 16);
   }
 
-  if (tid == 0) stage.announceStart(p.launched);
-
   const uint32_t numTiles = stage.numTiles();
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
   const bool chunkSync = consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
                          stage.d.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC;
 
-  uint32_t dryXcds = 0;
+  // Thread 0 keeps the ticket state: the start count is issued first and settled after the
+  // first tile's loads are under way; the draw of the next ticket is issued while a tile is
+  // being computed and settled when the tile is done.
+  uint32_t dryXcds = 0, nextRaw = 0;
+  const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = stage.drawTicket(p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
     __syncthreads();
     const uint32_t ticket = sTicket;
-    if (ticket >= numTiles) break;
+    if (ticket >= numTiles) {
+      if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+      break;
+    }
     const cusync_dim3 t = stage.ticketToTile(ticket);
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
@@ -357,6 +362,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); issueAll(Parity<2>{}, 2); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 4, "prologue written for 2..4 stages");
     earlyPoll(kBegin + (C::STAGES - 1) * C::BK);
+    if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
 
     for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
       step(Parity<0>{}, kt);
@@ -365,6 +371,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
     }
 
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
 
     // All waves must be past their last LDS read before the next tile's loads

@@ -63,8 +63,6 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   const int aFragOff = (wm * C::WTM + (lane & 31)) * C::PA + 8 * (lane >> 5);
   const int bFragOff = (8 * (lane >> 5) + ((lane & 15) >> 2)) * C::PB + wn * C::WTN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  if (tid == 0) stage.announceStart(p.launched);
-
   const uint32_t numTiles = stage.numTiles();
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
@@ -73,12 +71,19 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   const bool chunkSync = consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
                          stage.d.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC;
 
-  uint32_t dryXcds = 0;
+  // Thread 0 keeps the ticket state: the start count is issued first and settled after the
+  // first tile's loads are under way; the draw of the next ticket is issued while a tile is
+  // being computed and settled when the tile is done.
+  uint32_t dryXcds = 0, nextRaw = 0;
+  const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = stage.drawTicket(p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
     __syncthreads();
     const uint32_t ticket = sTicket;
-    if (ticket >= numTiles) break;
+    if (ticket >= numTiles) {
+      if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+      break;
+    }
     const cusync_dim3 t = stage.ticketToTile(ticket);      // x = column tile, y = row tile
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
@@ -240,6 +245,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
 
     issue(Parity<0>{}, 0);
     if (nk > 1) issue(Parity<1>{}, 1);
+    if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     earlyPoll(kBegin + 2 * C::BK);
     stash(Parity<0>{});
     __syncthreads();
@@ -249,6 +255,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
       if (kt + 1 < nk) step(Parity<1>{}, kt + 1);
     }
 
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
     cusync_dim3 done = {m0, n0, t.z};
     if (completed) stage.post(done);    // barrier inside when the stage is a producer (the decision is workgroup-uniform)

@@ -109,6 +109,12 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   d->xcdTickets = (uint32_t*)(counters + 4 * line);
   const bool producer = d->out.kind != CUSYNC_POLICY_NOSYNC;
   if (producer && !(d->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) d->kernelExecuted = (uint32_t*)(counters + 3 * line);
+  bool identity = true;
+  for (uint32_t i = 0; i < n && identity; i++) {
+    const cusync_dim3& t = host_tile_order[i];
+    identity = t.x == i % d->grid.x && t.y == (i / d->grid.x) % d->grid.y && t.z == i / (d->grid.x * d->grid.y);
+  }
+  d->flags = identity ? CUSYNC_STAGE_IDENTITY_ORDER : 0;
   if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return CUSYNC_ERROR_DEVICE;
   if (RT(hipMemcpy(d->tileOrder, host_tile_order, sizeof(cusync_dim3) * n, hipMemcpyHostToDevice))) return CUSYNC_ERROR_DEVICE;
   if (producer) {

@@ -36,67 +36,127 @@ struct DynStage {
   __device__ __forceinline__ uint32_t numTiles() const { return d.grid.x * d.grid.y * d.grid.z; }
   __device__ __forceinline__ bool customOrder() const { return !(d.opts & CUSYNC_OPT_AVOID_CUSTOM_ORDER); }
 
-  // Called once per workgroup by its first thread, before the first tile.
-  // `launched` = number of workgroups in this launch.
-  __device__ __forceinline__ void announceStart(uint32_t launched) const {
+  // ---- tickets -------------------------------------------------------------
+  // A launch may hold fewer workgroups than the stage has tiles; each workgroup
+  // then takes tickets until the tiles run out.  All of the following are
+  // called by the first thread of a workgroup only.
+  //
+  // Each of the eight XCDs has its own L2, so which workgroup gets which tile
+  // decides how much of the operands is re-fetched from memory.  The tiles are
+  // therefore dealt per XCD.  With at least eight column tiles XCD x owns the
+  // column tiles [x*gx/8, (x+1)*gx/8) of every row, in row-major order: its
+  // workgroups share the same few B column panels (and, row by row, the same
+  // A panels) in their L2.  With fewer column tiles (a convolution with 64
+  // output channels has one) XCD x owns the row tiles [x*gy/8, (x+1)*gy/8)
+  // instead, so that the rows of A it reads — for a convolution each input
+  // pixel is read by up to R*S neighbouring rows — stay in its L2.  The
+  // ticket is the tile's position in the row-major schedule; it still goes
+  // through the stage's ticket -> tile table.
+  //
+  // A device-wide atomic takes the better part of a microsecond, several when
+  // hundreds of workgroups hit one address at kernel start, and a kernel of a
+  // few tens of microseconds cannot afford a chain of them:
+  //  * Workgroups are dispatched to the XCDs round-robin: the workgroups
+  //    with the same index modulo 8 share an XCD (which one varies from launch
+  //    to launch, so the hardware XCD id is of no use here).  Workgroup b
+  //    therefore works on list b%8.  Where it really runs only matters for
+  //    locality: every position is taken exactly once either way.
+  //  * The first tile of a workgroup needs no atomic: it is position b/8 of
+  //    its list.
+  //  * Later tiles come from a dispenser per list that starts behind those
+  //    static positions.  The draw is split in two so that a kernel can issue
+  //    it before the epilogue of a tile and pick the result up afterwards.
+  //    (Not earlier: a workgroup that reserved its next tile at the start of
+  //    the current one would take work from workgroups that have none.)
+  //  * A workgroup whose own list is used up looks at all dispensers at once
+  //    (plain loads, one round trip): a counter seen at or above its list's
+  //    length is dry for good, the others are tried in turn, so the end of the
+  //    launch stays balanced.  The last workgroup to find everything dry
+  //    re-arms the dispensers for the next run.
+  __device__ __forceinline__ bool dealtByRows() const { return d.grid.x < 8; }
+  __device__ __forceinline__ uint32_t xcdTiles(uint32_t x) const {
+    const uint32_t span = dealtByRows() ? d.grid.y : d.grid.x;
+    return ((x + 1) * span / 8 - x * span / 8) * (dealtByRows() ? d.grid.x : d.grid.y) * d.grid.z;
+  }
+  // Positions of XCD x's list that are handed out statically to the first tiles of the workgroups.
+  __device__ __forceinline__ uint32_t xcdStatic(uint32_t x, uint32_t launched) const {
+    const uint32_t wgs = launched > x ? (launched - x + 7) / 8 : 0;
+    return min(wgs, xcdTiles(x));
+  }
+  __device__ __forceinline__ uint32_t xcdTicket(uint32_t x, uint32_t l) const {
+    const uint32_t span = dealtByRows() ? d.grid.y : d.grid.x;
+    const uint32_t lo = x * span / 8, width = (x + 1) * span / 8 - lo;
+    if (!dealtByRows()) return lo + l % width + (l / width) * d.grid.x;
+    const uint32_t perSlice = width * d.grid.x;          // this XCD's tiles in one k-slice
+    return (l / perSlice) * d.grid.x * d.grid.y + lo * d.grid.x + l % perSlice;
+  }
+  static __device__ __forceinline__ uint32_t workgroupIndex() {
+    return blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  }
+  static __device__ __forceinline__ uint32_t homeList() { return workgroupIndex() & 7u; }
+
+  // Counts this workgroup as started; give the result to finishStart() later
+  // (after other work has been issued, so that the round trip is hidden).
+  __device__ __forceinline__ uint32_t beginStart() const {
+    if (!isProducer() || (d.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) return 0;
+    return dev::ticketAdd(d.startCounter, 1);
+  }
+  // The workgroup that started last raises the wait-kernel flag.
+  __device__ __forceinline__ void finishStart(uint32_t token, uint32_t launched) const {
     if (!isProducer() || (d.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) return;
-    const uint32_t arrived = dev::ticketAdd(d.startCounter, 1);
-    if (arrived == launched - 1) {
+    if (token == launched - 1) {
       dev::storeRelaxed(d.startCounter, 0);
       dev::releaseStore(d.kernelExecuted, (uint32_t)d.iter);
     }
   }
 
-  // Id of the XCD (accelerator die) this wave runs on, 0..7.
-  static __device__ __forceinline__ uint32_t xcdId() {
-    uint32_t x;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
-    return x & 7u;
+  // Issues the draw of the next ticket; `dry` is the mask drawFinish() keeps.
+  __device__ __forceinline__ uint32_t drawBegin(uint32_t dry) const {
+    if (!customOrder()) return 0;
+    const uint32_t mine = homeList();
+    if (dry & (1u << mine)) return 0xffffffffu;
+    return dev::ticketAdd(&d.xcdTickets[mine * 32], 1);
   }
-
-  // Draws the next ticket for this workgroup (first thread only).  `round` is
-  // how many tickets this workgroup has already drawn, `dry` a bit mask the
-  // caller keeps across rounds (start it at 0).  Returns numTiles() or more
-  // when the tiles have run out.
-  //
-  // Each of the eight XCDs has its own L2, so which workgroup gets which tile
-  // decides how much of the operands is re-fetched from memory.  The tiles are
-  // therefore dealt per XCD: XCD x owns the column tiles [x*gx/8, (x+1)*gx/8) of
-  // every row, in row-major order, and a workgroup draws from the dispenser of
-  // the XCD it runs on.  The workgroups of one XCD thus share the same few B
-  // column panels (and, row by row, the same A panels) in their L2.  A
-  // workgroup whose own dispenser is empty helps the next XCD, so the end of the
-  // launch stays balanced.  The ticket returned is the tile's position in the
-  // row-major schedule; it still goes through the stage's ticket -> tile table.
-  __device__ __forceinline__ uint32_t drawTicket(uint32_t launched, uint32_t round, uint32_t& dry) const {
-    if (!customOrder()) {
-      const uint32_t wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-      return wg + round * launched;
-    }
+  // Turns the result of drawBegin() into a ticket; numTiles() or more when the
+  // tiles have run out.  `round` = tickets this workgroup has drawn before.
+  __device__ __forceinline__ uint32_t drawFinish(uint32_t raw, uint32_t launched, uint32_t round, uint32_t& dry) const {
+    if (!customOrder()) return workgroupIndex() + round * launched;
     constexpr uint32_t kLine = 32;          // counters are 128 bytes apart
-    const uint32_t mine = xcdId();
-    for (uint32_t s = 0; s < 8; s++) {
+    const uint32_t mine = homeList();
+    if (raw != 0xffffffffu) {
+      const uint32_t l = raw + xcdStatic(mine, launched);
+      if (l < xcdTiles(mine)) return xcdTicket(mine, l);
+    }
+    dry |= 1u << mine;
+    uint32_t seen[8];
+#pragma unroll
+    for (uint32_t x = 0; x < 8; x++) seen[x] = dev::loadRelaxed(&d.xcdTickets[x * kLine]);
+#pragma unroll
+    for (uint32_t x = 0; x < 8; x++)
+      if (seen[x] + xcdStatic(x, launched) >= xcdTiles(x)) dry |= 1u << x;
+    for (uint32_t s = 1; s < 8; s++) {
       const uint32_t x = (mine + s) & 7u;
       if (dry & (1u << x)) continue;
-      const uint32_t lo = x * d.grid.x / 8, cols = (x + 1) * d.grid.x / 8 - lo;
-      const uint32_t count = cols * d.grid.y * d.grid.z;
-      if (count != 0) {
-        const uint32_t l = dev::ticketAdd(&d.xcdTickets[x * kLine], 1);
-        if (l < count) return lo + l % cols + (l / cols) * d.grid.x;
-      }
+      const uint32_t l = dev::ticketAdd(&d.xcdTickets[x * kLine], 1) + xcdStatic(x, launched);
+      if (l < xcdTiles(x)) return xcdTicket(x, l);
       dry |= 1u << x;
     }
-    // Nothing left anywhere.  The last workgroup to find that out re-arms the
-    // dispensers for the next run.
     const uint32_t finished = dev::ticketAdd(&d.xcdTickets[8 * kLine], 1);
     if (finished == launched - 1) {
       for (uint32_t x = 0; x < 9; x++) dev::storeRelaxed(&d.xcdTickets[x * kLine], 0);
     }
     return 0xffffffffu;
   }
+  // First ticket of a workgroup: its static position if its XCD's list is long enough.
+  __device__ __forceinline__ uint32_t firstTicket(uint32_t launched, uint32_t& dry) const {
+    if (!customOrder()) return workgroupIndex();
+    const uint32_t b = workgroupIndex(), x = b & 7u, pos = b >> 3;
+    if (pos < xcdTiles(x)) return xcdTicket(x, pos);
+    return drawFinish(drawBegin(dry), launched, 0, dry);
+  }
 
   __device__ __forceinline__ cusync_dim3 ticketToTile(uint32_t ticket) const {
-    if (customOrder()) return d.tileOrder[ticket];
+    if (customOrder() && !(d.flags & CUSYNC_STAGE_IDENTITY_ORDER)) return d.tileOrder[ticket];
     cusync_dim3 t;
     t.x = ticket % d.grid.x;
     t.y = (ticket / d.grid.x) % d.grid.y;

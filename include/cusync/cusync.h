@@ -84,6 +84,7 @@ private:
   volatile uint32_t* tileStatusWrite_;
   volatile uint32_t* tileStatusRead_;
   int status_;                      // outcome of the constructor
+  uint32_t flags_;                  // CUSYNC_STAGE_* bits reported by cusync_stage_alloc
 
   friend class CuSyncTest;
   friend struct CuSync;
@@ -114,6 +115,7 @@ private:
     tileCounter = d.tileCounter;
     startCounter_ = d.startCounter;
     xcdTickets_ = d.xcdTickets;
+    flags_ = d.flags;
     kernelExecuted_ = d.kernelExecuted;
     spinTimeouts_ = d.spinTimeouts;
     tileStatusWrite_ = d.tileStatusWrite;
@@ -134,7 +136,7 @@ public:
       : grid_(grid), prodGrid_(0, 0, 0), tileSize_(tileSize), iter(1),
         inputPolicy_(inputPolicy), outputPolicy_(outputPolicy),
         tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), xcdTickets_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
-        tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncSuccess) {
+        tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncSuccess), flags_(0) {
     static_assert(!((Opts & NoAtomicAdd) && std::is_same<OutputSyncPolicy, NoSync>::value &&
                     std::is_same<InputSyncPolicy, NoSync>::value), "NoAtomicAdd on a stage that never syncs");
     status_ = buildScheduleBuffer();
@@ -143,7 +145,7 @@ public:
   CUSYNC_DEVICE_HOST CuStage()
       : grid_(0, 0, 0), prodGrid_(0, 0, 0), tileSize_(0, 0, 0), iter(1),
         tileOrder(nullptr), tileCounter(nullptr), startCounter_(nullptr), xcdTickets_(nullptr), kernelExecuted_(nullptr), spinTimeouts_(nullptr),
-        tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncErrorNotInitialized) {}
+        tileStatusWrite_(nullptr), tileStatusRead_(nullptr), status_(CuSyncErrorNotInitialized), flags_(0) {}
 
   // Outcome of construction: CuSyncSuccess, or CuSyncErrorInvalidLinearBlockIndex
   // when TileOrder::blockIndex is not a bijection onto [0, numTiles).
@@ -190,6 +192,7 @@ public:
     d.tileSize = {tileSize_.x, tileSize_.y, tileSize_.z};
     d.iter = iter;
     d.opts = Opts;
+    d.flags = flags_;
     d.in = inputPolicy_.desc();
     d.out = outputPolicy_.desc();
     d.tileOrder = (cusync_dim3*)tileOrder;

@@ -72,12 +72,18 @@ typedef struct cusync_policy_desc {
 
 /* Run-time image of a CuStage object (CS/cusync.h:93-117): what a kernel gets
  * by value.  Device pointers are owned by whoever called cusync_stage_alloc. */
+/* tileOrder[i] == (i % gx, (i / gx) % gy, i / (gx*gy)) for every i: true of both tile orders the reference
+ * ships (CS/tile-orders.h:52-75).  The prebuilt kernels then compute a ticket's tile instead of loading it. */
+enum { CUSYNC_STAGE_IDENTITY_ORDER = 1 };
+
 typedef struct cusync_stage_desc {
   cusync_dim3 grid;           /* grid_     : logical tile grid of this stage */
   cusync_dim3 prodGrid;       /* prodGrid_ : logical tile grid of its producer */
   cusync_dim3 tileSize;       /* tileSize_ : stored, never read (as in the reference) */
   int32_t iter;               /* run counter, starts at 1 */
   int32_t opts;               /* CUSYNC_OPT_* bits */
+  uint32_t flags;             /* CUSYNC_STAGE_* bits, filled in by cusync_stage_alloc */
+  uint32_t reserved;
   cusync_policy_desc in;      /* inputPolicy_  */
   cusync_policy_desc out;     /* outputPolicy_ */
   cusync_dim3 *tileOrder;     /* [numTiles] ticket -> tile */
@@ -253,6 +259,31 @@ int cusync_conv2d_max_resident(int tile);
 /* operator()(stream) (cusyncimplicit_gemm_convolution.h:283-298).  A consumer stage waits, per producer
  * channel tile, for every producer row block reached by the filter window of its rows. */
 cusync_error cusync_conv2d_run(const cusync_conv2d_args *args, void *stream);
+
+/* Chain of `layers` 3x3, pad 1, stride 1 convolutions with C input and C output channels each:
+ * two layers are the ResNet block of CV/resnet.cu:560-830 (producer + consumer), four are the VGG
+ * block of CV/vgg.cu, whose middle layers are consumer and producer at once. */
+typedef struct cusync_conv_chain_config {
+  uint32_t N, H, W, C;
+  uint32_t layers;             /* 1..16 */
+  int32_t sync;                /* CUSYNC_SYNC_STREAM, _ROW (RowSync both sides) or _TILE (TileSync -> Conv2DTileSync) */
+  int32_t tile;                /* CUSYNC_CONV_TILE_*, -1 = built-in choice */
+  int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = none */
+  int32_t relu;                /* 1: ReLU after every layer but the last */
+} cusync_conv_chain_config;
+
+typedef struct cusync_conv_chain cusync_conv_chain;
+
+/* weights[i]: filter of layer i, [C][3][3][C] fp16 device pointer. */
+cusync_conv_chain *cusync_conv_chain_create(const cusync_conv_chain_config *cfg, const void *const *weights);
+void cusync_conv_chain_destroy(cusync_conv_chain *chain);
+/* x: [N][H][W][C]; ys[i]: output of layer i, same shape.  Synchronises after each of the `runs` runs;
+ * times_us[r] = start of the first kernel to end of the last; in the stream-ordered mode
+ * layer_us[r*layers + i] receives the time of layer i. */
+cusync_error cusync_conv_chain_run(cusync_conv_chain *chain, const void *x, void *const *ys, int runs,
+                                   double *times_us, double *layer_us);
+const cusync_stage_desc *cusync_conv_chain_stage(const cusync_conv_chain *chain, uint32_t which);
+int cusync_conv_chain_tile(const cusync_conv_chain *chain);
 
 /* ------------------------------------------------------------------------- */
 /* Fused multi-head attention stage: O = softmax(mask(Q K^T * scale)) V per    */

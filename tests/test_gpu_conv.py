@@ -212,3 +212,47 @@ def test_resnet_conv_pair_full_size(shape, tile, kind):
     y2s = run_conv(y1s, w2, tile)
     assert np.array_equal(y1.view(np.uint16), y1s.view(np.uint16))
     assert np.array_equal(y2.view(np.uint16), y2s.view(np.uint16))
+
+
+def run_chain(N, H, W, Cc, layers, sync, runs=2, seed=30, **kw):
+    import torch
+    x = uniform_f16((N, H, W, Cc), seed)
+    ws = [he_filters(Cc, 3, 3, Cc, seed + 1 + i) for i in range(layers)]
+    dx = to_dev(x)
+    dws = [to_dev(w) for w in ws]
+    dys = [empty_dev((N, H, W, Cc), fill=float("nan")) for _ in range(layers)]
+    torch.cuda.synchronize()
+    chain = api.ConvChain(N, H, W, Cc, [w.data_ptr() for w in dws], sync, **kw)
+    times = chain.run(dx.data_ptr(), [y.data_ptr() for y in dys], runs=runs)
+    states = [chain.stage_state(i) for i in range(layers)]
+    tile = chain.tile()
+    chain.destroy()
+    return x, ws, [to_host(y) for y in dys], states, tile, times
+
+
+@pytest.mark.parametrize("shape,layers", [((4, 20, 20, 64), 2), ((32, 56, 56, 64), 2), ((32, 28, 28, 128), 2),
+                                          ((2, 24, 24, 64), 4), ((8, 28, 28, 128), 4), ((16, 56, 56, 64), 4)])
+def test_conv_chain_all_sync_modes(shape, layers):
+    # two layers: the ResNet block; four layers: the VGG block whose middle layers both wait and post
+    print("conv chain", shape, layers, flush=True)
+    outs = {}
+    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE):
+        x, ws, ys, states, tile, _ = run_chain(*shape, layers, sync, runs=2)
+        outs[sync] = ys
+        tm, tn, _ = api.conv2d_tile_shape(tile)
+        for i, st in enumerate(states):
+            assert st.spin_timeouts == 0 and st.tile_counter == 0 and st.start_counter == 0
+            if sync != api.SYNC.STREAM and i + 1 < layers:
+                d = st.desc
+                p = orc.Policy(d.out.kind, d.out.order, d.out.tileM, d.out.tileN, d.out.waitValue, d.out.postValue,
+                               d.out.gridN, d.out.stride, d.out.R, d.out.S, d.out.H)
+                assert np.array_equal(st.sems, orc.expected_sems_gemm(p, st.grid, tm, tn, 2, d.opts))
+                assert st.kernel_executed == 2
+    ys = outs[api.SYNC.STREAM]
+    src = x
+    for i in range(layers):      # each layer is checked on the input the GPU produced for it
+        assert_close(ys[i], orc.conv2d_nhwc(src, ws[i], epilogue=orc.EPI_RELU if i + 1 < layers else orc.EPI_NONE), "y%d" % i)
+        src = ys[i]
+    for sync in (api.SYNC.ROW, api.SYNC.TILE):
+        for i in range(layers):
+            assert np.array_equal(outs[sync][i].view(np.uint16), ys[i].view(np.uint16)), (sync, i)
