@@ -212,7 +212,7 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
   if (cfg->layers < 1 || cfg->layers > 16) { setError("conv chain: 1 to 16 layers"); return nullptr; }
   cusync_conv_chain* c = new cusync_conv_chain();
   c->cfg = *cfg;
-  if (c->cfg.tile < 0) c->cfg.tile = cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_128x64x32;
+  if (c->cfg.tile < 0) c->cfg.tile = cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_256x64x32;   // measured on 32x56x56x64 and 32x28x28x128
   uint32_t tm = 0, tn = 0;
   if (cusync_conv2d_tile_shape(c->cfg.tile, &tm, &tn, nullptr)) { setError("conv chain: unknown tile id"); delete c; return nullptr; }
   const cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);

@@ -362,6 +362,7 @@ typedef struct cusync_mlp_config {
                                   in GEMM2's A loader, 0 = GEMM2 reads the gate half as is (TB/mlp.cu:785-792) */
   int32_t split_k1, split_k2;  /* k-slices per GEMM (--split-k1/--split-k2, TB/mlp.cu:880-931); 0 = pick so that
                                   the launch fills the device */
+  int32_t max_wg1, max_wg2;    /* workgroups per launch of each GEMM; 0 = built-in choice, -1 = as many as stay resident */
 } cusync_mlp_config;
 
 typedef struct cusync_mlp cusync_mlp;   /* opaque */
