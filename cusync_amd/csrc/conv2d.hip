@@ -110,7 +110,7 @@ cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
     setError("conv2d: operand larger than 2 GiB is not addressable by one buffer descriptor");
     return CUSYNC_ERROR_NOT_INITIALIZED;
   }
-  if (((uintptr_t)a->x | (uintptr_t)a->w) % 16 || (uintptr_t)a->y % 8) { setError("conv2d: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (((uintptr_t)a->x | (uintptr_t)a->w | (uintptr_t)a->y) % 16) { setError("conv2d: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_RELU) { setError("conv2d: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const cusync_dim3 g = cusync_conv2d_grid(a->tile, a->N, a->H, a->W, a->K, a->R, a->S, a->pad, a->stride);
   const cusync_stage_desc& s = a->stage;

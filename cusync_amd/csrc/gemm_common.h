@@ -36,7 +36,7 @@ struct GemmParams {
   uint32_t launched;       // workgroups in this launch
   // split-K: slice z of a tile covers K columns [z*kPerSlice, (z+1)*kPerSlice)
   uint32_t splitK, kPerSlice;
-  float* partials;         // [splitK][mPad][N] fp32 partial sums
+  float* partials;         // [splitK][m-tiles][n-tiles][BM*BN] fp32 partial sums in register order
   uint32_t* arrivals;      // [m-tiles * n-tiles] slices finished per output tile; 0 between launches
   uint32_t mPad;           // m-tiles * BM
   // implicit-GEMM convolution (A is gathered from an NHWC tensor): M = n*P*Q, K = R*S*C, k = (r*S + s)*C + c
@@ -134,53 +134,70 @@ __device__ __forceinline__ void schedPass() {
 // counter and posts.  Must be called by all threads of the workgroup.
 template<class C>
 __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
-                                           const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast) {
+                                           const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
   const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
+  // Final values go through LDS so that global memory sees whole rows: a lane holds 4 consecutive columns of
+  // 32 different rows, which stored directly would be 8-byte pieces scattered over 32 cache lines per
+  // instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
+  // applied) into a [WM*32][BN] buffer (rows padded by 16 bytes against bank conflicts), then all threads
+  // copy the buffer out, 16 bytes per lane, consecutive lanes along a row.
   auto storeFinal = [&](auto&& value) {
+    constexpr int PITCH = C::BN * 2 + 16;
+    constexpr int ROWS = C::WM * 32;
+    constexpr int CPR = C::BN / 8;
+    constexpr int STEPS = ROWS * CPR / kThreads;
+    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
+    static_assert((ROWS * CPR) % kThreads == 0, "whole copy steps");
 #pragma unroll
     for (int i = 0; i < C::TM; i++) {
-      const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
+      __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
 #pragma unroll
-      for (int j = 0; j < C::TN; j++) {
+      for (int j = 0; j < C::TN; j++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-          const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
-          if (m < p.M && n < p.N) {
-            const floatx4 v = value(i, j, g, m, n);
-            half4 o;
+          const floatx4 v = value(i, j, g);
+          half4 o;
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
-            *reinterpret_cast<half4*>(p.D + (size_t)m * p.ldd + n) = o;
-          }
+          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
+          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = o;
         }
+      __syncthreads();
+#pragma unroll
+      for (int s = 0; s < STEPS; s++) {
+        const uint32_t idx = s * kThreads + threadIdx.x;
+        const uint32_t lr = idx / CPR, c = idx % CPR;
+        const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
+        if (m < p.M && n < p.N)
+          *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
       }
     }
   };
   if (p.splitK <= 1) {
-    storeFinal([&](int i, int j, int g, uint32_t, uint32_t) {
+    storeFinal([&](int i, int j, int g) {
       return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
     });
     return true;
   }
-  const size_t sliceStride = (size_t)p.mPad * p.N;
+  // Partial sums live in the workspace in register order: value g of MFMA tile (i, j) of every thread is one
+  // contiguous 4 KiB run (256 threads x 16 bytes), so slices write and the finishing slice reads with fully
+  // coalesced accesses; the padding rows and columns of edge tiles are carried along.
+  constexpr size_t kTileFloats = (size_t)C::BM * C::BN;
+  const size_t sliceStride = (size_t)p.stage.d.grid.x * p.stage.d.grid.y * kTileFloats;
+  float* mine = p.partials + ((size_t)t.y * p.stage.d.grid.x + t.x) * kTileFloats + (size_t)threadIdx.x * 4;
+  auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (kThreads * 4); };
 #pragma unroll
-  for (int i = 0; i < C::TM; i++) {
-    const uint32_t m = m0 + wm * C::WTM + i * 32 + (lane & 31);
+  for (int i = 0; i < C::TM; i++)
 #pragma unroll
-    for (int j = 0; j < C::TN; j++) {
+    for (int j = 0; j < C::TN; j++)
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const uint32_t n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5);
-        if (m < p.M && n < p.N)
-          *reinterpret_cast<floatx4*>(p.partials + t.z * sliceStride + (size_t)m * p.N + n) =
-              floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-      }
-    }
-  }
+      for (int g = 0; g < 4; g++)
+        *reinterpret_cast<floatx4*>(mine + t.z * sliceStride + slot(i, j, g)) =
+            floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
   __syncthreads();
+  uint32_t* counter = p.arrivals + t.y * p.stage.d.grid.x + t.x;
   if (threadIdx.x == 0) {
-    uint32_t* counter = p.arrivals + t.y * p.stage.d.grid.x + t.x;
-    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    // release only: an acquire here would empty this XCD's L2 once per slice; the finishing slice acquires below
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     const bool last = before == p.splitK - 1;
     if (last) dev::storeRelaxed(counter, 0);
     *sLast = last;
@@ -188,10 +205,22 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   __syncthreads();
   if (!*sLast) return false;
   dev::acquireFence();
-  storeFinal([&](int, int, int, uint32_t m, uint32_t n) {
+  // The slice that arrived last adds the slices in index order, eight loads of a position in flight at a time.
+  // (Accumulating into `acc` inside a loop over the slices makes the compiler spill in the main loop.  Letting
+  // all slices wait for each other and add up a share each was measured and is slower: every waiting slice
+  // ends with an acquire that empties its XCD's L2 under the workgroups still streaming weights; the GPT-3
+  // MLP at one row went from 108 to 156 us.)
+  storeFinal([&](int i, int j, int g) {
+    const float* src = mine + slot(i, j, g);
     floatx4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (uint32_t z = 0; z < p.splitK; z++)
-      sum += *reinterpret_cast<const floatx4*>(p.partials + z * sliceStride + (size_t)m * p.N + n);
+    for (uint32_t z0 = 0; z0 < p.splitK; z0 += 8) {
+      floatx4 v[8];
+#pragma unroll
+      for (uint32_t u = 0; u < 8; u++) v[u] = *reinterpret_cast<const floatx4*>(src + min(z0 + u, p.splitK - 1) * sliceStride);
+#pragma unroll
+      for (uint32_t u = 0; u < 8; u++)
+        if (z0 + u < p.splitK) sum = (z0 + u == 0) ? v[u] : sum + v[u];
+    }
     return sum;
   });
   return true;

@@ -70,6 +70,8 @@ TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
   CUSYNC_TILE_DMA(256, 128, 32, 2, 2, 3, 2),   // CUSYNC_TILE_256x128x32: direct-to-LDS, 3 stages, two workgroups per CU
   CUSYNC_TILE_DMA(128, 256, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x256x32
   CUSYNC_TILE_DMA(128, 128, 32, 2, 2, 3, 3),   // CUSYNC_TILE_128x128x32: three workgroups per CU
+  CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x192x32: 6144 and 12288 columns are 32 and 64 tiles
+  CUSYNC_TILE_DMA(256, 192, 32, 2, 2, 3, 1),   // CUSYNC_TILE_256x192x32
 };
 
 std::mutex g_mutex;
@@ -137,14 +139,14 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   if (!ti) { setError("gemm: unknown tile id"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->M == 0 || a->N == 0 || a->K == 0) { setError("gemm: empty problem"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->K % 8 || a->N % 8) { setError("gemm: K and N must be multiples of 8 (16-byte loads)"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if (a->lda % 8 || a->ldb % 8 || a->ldd % 4) { setError("gemm: leading dimensions must keep 16-byte alignment"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->lda % 8 || a->ldb % 8 || a->ldd % 8) { setError("gemm: leading dimensions must keep 16-byte alignment"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const uint32_t aCols = a->a_mode == CUSYNC_A_SWIGLU ? 2 * a->K : a->K;
   if (a->lda < aCols || a->ldb < a->N || a->ldd < a->N) { setError("gemm: leading dimension smaller than the row"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if ((uint64_t)a->M * a->lda * 2 >= 0x80000000ull || (uint64_t)a->K * a->ldb * 2 >= 0x80000000ull) {
     setError("gemm: operand larger than 2 GiB is not addressable by one buffer descriptor");
     return CUSYNC_ERROR_NOT_INITIALIZED;
   }
-  if (((uintptr_t)a->A | (uintptr_t)a->B) % 16 || (uintptr_t)a->D % 8) { setError("gemm: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (((uintptr_t)a->A | (uintptr_t)a->B | (uintptr_t)a->D) % 16) { setError("gemm: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->a_mode == CUSYNC_A_SWIGLU && !ti->kernel[1]) { setError("gemm: this tile shape has no SwiGLU variant"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->split_k < 1) { setError("gemm: split_k must be at least 1"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->split_k > 1) {
@@ -174,10 +176,11 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   return CUSYNC_SUCCESS;
 }
 
-// [split_k][m-tiles*BM][N] fp32 partial sums, then one arrival counter per output tile.
+// [split_k][m-tiles][n-tiles][BM*BN] fp32 partial sums (each tile in the order its workgroup holds it in
+// registers), then one arrival counter per output tile.
 static size_t partialBytes(const cusync_gemm_args* a, const TileInfo* ti) {
   const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
-  return (size_t)a->split_k * g.y * ti->bm * a->N * sizeof(float);
+  return (size_t)a->split_k * g.y * g.x * ti->bm * ti->bn * sizeof(float);
 }
 
 size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {

@@ -43,12 +43,13 @@ struct DmaCfg {
   static constexpr int A_STAGE = BM * A_ROW_BYTES, B_STAGE = B_ROWS * B_ROW_BYTES;
   static constexpr int A_LOADS = A_STAGE / 1024 / 4, B_LOADS = B_STAGE / 1024 / 4;   // per wave per chunk
   static constexpr int LOADS = A_LOADS + B_LOADS;
-  static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES, B_ROWS_PER_LOAD = 1024 / B_ROW_BYTES;
+  static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES;
   static constexpr int LDS_BYTES = STAGES * (A_STAGE + B_STAGE);
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile is made of 32x32 MFMA tiles");
   static_assert(A_CPR == 4 || A_CPR == 8, "BK is 32 or 64");
   static_assert(BT || B_CPR % 8 == 0, "a B row covers whole 128-byte bank sweeps");
+  static_assert(BT || WTN % 32 == 0, "MFMA tiles of B start on 64-byte groups");
   static_assert(A_STAGE % 4096 == 0 && B_STAGE % 4096 == 0, "whole 1 KiB loads per wave");
   static_assert(LDS_BYTES * WAVES_PER_SIMD <= 160 * 1024, "fits the LDS of one CU");
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
@@ -96,13 +97,19 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   constexpr int A_SWZ_DIV = 8 / C::A_CPR;                     // rows that share a swizzle value
   const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + lane / C::A_CPR;
   const uint32_t aLoadChunk = (lane % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
-  // B: load q fills rows (wave*B_LOADS + q)*B_ROWS_PER_LOAD + lane/B_CPR, slot lane%B_CPR.
-  // With B given k-contiguous ([N][K]) its stage is laid out and swizzled exactly like A's.
-  const uint32_t bLoadRow = wave * C::B_LOADS * C::B_ROWS_PER_LOAD + lane / C::B_CPR;
-  const uint32_t bLoadChunk = C::BT ? (lane % C::B_CPR) ^ ((bLoadRow / A_SWZ_DIV) & (C::B_CPR - 1))
-                                    : (lane % C::B_CPR) ^ (4 * (bLoadRow & 1));
+  // B: the 16-byte slots of a stage are numbered row by row; load q of this wave fills slots
+  // (wave*B_LOADS + q)*64 + lane, i.e. row slot / B_CPR, position slot % B_CPR (a row need not be a
+  // power of two long: 192 columns are 24 slots).  With B given k-contiguous ([N][K]) its stage is laid
+  // out and swizzled exactly like A's.
+  uint32_t bLoadRow[C::B_LOADS], bLoadChunk[C::B_LOADS];
+#pragma unroll
+  for (int q = 0; q < C::B_LOADS; q++) {
+    const uint32_t slot = (wave * C::B_LOADS + q) * 64 + lane;
+    bLoadRow[q] = slot / C::B_CPR;
+    const uint32_t pos = slot % C::B_CPR;
+    bLoadChunk[q] = C::BT ? pos ^ ((bLoadRow[q] / A_SWZ_DIV) & (C::B_CPR - 1)) : pos ^ (4 * (bLoadRow[q] & 1));
+  }
   static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
-  static_assert(C::B_ROWS_PER_LOAD % (C::BT ? A_SWZ_DIV * C::A_CPR : 2) == 0, "swizzle repeats per load");
 
   // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
   // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
@@ -116,11 +123,13 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   }
   // B fragment: transpose read of rows kk*16 + 8*(lane/32) + 4*t + (lane&15)/4,
   // 4 halfs at column wn*WTN + j*32 + 16*((lane/16)&1) + 4*(lane&3).
+  // A stage row is kept as 64-byte groups; the group of MFMA tile j is swapped with its neighbour on odd rows.
   const uint32_t bFlip = (lane >> 2) & 1;                      // parity of the row this lane reads
   const uint32_t bRowOff = (8 * (lane >> 5) + ((lane & 15) >> 2)) * C::B_ROW_BYTES;
-  const uint32_t bColOff = (wn * (C::WTN / 8) + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 + (lane & 1) * 8;
-  const uint32_t bFragEven = bRowOff + bColOff + 64 * bFlip;  // MFMA tiles j = 0, 2, ...: slot group j ^ flip
-  const uint32_t bFragOdd = bRowOff + bColOff - 64 * bFlip;   // MFMA tiles j = 1, 3, ...
+  const uint32_t bInGroup = (2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 + (lane & 1) * 8;
+  uint32_t bFrag[C::TN];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++) bFrag[j] = bRowOff + (((wn * C::TN + j) ^ bFlip) * 64) + bInGroup;
   // k-contiguous B: same addressing as the A fragment, rows are output columns.
   uint32_t bFragT[C::KS];
   {
@@ -167,10 +176,13 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     // Per-tile byte offsets of this lane's loads at k0 = 0.
     const uint32_t aVoff0 = ((m0 + aLoadRow) * p.lda + aLoadChunk * 8) * 2;
     const uint32_t aVstep = C::A_ROWS_PER_LOAD * p.lda * 2;
-    const bool bInRange = C::BT ? true : n0 + bLoadChunk * 8 < p.N;
-    const uint32_t bVoff0 = C::BT ? ((n0 + bLoadRow) * p.ldb + bLoadChunk * 8) * 2     // rows past N fall outside the buffer
-                                  : (bLoadRow * p.ldb + n0 + bLoadChunk * 8) * 2;
-    const uint32_t bVstep = C::B_ROWS_PER_LOAD * p.ldb * 2;
+    // B offsets at k0 = 0; columns (or, k-contiguous, rows) outside the matrix are sent out of range.
+    uint32_t bVoff0[C::B_LOADS];
+#pragma unroll
+    for (int q = 0; q < C::B_LOADS; q++) {
+      if constexpr (C::BT) bVoff0[q] = ((n0 + bLoadRow[q]) * p.ldb + bLoadChunk[q] * 8) * 2;     // rows past N fall outside the buffer
+      else bVoff0[q] = n0 + bLoadChunk[q] * 8 < p.N ? (bLoadRow[q] * p.ldb + n0 + bLoadChunk[q] * 8) * 2 : kOutOfRange;
+    }
 
     // Convolution: the pixel each of this lane's A rows stands for.
     int32_t cvIh0[C::A_LOADS], cvIw0[C::A_LOADS];
@@ -255,8 +267,8 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       if constexpr (Q < C::B_LOADS) {
         const uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
         uint32_t off;
-        if constexpr (C::BT) off = k0 + bLoadChunk * 8 < kEnd ? bVoff0 + k0 * 2 + Q * bVstep : kOutOfRange;
-        else off = (bInRange && k0 < kEnd) ? bVoff0 + k0 * p.ldb * 2 + Q * bVstep : kOutOfRange;
+        if constexpr (C::BT) off = k0 + bLoadChunk[Q] * 8 < kEnd ? bVoff0[Q] + k0 * 2 : kOutOfRange;
+        else off = (bVoff0[Q] != kOutOfRange && k0 < kEnd) ? bVoff0[Q] + k0 * p.ldb * 2 : kOutOfRange;
         loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), off);
       } else {
         constexpr int QA = Q - C::B_LOADS;
@@ -283,8 +295,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     auto compute = [&](auto SP, auto SLP, uint32_t ktLoad) {
       constexpr int S = decltype(SP)::value;
       const char* sa = smem + S * C::A_STAGE;
-      const char* sbE = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE + bFragEven;
-      const char* sbO = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE + bFragOdd;
+      const char* sb = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE;
       half8 fa[2][C::TM], fb[2][C::TN];
       constexpr int R = C::TM + C::TN;                 // fragment loads per k-step (a B fragment is two reads)
       // Fragment f of a k-step: f < TM is A tile f, otherwise B tile f - TM.
@@ -299,7 +310,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
             return;
           }
           typedef short4v __attribute__((address_space(3))) * lds_ptr;
-          const char* q = ((J & 1) ? sbO : sbE) + J * 64 + kk * 16 * C::B_ROW_BYTES;
+          const char* q = sb + bFrag[J] + kk * 16 * C::B_ROW_BYTES;
           short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
           short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * C::B_ROW_BYTES));
           half4 l4 = __builtin_bit_cast(half4, lo), h4 = __builtin_bit_cast(half4, hi);
@@ -371,8 +382,11 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
     }
 
+    // The loads issued for chunks past the end of K (zeros) may still be on their way into LDS, which the
+    // epilogue is about to reuse.
+    waitVmcnt<0>();
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
-    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
+    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
 
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.

@@ -256,9 +256,11 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     }
 
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
-    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast);
+    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, t.z};
-    if (completed) stage.post(done);    // barrier inside when the stage is a producer (the decision is workgroup-uniform)
+    // the post's barrier (or this one) keeps the next tile's LDS writes behind the epilogue's LDS reads
+    if (completed && stage.isProducer()) stage.post(done);
+    else __syncthreads();
   }
 }
 

@@ -190,7 +190,9 @@ enum {
   CUSYNC_TILE_256x128x32 = 8,
   CUSYNC_TILE_128x256x32 = 9,
   CUSYNC_TILE_128x128x32 = 10,
-  CUSYNC_TILE_COUNT = 11
+  CUSYNC_TILE_128x192x32 = 11,       /* direct-to-LDS; 6144 = 32 x 192, 12288 = 64 x 192: whole waves on 256 CUs */
+  CUSYNC_TILE_256x192x32 = 12,
+  CUSYNC_TILE_COUNT = 13
 };
 
 typedef struct cusync_gemm_args {

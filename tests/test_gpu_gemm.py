@@ -44,6 +44,7 @@ def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups
         assert L.cusync_rt_device_sync() == 0, api.last_error()
     state = st.read_state()
     assert state.tile_counter == 0       # dispenser re-armed
+    assert state.spin_timeouts == 0      # no k-slice gave up waiting for its siblings
     st.destroy()
     return to_host(dd)
 
