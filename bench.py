@@ -178,6 +178,55 @@ def main():
                 "roofline_frac": round(ideal_us(b) / best, 4),
             })
 
+    # ---- the other chains of the benchmark set: self-attention and the convolution pair --------
+    other = {}
+    if not args.no_sweep:
+        other["attention"] = []
+        heads, e = 12, 12 * 128
+        g = torch.Generator(device="cuda").manual_seed(4)
+        wqkv = (torch.randn((HIDDEN, 3 * e), device="cuda", generator=g) * 0.02).half()
+        wo = (torch.randn((e, HIDDEN), device="cuda", generator=g) * 0.02).half()
+        for seq in (256, 512, 1024, 2048):
+            x = x_all[:seq]
+            qkv = torch.empty((seq, 3 * e), dtype=torch.float16, device="cuda")
+            o = torch.empty((seq, e), dtype=torch.float16, device="cuda")
+            y = torch.empty((seq, HIDDEN), dtype=torch.float16, device="cuda")
+            torch.cuda.synchronize()
+            row = {"S": seq}
+            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE),
+                               ("consecutivesync", api.SYNC.STRIDED)):
+                layer = api.AttnLayer(seq, HIDDEN, heads, sync, wqkv.data_ptr(), wo.data_ptr())
+                layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=10)
+                t, st = layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=20, stages=True)
+                if any(layer.stage_state(i).spin_timeouts for i in range(3)):
+                    sys.exit("bench.py: attention chain waits timed out — results invalid")
+                row[name + "_us"] = round(trimmed(t)[0], 2)
+                if sync == api.SYNC.STREAM:
+                    row["stage_us"] = [round(trimmed([v[i] for v in st])[0], 2) for i in range(3)]
+                    row["tiles"] = list(layer.tiles())
+                layer.destroy()
+            best = min(row[k] for k in ("rowsync_us", "tilesync_us", "consecutivesync_us"))
+            row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)
+            other["attention"].append(row)
+        other["conv_pair"] = []
+        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128)):
+            xc = (torch.rand((n, hh, ww, cc), device="cuda", generator=g) * 2 - 1).half()
+            ws = [(torch.randn((cc, 3, 3, cc), device="cuda", generator=g) * (2.0 / (9 * cc)) ** 0.5).half() for _ in range(2)]
+            ys = [torch.empty((n, hh, ww, cc), dtype=torch.float16, device="cuda") for _ in range(2)]
+            torch.cuda.synchronize()
+            row = {"shape": [n, hh, ww, cc], "gflop": round(2 * 2.0 * n * hh * ww * cc * 9 * cc / 1e9, 2)}
+            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):
+                ch = api.ConvChain(n, hh, ww, cc, [w.data_ptr() for w in ws], sync)
+                ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=10)
+                t = ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=20)
+                if any(ch.stage_state(i).spin_timeouts for i in range(2)):
+                    sys.exit("bench.py: convolution chain waits timed out — results invalid")
+                row[name + "_us"] = round(trimmed(t)[0], 2)
+                row["tile"] = ch.tile()
+                ch.destroy()
+            row["gain_pct"] = round(100 - min(row["rowsync_us"], row["tilesync_us"]) / row["stream_us"] * 100, 2)
+            other["conv_pair"].append(row)
+
     # ---- the timed step: B = args.batch under the better CuSync policy ----------
     cand = {}
     for name, sync in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):
@@ -217,6 +266,7 @@ def main():
         "tflops": round(mlp_flops(B) / statistics.fmean(step_times) / 1e6, 1),
         "roofline": roof,
         "per_batch": per_batch,
+        "other_chains": other,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x_host, w1_host, w2_host)

@@ -152,8 +152,10 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   // cover the device, 128x256 from 2048 rows on.
   const int small = cfg->seq <= 32 ? CUSYNC_TILE_32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : dflt;
-  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : dflt;
+  // widths that are multiples of 192 (4608 = 24 x 192, 12288 = 64 x 192) fill whole rounds with 128x192 tiles
+  const int wide = cfg->seq > 512 ? CUSYNC_TILE_128x192x32 : dflt;
+  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide : dflt;
+  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide : dflt;
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
     setError("attn layer: unknown tile id");

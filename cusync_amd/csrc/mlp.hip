@@ -44,9 +44,14 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   else if (c.batch <= 64) small = CUSYNC_TILE_64x128x64;
   else small = CUSYNC_TILE_128x128x64;
   const bool big = c.batch > 128;
-  // measured on the GPT-3 shard: 128x128 wins up to 512 rows (more tiles to spread), 128x256 from 2048 on
+  // measured on the GPT-3 shard: 128x128 wins up to 512 rows (more tiles to spread), 128x256 from 2048 on;
+  // where the width is a multiple of 192, 128x192 beats both above 512 rows (6144 and 12288 columns are 32
+  // and 64 tiles: whole rounds on 256 CUs at two workgroups each)
+  const uint32_t n1 = c.model == CUSYNC_MLP_LLAMA ? 2 * c.inner : c.inner, n2 = c.hidden;
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
+  if (c.batch > 512 && n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
+  if (c.batch > 512 && n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
   if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
