@@ -29,8 +29,8 @@ BATCHES = [1, 16, 64, 256, 512, 1024, 2048]
 PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes one GEMM launch of the B = 2048 step moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by
-# a plain copy of known size (profiles/gemm_dma_128x256x32_gpt3_mlp_b2048.md).
-TRAFFIC_BYTES_PER_LAUNCH = 845e6
+# a plain copy of known size (profiles/gemm_dma_128x192x32_gpt3_mlp_b2048.md).
+TRAFFIC_BYTES_PER_LAUNCH = 877e6
 
 
 def trimmed(times):
@@ -87,6 +87,8 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the leg that times the dominant kernel (stream-ordered GEMM1/GEMM2 at --batch) "
                          "plus a plain copy of known size; used under rocprofv3 so its per-kernel averages match")
+    ap.add_argument("--profile-chain", choices=["attention", "conv"], default=None,
+                    help="run only the stream-ordered attention chain (S = 2048) or convolution pairs, for rocprofv3")
     ap.add_argument("--tile1", type=int, default=-1)
     ap.add_argument("--tile2", type=int, default=-1)
     args = ap.parse_args()
@@ -149,6 +151,41 @@ def main():
                 "kernel": "gemmDmaKernel/gemmKernel tile %dx%dx%d (mean of GEMM1 %.1f us and GEMM2 %.1f us, stream-ordered, "
                           "%.1f GFLOP per launch)" % (tm, tn, tk, statistics.fmean(g1), statistics.fmean(g2), flops_per_launch / 1e9),
                 }, trimmed(t_s)[0], tiles
+
+    if args.profile_chain == "attention":
+        heads, e, seq = 12, 12 * 128, 2048
+        g = torch.Generator(device="cuda").manual_seed(4)
+        wqkv = (torch.randn((HIDDEN, 3 * e), device="cuda", generator=g) * 0.02).half()
+        wo = (torch.randn((e, HIDDEN), device="cuda", generator=g) * 0.02).half()
+        qkv = torch.empty((seq, 3 * e), dtype=torch.float16, device="cuda")
+        o = torch.empty((seq, e), dtype=torch.float16, device="cuda")
+        y = torch.empty((seq, HIDDEN), dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()
+        layer = api.AttnLayer(seq, HIDDEN, heads, api.SYNC.STREAM, wqkv.data_ptr(), wo.data_ptr())
+        layer.run(x_all[:seq].data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=args.warmup)
+        t, st = layer.run(x_all[:seq].data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=max(10, args.steps), stages=True)
+        print(json.dumps({"metric": "attention chain, stream-ordered, S=2048", "chain_us": round(trimmed(t)[0], 2),
+                          "stage_us": [round(trimmed([v[i] for v in st])[0], 2) for i in range(3)], "tiles": list(layer.tiles()),
+                          "attention_gflop": round(4.0 * seq * seq * 128 * heads / 2 / 1e9, 2)}))
+        layer.destroy()
+        return
+    if args.profile_chain == "conv":
+        g = torch.Generator(device="cuda").manual_seed(4)
+        rows = []
+        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128)):
+            xc = (torch.rand((n, hh, ww, cc), device="cuda", generator=g) * 2 - 1).half()
+            ws = [(torch.randn((cc, 3, 3, cc), device="cuda", generator=g) * (2.0 / (9 * cc)) ** 0.5).half() for _ in range(2)]
+            ys = [torch.empty((n, hh, ww, cc), dtype=torch.float16, device="cuda") for _ in range(2)]
+            torch.cuda.synchronize()
+            ch = api.ConvChain(n, hh, ww, cc, [w.data_ptr() for w in ws], api.SYNC.STREAM)
+            ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=args.warmup)
+            t, per = ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=max(10, args.steps), layers=True)
+            rows.append({"shape": [n, hh, ww, cc], "pair_us": round(trimmed(t)[0], 2),
+                         "layer_us": [round(trimmed([v[i] for v in per])[0], 2) for i in range(2)], "tile": ch.tile(),
+                         "gflop_per_layer": round(2.0 * n * hh * ww * cc * 9 * cc / 1e9, 2)})
+            ch.destroy()
+        print(json.dumps({"metric": "convolution pairs, stream-ordered", "rows": rows}))
+        return
 
     B = args.batch
     if args.roofline_only:
