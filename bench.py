@@ -264,6 +264,15 @@ def main():
             row["gain_pct"] = round(100 - min(row["rowsync_us"], row["tilesync_us"]) / row["stream_us"] * 100, 2)
             other["conv_pair"].append(row)
 
+        # cost of the synchronisation itself (src/examples/sync-overhead/sync-overhead.cu and a ping-pong)
+        with_sync, without = api.sync_overhead_pair(1280, 128, warmup=10, iters=100)
+        other["sync_overhead"] = {
+            "pair_with_sync_us": round(with_sync, 2), "pair_without_sync_us": round(without, 2),
+            "pair_overhead_pct": round((with_sync - without) / without * 100, 1),
+            "handover_ns_same_xcd": round(api.sync_overhead_pingpong(8) / 2, 1),
+            "handover_ns_other_xcd": round(api.sync_overhead_pingpong(1) / 2, 1),
+        }
+
     # ---- the timed step: B = args.batch under the better CuSync policy ----------
     cand = {}
     for name, sync in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):

@@ -332,6 +332,23 @@ class AttnLayer:
             self.h = None
 
 
+# ---- cost of the synchronisation itself ---------------------------------------------
+
+def sync_overhead_pair(blocks=1280, threads=128, warmup=10, iters=100):
+    """(with_sync_us, without_sync_us) of the reference's sync-overhead example
+    (src/examples/sync-overhead/sync-overhead.cu:70-104; its grid is 80*2*(1024/128) = 1280 blocks of 128)."""
+    a, b = C.c_double(0), C.c_double(0)
+    check(_lib.load().cusync_sync_overhead_pair(blocks, threads, warmup, iters, C.byref(a), C.byref(b)), "sync_overhead_pair")
+    return a.value, b.value
+
+
+def sync_overhead_pingpong(partner, rounds=2000):
+    """Nanoseconds per post -> wait -> post -> wait round trip between workgroup 0 and workgroup `partner`."""
+    t = C.c_double(0)
+    check(_lib.load().cusync_sync_overhead_pingpong(partner, rounds, C.byref(t)), "sync_overhead_pingpong")
+    return t.value
+
+
 # ---- MLP chain -------------------------------------------------------------------
 
 class Mlp:

@@ -388,6 +388,21 @@ const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 
 int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
 int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 
+/* ------------------------------------------------------------------------- */
+/* Cost of the synchronisation itself (src/examples/sync-overhead/sync-overhead.cu) */
+/* ------------------------------------------------------------------------- */
+
+/* The example's experiment (sync-overhead.cu:40-105): a producer kernel that writes one value per thread and a
+ * consumer kernel that adds one to it, `blocks` x `threads`, timed from the host over `iters` runs after `warmup`:
+ * once with CuStage tile/post/wait per block on two streams, once stream-ordered without any of it.
+ * Overhead in percent = (with - without) / without * 100 (:104). */
+cusync_error cusync_sync_overhead_pair(uint32_t blocks, uint32_t threads, int warmup, int iters,
+                                       double *with_sync_us, double *without_sync_us);
+/* Latency of a post -> wait hand-over: workgroup 0 and workgroup `partner` (1..63) of one launch pass a
+ * semaphore back and forth `rounds` times.  Workgroups go to the eight XCDs round-robin, so partner 8 shares
+ * workgroup 0's XCD and partner 1 does not.  No counterpart in the reference, whose GPUs have one L2. */
+cusync_error cusync_sync_overhead_pingpong(uint32_t partner, uint32_t rounds, double *ns_per_round_trip);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,28 @@
+"""The sync-overhead experiment of the reference (src/examples/sync-overhead/sync-overhead.cu) and the
+post -> wait hand-over latency between workgroups on the same and on different XCDs."""
+import pytest
+
+from cusync_amd import api
+
+pytestmark = pytest.mark.gpu
+
+
+def test_sync_overhead_pair_runs():
+    # the example's grid: 80 * 2 * (1024 / 128) blocks of 128 threads (sync-overhead.cu:69-71)
+    with_sync, without = api.sync_overhead_pair(1280, 128, warmup=5, iters=30)
+    print("pair: with sync %.1f us, without %.1f us, overhead %.1f %%" % (with_sync, without, (with_sync - without) / without * 100))
+    assert 0 < without < 1e4 and 0 < with_sync < 1e4
+
+
+@pytest.mark.parametrize("partner", [1, 7, 8, 9, 63])
+def test_pingpong_terminates_with_sane_latency(partner):
+    ns = api.sync_overhead_pingpong(partner, rounds=500)
+    print("partner %d: %.0f ns per round trip" % (partner, ns))
+    assert 100 < ns < 100000      # a round trip is two hand-overs through the coherent level of the memory system
+
+
+def test_pingpong_rejects_bad_arguments():
+    with pytest.raises(api.CuSyncError):
+        api.sync_overhead_pingpong(0)
+    with pytest.raises(api.CuSyncError):
+        api.sync_overhead_pingpong(64)
