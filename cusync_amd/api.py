@@ -363,6 +363,23 @@ class Mlp:
         if not self.h:
             raise RuntimeError("cusync_mlp_create failed: " + last_error())
 
+    @classmethod
+    def from_db(cls, entry, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, activation=1):
+        """Builds the chain from one entry of a tile table in the reference's schema
+        (src/ml-bench/transformer/tile_sizes_db.py; cusync_amd/tile_sizes_db.py is written by cusync_amd.tuner)."""
+        key = {SYNC.STREAM: "baseline", SYNC.ROW: "rowsync", SYNC.TILE: "tilesync", SYNC.STRIDED: "tilesync"}[sync]
+        cfg = entry[key]
+        opts = -1
+        if key == "tilesync":
+            opts = ((OPT.AVOID_CUSTOM_ORDER if cfg.get("AvoidCustomOrder") else 0) |
+                    (OPT.AVOID_WAIT_KERNEL if cfg.get("AvoidWaitKernel") else 0) |
+                    (OPT.REORDER_TILE_LOADS if cfg.get("ReorderTileLoads") else 0) |
+                    (OPT.NO_ATOMIC_ADD if cfg.get("NoAtomicAdd") and sync == SYNC.TILE else 0))
+        t1, t2 = entry["TileIds"]
+        k1, k2 = cfg["split_ks"]
+        return cls(model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=t1, tile2=t2, opts=opts,
+                   activation=activation, split_k1=k1, split_k2=k2)
+
     def run(self, x_ptr, h_ptr, y_ptr, runs=1, split=False):
         times = (C.c_double * runs)()
         if split:

@@ -50,8 +50,13 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   const uint32_t n1 = c.model == CUSYNC_MLP_LLAMA ? 2 * c.inner : c.inner, n2 = c.hidden;
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  if (c.batch > 512 && n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
-  if (c.batch > 512 && n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
+  // (the per-batch tuner, cusync_amd/tuner.py, found the same tile best at 256 rows — with 4 and 2 k-slices —
+  // and 128x128 at 512 rows)
+  const bool wide = big && (c.batch <= 384 || c.batch > 768);
+  // GEMM1 keeps 128x256 above 1024 rows: at 2048 rows 128x192 makes 512 tiles, one per slot, and leaves a
+  // consumer launched next to it nowhere to start
+  if (wide && c.batch <= 1024 && n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
+  if (wide && n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
   if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
