@@ -55,13 +55,13 @@ class ConvChainConfig(C.Structure):
 
 
 class AttentionArgs(C.Structure):
-    _fields_ = [("stage", StageDesc), ("seq", u32), ("heads", u32), ("head_dim", u32), ("qkv", vp), ("ldqkv", u32),
+    _fields_ = [("stage", StageDesc), ("seq", u32), ("heads", u32), ("head_dim", u32), ("cached_rows", u32), ("qkv", vp), ("ldqkv", u32),
                 ("out", vp), ("ldo", u32), ("scale", C.c_float), ("causal", i32), ("max_workgroups", i32)]
 
 
 class AttnLayerConfig(C.Structure):
     _fields_ = [("seq", u32), ("hidden", u32), ("heads", u32), ("head_dim", u32), ("sync", i32),
-                ("tile1", i32), ("tile3", i32), ("opts", i32), ("causal", i32)]
+                ("tile1", i32), ("tile3", i32), ("opts", i32), ("causal", i32), ("cached_rows", u32)]
 
 
 class MlpConfig(C.Structure):

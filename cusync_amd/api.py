@@ -270,10 +270,10 @@ def attention_grid(seq, heads):
     return _lib.load().cusync_attention_grid(seq, heads).tup()
 
 
-def attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, head_dim=128, scale=0.0, causal=True, max_workgroups=0):
+def attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, head_dim=128, scale=0.0, causal=True, max_workgroups=0, cached_rows=0):
     a = AttentionArgs()
     a.stage = stage.desc
-    a.seq, a.heads, a.head_dim = seq, heads, head_dim
+    a.seq, a.heads, a.head_dim, a.cached_rows = seq, heads, head_dim, cached_rows
     a.qkv, a.ldqkv, a.out, a.ldo = qkv, ldqkv, out, ldo
     a.scale, a.causal, a.max_workgroups = scale, int(causal), max_workgroups
     return a
@@ -303,9 +303,10 @@ class AttnLayer:
     """Handle over cusync_attn_layer_*: X Wqkv -> fused attention -> O Wo, stream-ordered or as three
     CuSync stages (the chain of src/ml-bench/transformer/attention.cu:702-830)."""
 
-    def __init__(self, seq, hidden, heads, sync, wqkv_ptr, wo_ptr, head_dim=128, tile1=-1, tile3=-1, opts=-1, causal=True):
+    def __init__(self, seq, hidden, heads, sync, wqkv_ptr, wo_ptr, head_dim=128, tile1=-1, tile3=-1, opts=-1, causal=True,
+                 cached_rows=0):
         self.L = _lib.load()
-        self.cfg = AttnLayerConfig(seq, hidden, heads, head_dim, sync, tile1, tile3, opts, int(causal))
+        self.cfg = AttnLayerConfig(seq, hidden, heads, head_dim, sync, tile1, tile3, opts, int(causal), cached_rows)
         self.h = self.L.cusync_attn_layer_create(C.byref(self.cfg), wqkv_ptr, wo_ptr)
         if not self.h:
             raise RuntimeError("cusync_attn_layer_create failed: " + last_error())

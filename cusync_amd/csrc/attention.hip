@@ -84,7 +84,7 @@ cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
   if (a->head_dim != (uint32_t)kHD) { setError("attention: head width must be 128"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const uint32_t E = a->heads * kHD;
   if (a->ldqkv < 3 * E || a->ldqkv % 8 || a->ldo < E || a->ldo % 4) { setError("attention: row pitch too small or misaligned"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if ((uint64_t)a->seq * a->ldqkv * 2 >= 0x80000000ull) { setError("attention: QKV larger than 2 GiB is not addressable by one buffer descriptor"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if ((uint64_t)(a->seq + a->cached_rows) * a->ldqkv * 2 >= 0x80000000ull) { setError("attention: QKV larger than 2 GiB is not addressable by one buffer descriptor"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if ((uintptr_t)a->qkv % 16 || (uintptr_t)a->out % 8 || !a->qkv || !a->out) { setError("attention: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const cusync_dim3 g = cusync_attention_grid(a->seq, a->heads);
   const cusync_stage_desc& s = a->stage;
@@ -126,7 +126,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.stage.d = s;
   p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->qkv % 128 == 0 && (a->ldqkv * 2) % 128 == 0 &&
                         (s.in.kind != CUSYNC_POLICY_TILESYNC || (s.in.tileN * 2) % 128 == 0);
-  p.S = a->seq; p.heads = a->heads;
+  p.S = a->seq; p.heads = a->heads; p.cached = a->cached_rows;
   p.qkv = (const half_t*)a->qkv; p.ldq = a->ldqkv;
   p.out = (half_t*)a->out; p.ldo = a->ldo;
   const float scale = a->scale > 0.0f ? a->scale : 1.0f / sqrtf((float)kHD);
@@ -239,12 +239,14 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     cusync_gemm_args a1, a3;
     memset(&a1, 0, sizeof a1); memset(&a3, 0, sizeof a3);
     a1.stage = L->st[0]; a1.M = S; a1.N = 3 * E; a1.K = H;
-    a1.A = x; a1.lda = H; a1.B = L->wqkv; a1.ldb = 3 * E; a1.D = qkv; a1.ldd = 3 * E;
+    a1.A = x; a1.lda = H; a1.B = L->wqkv; a1.ldb = 3 * E; a1.ldd = 3 * E;
+    a1.D = (char*)qkv + (size_t)L->cfg.cached_rows * 3 * E * 2;       // behind the cache rows (attention.cu:289)
     a1.tile = L->tile1; a1.split_k = 1;
     cusync_attention_args a2;
     memset(&a2, 0, sizeof a2);
     a2.stage = L->st[1]; a2.seq = S; a2.heads = L->cfg.heads; a2.head_dim = kHD;
     a2.qkv = qkv; a2.ldqkv = 3 * E; a2.out = o; a2.ldo = E; a2.scale = 0.0f; a2.causal = L->cfg.causal;
+    a2.cached_rows = L->cfg.cached_rows;
     a3.stage = L->st[2]; a3.M = S; a3.N = H; a3.K = E;
     a3.A = o; a3.lda = E; a3.B = L->wo; a3.ldb = H; a3.D = y; a3.ldd = H;
     a3.tile = L->tile3; a3.split_k = 1;

@@ -36,8 +36,9 @@ constexpr float kMasked = -1.0e30f;
 
 struct AttnParams {
   cusync::DynStage stage;
-  uint32_t S, heads;
-  const half_t* qkv; uint32_t ldq;   // [S][ldq]: Q at column 0, K at heads*128, V at 2*heads*128
+  uint32_t S, heads;                 // S query rows (= rows the stage produces)
+  uint32_t cached;                   // rows of qkv in front of the query rows: the key/value cache
+  const half_t* qkv; uint32_t ldq;   // [cached + S][ldq]: Q at column 0, K at heads*128, V at 2*heads*128
   half_t* out; uint32_t ldo;         // [S][ldo]
   float scaleLog2;                   // softmax scale * log2(e)
   uint32_t causal;
@@ -54,7 +55,8 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   const uint32_t hi = lane >> 5;
   const cusync::DynStage& stage = p.stage;
   const uint32_t E = p.heads * kHD;
-  const uint32_t bufBytes = p.S * p.ldq * 2;
+  const uint32_t total = p.cached + p.S;               // key/value rows
+  const uint32_t bufBytes = total * p.ldq * 2;
   const uint4v rLds = rawRsrc(p.qkv, bufBytes);
   const __amdgpu_buffer_rsrc_t rReg = makeRsrc(p.qkv, bufBytes);
   const uint32_t ldsBase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
@@ -117,11 +119,12 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     const cusync_dim3 t = stage.ticketToTile(ticket);
     const uint32_t head = t.x, q0 = t.y * kBQ;
     const uint32_t qEnd = min(q0 + (uint32_t)kBQ, p.S);
-    const uint32_t nkv = p.causal ? qEnd : p.S;
+    const uint32_t nkv = p.causal ? p.cached + qEnd : total;
     const uint32_t nblk = (nkv + kBKV - 1) / kBKV;
     const uint32_t qw = q0 + 32 * wave;                 // first query row of this wave
     const uint32_t myq = qw + (lane & 31);
-    const uint32_t limit = p.causal ? min(myq, p.S - 1) : p.S - 1;   // last kv position this query sees
+    // positions are rows of qkv: query i sits at cached + i and, when causal, sees keys 0 .. cached + i
+    const uint32_t limit = p.causal ? p.cached + min(myq, p.S - 1) : total - 1;   // last kv position this query sees
 
     // Direct loads of block j into stage st.  Rows past the end of the
     // sequence lie outside the buffer and arrive as zeros.
@@ -138,9 +141,11 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
                   (rowOff + q * 4 * p.ldq + 2 * E + head * kHD + vChunk * 8) * 2);
     };
     auto waitKV = [&](uint32_t j) {
-      const uint32_t rowBegin = j * kBKV, rowEnd = min(rowBegin + (uint32_t)kBKV, p.S);
-      waitRows(rowBegin, rowEnd, E + head * kHD);
-      waitRows(rowBegin, rowEnd, 2 * E + head * kHD);
+      // only the rows behind the cache come from the producer; its tiles count rows from there
+      const uint32_t lo = max(j * kBKV, p.cached), hi = min(j * kBKV + (uint32_t)kBKV, total);
+      if (lo >= hi) return;
+      waitRows(lo - p.cached, hi - p.cached, E + head * kHD);
+      waitRows(lo - p.cached, hi - p.cached, 2 * E + head * kHD);
     };
 
     // Q fragments stay in registers for the whole tile: k-step s is head-dim 16s + 8hi .. + 7 of row myq.
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     half8 qf[8];
 #pragma unroll
     for (int s = 0; s < 8; s++)
-      qf[s] = __builtin_bit_cast(half8, loadChunk(rReg, myq < p.S ? (myq * p.ldq + head * kHD + 16 * s + 8 * hi) * 2 : kOutOfRange));
+      qf[s] = __builtin_bit_cast(half8, loadChunk(rReg, myq < p.S ? ((p.cached + myq) * p.ldq + head * kHD + 16 * s + 8 * hi) * 2 : kOutOfRange));
 
     waitKV(0);
     issue(0, 0);
@@ -167,7 +172,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
       __builtin_amdgcn_s_barrier();       // block j is in LDS for everyone; everyone is done with block j-1
       asm volatile("" ::: "memory");
       if (j + 1 < nblk) { waitKV(j + 1); issue(j + 1, st ^ 1); }
-      if (p.causal && j * kBKV > qw + 31) continue;       // wholly in this wave's future (wave-uniform)
+      if (p.causal && j * kBKV > p.cached + qw + 31) continue;       // wholly in this wave's future (wave-uniform)
 
       const char* ks = smem + st * 2 * kStageBytes;
       const char* vs = ks + kStageBytes;
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
 
       // scale, mask, running maximum
       const uint32_t kvBase = j * kBKV + 4 * hi;
-      const bool needMask = j * kBKV + kBKV - 1 > (p.causal ? min(qw, p.S - 1) : p.S - 1);
+      const bool needMask = j * kBKV + kBKV - 1 > (p.causal ? p.cached + min(qw, p.S - 1) : total - 1);
       float blockMax = kMasked;
 #pragma unroll
       for (int a = 0; a < 2; a++)

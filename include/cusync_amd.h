@@ -297,8 +297,10 @@ int cusync_conv_chain_tile(const cusync_conv_chain *chain);
 
 typedef struct cusync_attention_args {
   cusync_stage_desc stage;     /* grid = cusync_attention_grid(seq, heads) */
-  uint32_t seq, heads, head_dim;   /* head_dim must be 128 */
-  const void *qkv;             /* [seq][ldqkv] fp16: Q at column 0, K at heads*head_dim, V at 2*heads*head_dim */
+  uint32_t seq, heads, head_dim;   /* seq query rows; head_dim must be 128 */
+  uint32_t cached_rows;        /* rows of qkv in front of the query rows: the key/value cache of TB/attention.cu:272-276
+                                  (query i sits at row cached_rows + i and sees keys 0 .. cached_rows + i); 0 = none */
+  const void *qkv;             /* [cached_rows + seq][ldqkv] fp16: Q at column 0, K at heads*head_dim, V at 2*heads*head_dim */
   uint32_t ldqkv;
   void *out;                   /* [seq][ldo] fp16, head h in columns h*head_dim .. */
   uint32_t ldo;
@@ -327,6 +329,8 @@ typedef struct cusync_attn_layer_config {
   int32_t tile1, tile3;        /* GEMM tile ids, -1 = built-in choice */
   int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = none */
   int32_t causal;
+  uint32_t cached_rows;        /* key/value cache rows in front of the `seq` new ones (the reference's --seqlen with
+                                  --batch new rows, TB/attention.cu:265-276); qkv then has cached_rows + seq rows */
 } cusync_attn_layer_config;
 
 typedef struct cusync_attn_layer cusync_attn_layer;
@@ -334,7 +338,7 @@ typedef struct cusync_attn_layer cusync_attn_layer;
 /* wqkv: [hidden][3*heads*head_dim], wo: [heads*head_dim][hidden], both fp16 row-major device pointers. */
 cusync_attn_layer *cusync_attn_layer_create(const cusync_attn_layer_config *cfg, const void *wqkv, const void *wo);
 void cusync_attn_layer_destroy(cusync_attn_layer *layer);
-/* x: [seq][hidden]; qkv: [seq][3*heads*head_dim]; o: [seq][heads*head_dim]; y: [seq][hidden].  Runs `runs`
+/* x: [seq][hidden]; qkv: [cached_rows + seq][3*heads*head_dim] (the cache rows filled by the caller); o: [seq][heads*head_dim]; y: [seq][hidden].  Runs `runs`
  * times, synchronising after each; times_us[r] = start of the first kernel to end of the last.  For the
  * stream-ordered mode stage_us[3*r + i] receives the time of stage i. */
 cusync_error cusync_attn_layer_run(cusync_attn_layer *layer, const void *x, void *qkv, void *o, void *y, int runs,

@@ -91,6 +91,8 @@ def lib():
     L.orc_swiglu_f16.argtypes = [u32, u32, vp, u32, vp, u32]
     L.orc_attention_f16.restype = None
     L.orc_attention_f16.argtypes = [u32, u32, u32, vp, u32, vp, u32, i32]
+    L.orc_attention_kv_f16.restype = None
+    L.orc_attention_kv_f16.argtypes = [u32, u32, u32, u32, vp, u32, vp, u32, i32]
     L.orc_conv2d_nhwc_f16.restype = None
     L.orc_conv2d_nhwc_f16.argtypes = [u32] * 9 + [vp, vp, vp, i32]
     L.orc_equals_f16.restype = i32
@@ -228,6 +230,16 @@ def attention(qkv, heads, hd, causal=True):
     S, ld = qkv.shape
     out = np.empty((S, heads * hd), dtype=np.uint16)
     lib().orc_attention_f16(S, heads, hd, _ptr(qkv), ld, _ptr(out), heads * hd, int(causal))
+    return out.view(np.float16)
+
+
+def attention_kv(qkv, cached, heads, hd, causal=True):
+    """Attention of the rows behind `cached` cache rows over all rows of qkv ([cached + S, 3*heads*hd])."""
+    qkv = _h(qkv)
+    total, ld = qkv.shape
+    S = total - cached
+    out = np.empty((S, heads * hd), dtype=np.uint16)
+    lib().orc_attention_kv_f16(S, cached, heads, hd, _ptr(qkv), ld, _ptr(out), heads * hd, int(causal))
     return out.view(np.float16)
 
 

@@ -349,24 +349,28 @@ void orc_swiglu_f16(uint32_t M, uint32_t d, const uint16_t *gu, uint32_t ld_gu,
     }
 }
 
-/* Textbook softmax(mask(Q K^T / sqrt(hd))) V per head, all in fp32. */
-void orc_attention_f16(uint32_t S, uint32_t heads, uint32_t hd,
-                       const uint16_t *qkv, uint32_t ld_qkv,
-                       uint16_t *out, uint32_t ld_out, int causal) {
+/* Textbook softmax(mask(Q K^T / sqrt(hd))) V per head, all in fp32.  The S query rows are rows
+ * cached .. cached+S-1 of qkv; keys and values are rows 0 .. cached+S-1 (rows below `cached` are the
+ * key/value cache of TB/attention.cu:272-276, 289: the projection writes its rows behind `seqlen` cached
+ * ones).  Causal: query i sees keys 0 .. cached+i. */
+void orc_attention_kv_f16(uint32_t S, uint32_t cached, uint32_t heads, uint32_t hd,
+                          const uint16_t *qkv, uint32_t ld_qkv,
+                          uint16_t *out, uint32_t ld_out, int causal) {
   uint32_t D = heads * hd;
   float scale = 1.0f / sqrtf((float)hd);
   #pragma omp parallel for collapse(2)
   for (uint32_t h = 0; h < heads; h++)
     for (uint32_t i = 0; i < S; i++) {
-      float *p = (float *)malloc(sizeof(float) * S);
+      uint32_t total = cached + S;
+      float *p = (float *)malloc(sizeof(float) * total);
       float *o = (float *)calloc(hd, sizeof(float));
-      uint32_t lim = causal ? i + 1 : S;
+      uint32_t lim = causal ? cached + i + 1 : total;
+      const uint16_t *qrow = qkv + (size_t)(cached + i) * ld_qkv + h * hd;
       float mx = -INFINITY;
       for (uint32_t j = 0; j < lim; j++) {
         float s = 0;
         for (uint32_t c = 0; c < hd; c++)
-          s += orc_h2f(qkv[(size_t)i * ld_qkv + h * hd + c]) *
-               orc_h2f(qkv[(size_t)j * ld_qkv + D + h * hd + c]);
+          s += orc_h2f(qrow[c]) * orc_h2f(qkv[(size_t)j * ld_qkv + D + h * hd + c]);
         p[j] = s * scale;
         if (p[j] > mx) mx = p[j];
       }
@@ -380,6 +384,12 @@ void orc_attention_f16(uint32_t S, uint32_t heads, uint32_t hd,
       for (uint32_t c = 0; c < hd; c++) out[(size_t)i * ld_out + h * hd + c] = orc_f2h(o[c]);
       free(p); free(o);
     }
+}
+
+void orc_attention_f16(uint32_t S, uint32_t heads, uint32_t hd,
+                       const uint16_t *qkv, uint32_t ld_qkv,
+                       uint16_t *out, uint32_t ld_out, int causal) {
+  orc_attention_kv_f16(S, 0, heads, hd, qkv, ld_qkv, out, ld_out, causal);
 }
 
 /* Direct 7-loop NHWC forward convolution, cross-correlation, KRSC filters. */

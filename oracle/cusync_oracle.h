@@ -136,6 +136,12 @@ void orc_swiglu_f16(uint32_t M, uint32_t d, const uint16_t *gu, uint32_t ld_gu,
 void orc_attention_f16(uint32_t S, uint32_t heads, uint32_t hd,
                        const uint16_t *qkv, uint32_t ld_qkv,
                        uint16_t *out, uint32_t ld_out, int causal);
+/* Same with a key/value cache: the S query rows are rows cached..cached+S-1 of qkv ([cached+S, 3*heads*hd]),
+ * keys and values rows 0..cached+S-1 (TB/attention.cu:272-276, 289).  Pinned: equals the last S rows of
+ * orc_attention_f16 over all cached+S rows when causal. */
+void orc_attention_kv_f16(uint32_t S, uint32_t cached, uint32_t heads, uint32_t hd,
+                          const uint16_t *qkv, uint32_t ld_qkv,
+                          uint16_t *out, uint32_t ld_out, int causal);
 /* NHWC fprop, KRSC filter, cross-correlation (CV/resnet.cu:678), fp32 accumulate. */
 void orc_conv2d_nhwc_f16(uint32_t N, uint32_t H, uint32_t W, uint32_t C, uint32_t K,
                          uint32_t R, uint32_t S, uint32_t pad, uint32_t stride,

@@ -172,3 +172,70 @@ def test_attention_layer_small(S, tile):
 def test_attention_layer_gpt3_shard(S):
     print("attn layer gpt3", S, flush=True)
     check_layer(S, 12288, 12, sampled=True)
+
+
+# ---- key/value cache variant (src/ml-bench/transformer/attention.cu:265-276, 289) ----------------
+
+def run_attention_kv(qkv, cached, heads, causal=True):
+    import torch
+    L = _lib.load()
+    S = qkv.shape[0] - cached
+    dq = to_dev(qkv)
+    do = empty_dev((S, heads * 128), fill=float("nan"))
+    torch.cuda.synchronize()
+    st = api.Stage(api.attention_grid(S, heads), (1, 1, 1), api.no_sync(), api.no_sync())
+    rc = api.attention(st, S, heads, dq.data_ptr(), qkv.shape[1], do.data_ptr(), heads * 128, causal=causal, cached_rows=cached)
+    assert rc == api.ERR.SUCCESS, api.last_error()
+    assert L.cusync_rt_device_sync() == 0, api.last_error()
+    st.destroy()
+    return to_host(do)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("S,cached,heads", [(1, 1, 1), (1, 2047, 2), (16, 64, 1), (16, 100, 3), (200, 500, 2), (130, 63, 1), (256, 1024, 12)])
+def test_attention_with_cache_matches_oracle(S, cached, heads, causal):
+    print("attention kv", S, cached, heads, causal, flush=True)
+    qkv = normal_f16((cached + S, 3 * heads * 128), 15, std=1.0)
+    got = run_attention_kv(qkv, cached, heads, causal)
+    assert_close(got, orc.attention_kv(qkv, cached, heads, 128, causal), "O")
+    if causal:
+        # the same rows of plain causal attention over the whole sequence, bit for bit
+        full = run_attention(qkv, heads, True)
+        assert np.array_equal(got.view(np.uint16), full[cached:].view(np.uint16))
+
+
+@pytest.mark.parametrize("S,cached", [(16, 512), (64, 1024), (256, 2048), (200, 300)])
+def test_attention_layer_with_cache(S, cached):
+    # the reference's decode-time shape: `batch` new rows behind `seqlen` cached ones; the projection writes
+    # its rows behind the cache and the attention only waits for those
+    import torch
+    print("attn layer kv", S, cached, flush=True)
+    hidden, heads = 12288, 12
+    E = heads * 128
+    wqkv, wo, dwqkv, dwo = layer_weights(hidden, heads)
+    x = uniform_f16((S, hidden), 1)
+    cache = normal_f16((cached, 3 * E), 16, std=1.0)
+    dx = to_dev(x)
+    outs = {}
+    for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE, api.SYNC.STRIDED):
+        dqkv = empty_dev((cached + S, 3 * E), fill=float("nan"))
+        dqkv[:cached] = to_dev(cache)
+        do = empty_dev((S, E), fill=float("nan"))
+        dy = empty_dev((S, hidden), fill=float("nan"))
+        torch.cuda.synchronize()
+        layer = api.AttnLayer(S, hidden, heads, sync, dwqkv.data_ptr(), dwo.data_ptr(), cached_rows=cached)
+        layer.run(dx.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=2)
+        for i in range(3):
+            st = layer.stage_state(i)
+            assert st.spin_timeouts == 0 and st.tile_counter == 0
+        layer.destroy()
+        outs[sync] = (to_host(dqkv), to_host(do), to_host(dy))
+    qkv, o, y = outs[api.SYNC.STREAM]
+    assert np.array_equal(qkv[:cached].view(np.uint16), cache.view(np.uint16))       # the cache rows are untouched
+    rows = sample_rows(S)
+    assert_close(qkv[cached:][rows], orc.gemm(np.ascontiguousarray(x[rows]), wqkv), "new QKV rows")
+    assert_close(o, orc.attention_kv(qkv, cached, heads, 128, True), "O")
+    assert_close(y[rows], orc.gemm(np.ascontiguousarray(o[rows]), wo), "Y rows")
+    for sync in (api.SYNC.ROW, api.SYNC.TILE, api.SYNC.STRIDED):
+        for got, want, name in zip(outs[sync], outs[api.SYNC.STREAM], ("QKV", "O", "Y")):
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (sync, name)

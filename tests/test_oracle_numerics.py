@@ -185,3 +185,20 @@ def test_count_mismatch():
     b = np.array([1.005, 2.1, 0.0009], np.float16)
     bad, mx = orc.count_mismatch(a, b, 1e-2, 1e-3)
     assert bad == 1 and abs(mx - 0.1) < 2e-3
+
+
+def test_attention_with_cache_is_the_tail_of_full_causal_attention():
+    # queries behind a key/value cache see exactly what the same rows see in causal attention over
+    # the whole sequence; without cache rows the two functions are one
+    rng = np.random.default_rng(6)
+    heads, hd = 2, 16
+    for total, cached in ((50, 0), (50, 13), (70, 64), (33, 32)):
+        qkv = rng.uniform(-1, 1, (total, 3 * heads * hd)).astype(np.float16)
+        full = orc.attention(qkv, heads, hd, causal=True)
+        tail = orc.attention_kv(qkv, cached, heads, hd, causal=True)
+        assert np.array_equal(tail.view(np.uint16), full[cached:].view(np.uint16))
+    # not causal: every query sees all rows; permuting the cache rows changes nothing but rounding order
+    qkv = rng.uniform(-1, 1, (40, 3 * heads * hd)).astype(np.float16)
+    a = orc.attention_kv(qkv, 10, heads, hd, causal=False).astype(np.float32)
+    b = orc.attention(qkv, heads, hd, causal=False).astype(np.float32)[10:]
+    assert np.allclose(a, b, atol=1e-3)
