@@ -22,6 +22,7 @@
 #include "../../include/cusync_amd.h"
 #include "rt_internal.h"
 #include "gemm_kernel_dma.h"
+#include "conv3x3_kernel.h"
 
 namespace {
 
@@ -38,11 +39,29 @@ struct ConvTile {
   { BM, BN, BK, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>::LDS_BYTES, \
     gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>, kAConv>, -1 }
 
+using HaloA = Halo3x3Cfg<256, 64, 4, 1, 4, 2>;     // 64 output channels per tile: four waves of 64 x 64 stacked
+using HaloB = Halo3x3Cfg<128, 128, 2, 2, 3, 1>;    // 128 output channels per tile
+
 ConvTile g_convTiles[CUSYNC_CONV_TILE_COUNT] = {
   CUSYNC_CONV_TILE(128, 64, 32, 2, 2, 4, 3),    // CUSYNC_CONV_TILE_128x64x32
   CUSYNC_CONV_TILE(128, 128, 32, 2, 2, 4, 2),   // CUSYNC_CONV_TILE_128x128x32
   CUSYNC_CONV_TILE(256, 64, 32, 4, 1, 3, 2),    // CUSYNC_CONV_TILE_256x64x32
+  // the halo tiles: 3x3 / pad 1 / stride 1 only; LDS size depends on the image width and channels
+  { HaloA::BM, HaloA::BN, HaloA::BK, 0, convHalo3x3Kernel<HaloA>, -1 },   // CUSYNC_CONV_TILE_HALO_256x64x64
+  { HaloB::BM, HaloB::BN, HaloB::BK, 0, convHalo3x3Kernel<HaloB>, -1 },   // CUSYNC_CONV_TILE_HALO_128x128x64
 };
+
+bool isHalo(int tile) { return tile == CUSYNC_CONV_TILE_HALO_256x64x64 || tile == CUSYNC_CONV_TILE_HALO_128x128x64; }
+uint32_t haloLds(int tile, uint32_t W, uint32_t C) {
+  return tile == CUSYNC_CONV_TILE_HALO_256x64x64 ? HaloA::ldsBytes(W, C) : HaloB::ldsBytes(W, C);
+}
+constexpr uint32_t kMaxLds = 160 * 1024 - 1024;      // what one workgroup may ask for (the kernel has 8 bytes of static LDS)
+
+// The halo kernel needs 3x3, pad 1, stride 1, a power-of-two channel count of at least 64, and its tile plus
+// halo in LDS.
+bool haloEligible(int tile, uint32_t W, uint32_t C, uint32_t R, uint32_t S, uint32_t pad, uint32_t stride) {
+  return R == 3 && S == 3 && pad == 1 && stride == 1 && C >= 64 && (C & (C - 1)) == 0 && haloLds(tile, W, C) <= kMaxLds;
+}
 
 std::mutex g_convMutex;
 
@@ -52,19 +71,23 @@ ConvTile* convTile(int tile) {
 }
 
 int g_convNumCUs = 0;
+uint32_t g_haloLds[CUSYNC_CONV_TILE_COUNT] = {};      // LDS size the cached occupancy of a halo kernel was computed for
 
-int residentConv(ConvTile* ti) {
+int residentConv(ConvTile* ti, size_t lds) {
   std::lock_guard<std::mutex> lock(g_convMutex);
-  if (ti->residentPerCU < 0) {
+  const int idx = (int)(ti - g_convTiles);
+  const bool halo = isHalo(idx);
+  if (ti->residentPerCU < 0 || (halo && g_haloLds[idx] != lds)) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
     g_convNumCUs = prop.multiProcessorCount;
     if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds))) return 0;
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, halo ? (int)kMaxLds : (int)lds))) return 0;
     int n = 0;
-    if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel, kThreads, ti->lds))) return 0;
+    if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel, kThreads, lds))) return 0;
     ti->residentPerCU = n;
+    if (halo) g_haloLds[idx] = (uint32_t)lds;
   }
   return ti->residentPerCU * g_convNumCUs;
 }
@@ -104,7 +127,11 @@ cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
   if (!a->N || !a->H || !a->W || !a->C || !a->K || !a->R || !a->S || !a->stride) { setError("conv2d: empty problem"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->H + 2 * a->pad < a->R || a->W + 2 * a->pad < a->S) { setError("conv2d: filter larger than the padded image"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->pad >= a->R || a->pad >= a->S) { setError("conv2d: padding must be smaller than the filter"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if (a->C % ti->bk) { setError("conv2d: channels must be a multiple of the K chunk (32)"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->C % ti->bk) { setError("conv2d: channels must be a multiple of the K chunk"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (isHalo(a->tile) && !haloEligible(a->tile, a->W, a->C, a->R, a->S, a->pad, a->stride)) {
+    setError("conv2d: the halo tile needs a 3x3 filter, pad 1, stride 1, a power-of-two channel count >= 64 and its rows plus 2W + 2 pixels in LDS");
+    return CUSYNC_ERROR_NOT_INITIALIZED;
+  }
   if (a->K % 8) { setError("conv2d: output channels must be a multiple of 8"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if ((uint64_t)a->N * a->H * a->W * a->C * 2 >= 0x80000000ull || (uint64_t)a->K * a->R * a->S * a->C * 2 >= 0x80000000ull) {
     setError("conv2d: operand larger than 2 GiB is not addressable by one buffer descriptor");
@@ -133,14 +160,16 @@ cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
 
 int cusync_conv2d_max_resident(int tile) {
   ConvTile* ti = convTile(tile);
-  return ti ? residentConv(ti) : 0;
+  if (!ti) return 0;
+  return residentConv(ti, isHalo(tile) ? haloLds(tile, 56, 64) : ti->lds);     // the halo tiles: for 56 x 56 x 64 images
 }
 
 cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   cusync_error e = cusync_conv2d_can_implement(a);
   if (e != CUSYNC_SUCCESS) return e;
   ConvTile* ti = convTile(a->tile);
-  const int resident = residentConv(ti);
+  const size_t lds = isHalo(a->tile) ? haloLds(a->tile, a->W, a->C) : ti->lds;
+  const int resident = residentConv(ti, lds);
   if (resident <= 0) { cusync::rt::setError("conv2d: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
   const cusync_stage_desc& s = a->stage;
   const uint32_t tiles = s.grid.x * s.grid.y * s.grid.z;
@@ -167,7 +196,7 @@ cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
                         (a->C * 2) % 128 == 0 &&
                         (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
-  hipLaunchKernelGGL(ti->kernel, dim3(launched), dim3(kThreads), ti->lds, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(ti->kernel, dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }
@@ -212,7 +241,10 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
   if (cfg->layers < 1 || cfg->layers > 16) { setError("conv chain: 1 to 16 layers"); return nullptr; }
   cusync_conv_chain* c = new cusync_conv_chain();
   c->cfg = *cfg;
-  if (c->cfg.tile < 0) c->cfg.tile = cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_256x64x32;   // measured on 32x56x56x64 and 32x28x28x128
+  if (c->cfg.tile < 0)
+    c->cfg.tile = cfg->C % 128 == 0 && haloEligible(CUSYNC_CONV_TILE_HALO_128x128x64, cfg->W, cfg->C, 3, 3, 1, 1) ? CUSYNC_CONV_TILE_HALO_128x128x64
+                  : haloEligible(CUSYNC_CONV_TILE_HALO_256x64x64, cfg->W, cfg->C, 3, 3, 1, 1) ? CUSYNC_CONV_TILE_HALO_256x64x64
+                  : cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_256x64x32;
   uint32_t tm = 0, tn = 0;
   if (cusync_conv2d_tile_shape(c->cfg.tile, &tm, &tn, nullptr)) { setError("conv chain: unknown tile id"); delete c; return nullptr; }
   const cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);

@@ -235,7 +235,10 @@ enum {
   CUSYNC_CONV_TILE_128x64x32 = 0,    /* M x K_out x K chunk */
   CUSYNC_CONV_TILE_128x128x32 = 1,
   CUSYNC_CONV_TILE_256x64x32 = 2,
-  CUSYNC_CONV_TILE_COUNT = 3
+  CUSYNC_CONV_TILE_HALO_256x64x64 = 3,   /* 3x3, pad 1, stride 1, C a power of two >= 64: the input tile and its halo
+                                            stay in LDS, each pixel is fetched once instead of once per filter tap */
+  CUSYNC_CONV_TILE_HALO_128x128x64 = 4,
+  CUSYNC_CONV_TILE_COUNT = 5
 };
 
 typedef struct cusync_conv2d_args {

@@ -16,6 +16,17 @@ pytestmark = pytest.mark.gpu
 CONV_TILES = list(range(api.CONV_TILE.COUNT))
 
 
+def fits(tile, Cc, R=3, S=3, pad=1, stride=1, W=8):
+    """The halo tiles only do 3x3 / pad 1 / stride 1 with a power-of-two channel count of at least 64, and
+    need their rows plus 2W + 2 pixels of the image in LDS next to the filter stages."""
+    halo = {api.CONV_TILE.HALO_256x64x64: (256, 4 * 8192), api.CONV_TILE.HALO_128x128x64: (128, 3 * 16384)}
+    if tile not in halo:
+        return True
+    rows, filt = halo[tile]
+    lds = filt + -(-(rows + 2 * W + 2) * Cc * 2 // 1024) * 1024
+    return (R, S, pad, stride) == (3, 3, 1, 1) and Cc >= 64 and Cc & (Cc - 1) == 0 and lds <= 159 * 1024
+
+
 def he_filters(K, R, S, Cc, seed):
     rng = np.random.default_rng(seed)
     return (rng.standard_normal((K, R, S, Cc)) * np.sqrt(2.0 / (R * S * Cc))).astype(np.float16)
@@ -61,8 +72,9 @@ def test_conv_exact_on_integer_data(tile):
     # small integers: sums are exact, so a wrong pixel, channel or filter tap shows up bit-exactly
     print("conv int", tile, flush=True)
     rng = np.random.default_rng(tile)
-    x = rng.integers(-2, 3, (2, 13, 10, 96)).astype(np.float16)
-    w = rng.integers(-2, 3, (40, 3, 3, 96)).astype(np.float16)
+    Cc = 96 if fits(tile, 96) else 128
+    x = rng.integers(-2, 3, (2, 13, 10, Cc)).astype(np.float16)
+    w = rng.integers(-2, 3, (40, 3, 3, Cc)).astype(np.float16)
     got = run_conv(x, w, tile, launches=2)
     want = orc.conv2d_nhwc(x, w)
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
@@ -77,11 +89,14 @@ def test_conv_1x1_reduces_to_gemm():
 
 
 @pytest.mark.parametrize("tile", CONV_TILES)
-@pytest.mark.parametrize("geom", [(2, 12, 12, 64, 64, 3, 3, 1, 1), (3, 7, 9, 32, 72, 3, 3, 1, 1), (1, 15, 15, 64, 136, 5, 5, 2, 1),
+@pytest.mark.parametrize("geom", [(2, 12, 12, 64, 64, 3, 3, 1, 1), (3, 7, 9, 32, 72, 3, 3, 1, 1), (2, 5, 3, 128, 136, 3, 3, 1, 1),
+                                  (1, 1, 1, 64, 8, 3, 3, 1, 1), (3, 30, 200, 64, 64, 3, 3, 1, 1), (1, 9, 7, 256, 72, 3, 3, 1, 1), (1, 15, 15, 64, 136, 5, 5, 2, 1),
                                   (2, 14, 14, 64, 64, 3, 3, 1, 2), (2, 9, 9, 96, 32, 3, 3, 0, 1), (1, 8, 20, 64, 64, 1, 3, 0, 1)])
 def test_conv_matches_oracle(tile, geom):
     print("conv", tile, geom, flush=True)
     N, H, W, Cc, K, R, S, pad, stride = geom
+    if not fits(tile, Cc, R, S, pad, stride, W):
+        pytest.skip("geometry outside the halo tile's domain")
     x = uniform_f16((N, H, W, Cc), 5)
     w = he_filters(K, R, S, Cc, 6)
     got = run_conv(x, w, tile, pad=pad, stride=stride)
@@ -120,6 +135,12 @@ def test_conv_can_implement_rejects():
     assert rc(stride=0) != api.ERR.SUCCESS
     assert rc(epilogue=7) != api.ERR.SUCCESS
     assert "conv2d" in api.last_error()
+    halo = api.CONV_TILE.HALO_256x64x64
+    assert rc(tile=halo) == api.ERR.SUCCESS
+    assert rc(tile=halo, stride=2) != api.ERR.SUCCESS and rc(tile=halo, pad=0) != api.ERR.SUCCESS
+    assert rc(tile=halo, R=1, S=1, pad=0) != api.ERR.SUCCESS
+    assert rc(tile=halo, Cc=96) != api.ERR.SUCCESS              # channels not a power of two
+    assert rc(tile=halo, H=2, W=4096) != api.ERR.SUCCESS        # halo does not fit LDS (and the grid differs)
     st.destroy()
 
 
@@ -178,7 +199,9 @@ def check_chain(res, iters):
 
 @pytest.mark.parametrize("kind,opts", [("conv2dtile", 0), ("conv2dtile", api.OPT.NO_ATOMIC_ADD), ("tile", 0), ("row", 0)])
 @pytest.mark.parametrize("tiles", [(api.CONV_TILE.T128x64x32, api.CONV_TILE.T128x64x32),
-                                   (api.CONV_TILE.T256x64x32, api.CONV_TILE.T128x64x32)])
+                                   (api.CONV_TILE.T256x64x32, api.CONV_TILE.T128x64x32),
+                                   (api.CONV_TILE.HALO_256x64x64, api.CONV_TILE.HALO_256x64x64),
+                                   (api.CONV_TILE.T128x64x32, api.CONV_TILE.HALO_128x128x64)])
 def test_chained_conv_pair_small(kind, opts, tiles):
     print("conv chain", kind, opts, tiles, flush=True)
     check_chain(chained_convs(4, 20, 20, 64, tiles[0], tiles[1], kind, iters=2, opts=opts), 2)
@@ -190,6 +213,7 @@ def test_chained_conv_pair_two_channel_tiles(kind):
     # not for (k/64)/(R*S) as the reference's Conv2DTileSync::tileIndex would give (policies.h:197-199)
     print("conv chain 2 channel tiles", kind, flush=True)
     check_chain(chained_convs(2, 14, 14, 128, api.CONV_TILE.T128x64x32, api.CONV_TILE.T128x64x32, kind, iters=2), 2)
+    check_chain(chained_convs(2, 14, 14, 128, api.CONV_TILE.HALO_256x64x64, api.CONV_TILE.HALO_128x128x64, kind, iters=2), 2)
 
 
 def test_chained_conv_pair_producer_trails():
@@ -197,9 +221,12 @@ def test_chained_conv_pair_producer_trails():
     print("conv chain trailing producer", flush=True)
     check_chain(chained_convs(4, 20, 20, 64, api.CONV_TILE.T128x64x32, api.CONV_TILE.T128x64x32, "conv2dtile",
                               iters=2, max_wg=(1, 0)), 2)
+    check_chain(chained_convs(4, 20, 20, 64, api.CONV_TILE.HALO_256x64x64, api.CONV_TILE.HALO_256x64x64, "conv2dtile",
+                              iters=2, max_wg=(1, 0)), 2)
 
 
-@pytest.mark.parametrize("shape,tile", [((32, 56, 56, 64), api.CONV_TILE.T128x64x32), ((32, 28, 28, 128), api.CONV_TILE.T128x128x32)])
+@pytest.mark.parametrize("shape,tile", [((32, 56, 56, 64), api.CONV_TILE.T128x64x32), ((32, 28, 28, 128), api.CONV_TILE.T128x128x32),
+                                        ((32, 56, 56, 64), api.CONV_TILE.HALO_256x64x64), ((32, 28, 28, 128), api.CONV_TILE.HALO_128x128x64)])
 @pytest.mark.parametrize("kind", ["conv2dtile", "row"])
 def test_resnet_conv_pair_full_size(shape, tile, kind):
     # the two benchmark shapes of resnet_results.csv (batch 32): 56x56x64 and 28x28x128
