@@ -108,8 +108,9 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   // being computed and settled when the tile is done.
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
+  const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();
     const uint32_t ticket = sTicket;
     if (ticket >= numTiles) {
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
         }
     }
 
-    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     // Normalise and store: register r of tile tt is head-dim 32tt + 8(r/4) + 4hi + r%4 of query myq.
     rowSum += __shfl_xor(rowSum, 32);
     const float inv = 1.0f / rowSum;

@@ -90,8 +90,9 @@ __global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams
 
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
+  const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();
     const uint32_t ticket = sTicket;
     if (ticket >= numTiles) {
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams
     // The loads issued for chunks past the last one (zeros) may still be on their way into LDS, which the
     // epilogue is about to reuse.
     waitVmcnt<0>();
-    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, 0};
     if (completed && stage.isProducer()) stage.post(done);

@@ -151,8 +151,9 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
   // being computed and settled when the tile is done.
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
+  const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();
     const uint32_t ticket = sTicket;
     if (ticket >= numTiles) {
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
     // The loads issued for chunks past the end of K (zeros) may still be on their way into LDS, which the
     // epilogue is about to reuse.
     waitVmcnt<0>();
-    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
 
     // All waves must be past their last LDS read before the next tile's loads

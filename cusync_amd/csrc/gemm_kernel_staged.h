@@ -76,8 +76,9 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   // being computed and settled when the tile is done.
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
+  const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
-    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds) : stage.drawFinish(nextRaw, p.launched, round, dryXcds);
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();
     const uint32_t ticket = sTicket;
     if (ticket >= numTiles) {
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
       if (kt + 1 < nk) step(Parity<1>{}, kt + 1);
     }
 
-    if (tid == 0) nextRaw = stage.drawBegin(dryXcds);     // settled after the epilogue
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, t.z};
     // the post's barrier (or this one) keeps the next tile's LDS writes behind the epilogue's LDS reads

@@ -90,6 +90,15 @@ struct DynStage {
     const uint32_t perSlice = width * d.grid.x;          // this XCD's tiles in one k-slice
     return (l / perSlice) * d.grid.x * d.grid.y + lo * d.grid.x + l % perSlice;
   }
+  // True when the static first tiles already are all tiles (a launch of one round whose workgroups spread
+  // evenly over the lists): nobody then needs a dispenser, a look at the others or the count of workgroups
+  // that ran dry, and a workgroup leaves after its tile without a single atomic.
+  __device__ __forceinline__ bool allStatic(uint32_t launched) const {
+    if (!customOrder()) return false;
+    bool all = true;
+    for (uint32_t x = 0; x < 8; x++) all = all && xcdStatic(x, launched) == xcdTiles(x);
+    return all;
+  }
   static __device__ __forceinline__ uint32_t workgroupIndex() {
     return blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   }
@@ -111,16 +120,18 @@ struct DynStage {
   }
 
   // Issues the draw of the next ticket; `dry` is the mask drawFinish() keeps.
-  __device__ __forceinline__ uint32_t drawBegin(uint32_t dry) const {
-    if (!customOrder()) return 0;
+  __device__ __forceinline__ uint32_t drawBegin(uint32_t dry, bool noDraws = false) const {
+    if (!customOrder() || noDraws) return 0;
     const uint32_t mine = homeList();
     if (dry & (1u << mine)) return 0xffffffffu;
     return dev::ticketAdd(&d.xcdTickets[mine * 32], 1);
   }
   // Turns the result of drawBegin() into a ticket; numTiles() or more when the
   // tiles have run out.  `round` = tickets this workgroup has drawn before.
-  __device__ __forceinline__ uint32_t drawFinish(uint32_t raw, uint32_t launched, uint32_t round, uint32_t& dry) const {
+  __device__ __forceinline__ uint32_t drawFinish(uint32_t raw, uint32_t launched, uint32_t round, uint32_t& dry,
+                                                 bool noDraws = false) const {
     if (!customOrder()) return workgroupIndex() + round * launched;
+    if (noDraws) return 0xffffffffu;
     constexpr uint32_t kLine = 32;          // counters are 128 bytes apart
     const uint32_t mine = homeList();
     if (raw != 0xffffffffu) {
@@ -148,11 +159,11 @@ struct DynStage {
     return 0xffffffffu;
   }
   // First ticket of a workgroup: its static position if its XCD's list is long enough.
-  __device__ __forceinline__ uint32_t firstTicket(uint32_t launched, uint32_t& dry) const {
+  __device__ __forceinline__ uint32_t firstTicket(uint32_t launched, uint32_t& dry, bool noDraws = false) const {
     if (!customOrder()) return workgroupIndex();
     const uint32_t b = workgroupIndex(), x = b & 7u, pos = b >> 3;
     if (pos < xcdTiles(x)) return xcdTicket(x, pos);
-    return drawFinish(drawBegin(dry), launched, 0, dry);
+    return drawFinish(drawBegin(dry, noDraws), launched, 0, dry, noDraws);
   }
 
   __device__ __forceinline__ cusync_dim3 ticketToTile(uint32_t ticket) const {

@@ -39,6 +39,10 @@ CUSYNC_DEVICE void acquireFence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "ag
 #ifndef CUSYNC_SPIN_LIMIT
 #define CUSYNC_SPIN_LIMIT (1u << 20)
 #endif
+// Longest sleep between two polls, in units of 1024 clocks (about 0.43 us).
+#ifndef CUSYNC_MAX_NAPS
+#define CUSYNC_MAX_NAPS 8
+#endif
 
 // First half of a poll by a whole wave: only the first active lane touches
 // memory (sixty-four lanes loading the same coherent address are sixty-four
@@ -64,7 +68,7 @@ CUSYNC_DEVICE bool pollUntilAtLeast(const volatile uint32_t* addr, uint32_t want
   while (pollOnce(addr) < want) {
     if (++polls >= CUSYNC_SPIN_LIMIT) return false;
     for (uint32_t i = 0; i < naps; i++) __builtin_amdgcn_s_sleep(16);   // 16 * 64 clocks
-    if (naps < 8) naps <<= 1;
+    if (naps < CUSYNC_MAX_NAPS) naps <<= 1;
   }
   return true;
 }
