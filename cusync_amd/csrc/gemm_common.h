@@ -141,21 +141,21 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   // instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
   // applied) into a [WM*32][BN] buffer (rows padded by 16 bytes against bank conflicts), then all threads
   // copy the buffer out, 16 bytes per lane, consecutive lanes along a row.
-  auto storeFinal = [&](auto&& value) {
+  // storePass(i, value): MFMA row tile i of every wave, value(j, g) its four floats of tile j, group g.
+  auto storePass = [&](int i, auto&& value) {
     constexpr int PITCH = C::BN * 2 + 16;
     constexpr int ROWS = C::WM * 32;
     constexpr int CPR = C::BN / 8;
     constexpr int STEPS = ROWS * CPR / kThreads;
     static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
     static_assert((ROWS * CPR) % kThreads == 0, "whole copy steps");
-#pragma unroll
-    for (int i = 0; i < C::TM; i++) {
+    {
       __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
 #pragma unroll
       for (int j = 0; j < C::TN; j++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-          const floatx4 v = value(i, j, g);
+          const floatx4 v = value(j, g);
           half4 o;
 #pragma unroll
           for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
@@ -173,9 +173,11 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
     }
   };
   if (p.splitK <= 1) {
-    storeFinal([&](int i, int j, int g) {
-      return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-    });
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+      storePass(i, [&](int j, int g) {
+        return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+      });
     return true;
   }
   // Partial sums live in the workspace in register order: value g of MFMA tile (i, j) of every thread is one
@@ -205,24 +207,29 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   __syncthreads();
   if (!*sLast) return false;
   dev::acquireFence();
-  // The slice that arrived last adds the slices in index order, eight loads of a position in flight at a time.
-  // (Accumulating into `acc` inside a loop over the slices makes the compiler spill in the main loop.  Letting
-  // all slices wait for each other and add up a share each was measured and is slower: every waiting slice
-  // ends with an acquire that empties its XCD's L2 under the workgroups still streaming weights; the GPT-3
-  // MLP at one row went from 108 to 156 us.)
-  storeFinal([&](int i, int j, int g) {
-    const float* src = mine + slot(i, j, g);
-    floatx4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (uint32_t z0 = 0; z0 < p.splitK; z0 += 8) {
-      floatx4 v[8];
+  // The slice that arrived last adds the slices in index order, one row of MFMA tiles at a time: all loads
+  // of that row for one slice are issued together (TN * 4 of 16 bytes per thread).  One position at a time
+  // would be a chain of round trips to memory as long as the GEMM itself; everything at once, accumulated
+  // into `acc`, makes the compiler spill in the main loop.  (Letting all slices wait for each other and add
+  // up a share each was measured and is slower: every waiting slice ends with an acquire that empties its
+  // XCD's L2 under the workgroups still streaming weights; the GPT-3 MLP at one row went from 108 to 156 us.)
 #pragma unroll
-      for (uint32_t u = 0; u < 8; u++) v[u] = *reinterpret_cast<const floatx4*>(src + min(z0 + u, p.splitK - 1) * sliceStride);
+  for (int i = 0; i < C::TM; i++) {
+    floatx4 sum[C::TN][4];
+    for (uint32_t z = 0; z < p.splitK; z++) {
+      const float* src = mine + z * sliceStride;
+      floatx4 v[C::TN][4];
 #pragma unroll
-      for (uint32_t u = 0; u < 8; u++)
-        if (z0 + u < p.splitK) sum = (z0 + u == 0) ? v[u] : sum + v[u];
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) v[j][g] = *reinterpret_cast<const floatx4*>(src + slot(i, j, g));
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) sum[j][g] = z == 0 ? v[j][g] : sum[j][g] + v[j][g];
     }
-    return sum;
-  });
+    storePass(i, [&](int j, int g) { return sum[j][g]; });
+  }
   return true;
 }
 
