@@ -118,8 +118,8 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return CUSYNC_ERROR_DEVICE;
   if (RT(hipMemcpy(d->tileOrder, host_tile_order, sizeof(cusync_dim3) * n, hipMemcpyHostToDevice))) return CUSYNC_ERROR_DEVICE;
   if (producer) {
-    if (RT(hipMalloc((void**)&d->tileStatusWrite, sizeof(uint32_t) * n))) return CUSYNC_ERROR_DEVICE;
-    if (RT(hipMemset(d->tileStatusWrite, 0, sizeof(uint32_t) * n))) return CUSYNC_ERROR_DEVICE;
+    if (RT(hipMalloc((void**)&d->tileStatusWrite, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return CUSYNC_ERROR_DEVICE;
+    if (RT(hipMemset(d->tileStatusWrite, 0, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return CUSYNC_ERROR_DEVICE;
   }
   return CUSYNC_SUCCESS;
 }
@@ -189,7 +189,8 @@ cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems,
   int bad = 0;
   if (sems) {
     if (!d->tileStatusWrite) return CUSYNC_ERROR_NOT_PRODUCER;
-    bad |= RT(hipMemcpy(sems, d->tileStatusWrite, sizeof(uint32_t) * n, hipMemcpyDeviceToHost));
+    bad |= RT(hipMemcpy2D(sems, sizeof(uint32_t), d->tileStatusWrite, sizeof(uint32_t) * CUSYNC_SEM_STRIDE, sizeof(uint32_t), n,
+                          hipMemcpyDeviceToHost));      // one semaphore per 128-byte line on the device, packed for the caller
   }
   if (tile_order) bad |= RT(hipMemcpy(tile_order, d->tileOrder, sizeof(cusync_dim3) * n, hipMemcpyDeviceToHost));
   if (tile_counter) {

@@ -186,14 +186,14 @@ struct DynStage {
   // without ordering; dev::pollFinish() on the result, after other work, gives
   // the value to compare with waitTarget().
   __device__ __forceinline__ uint32_t peekBegin(const cusync_dim3& tile) const {
-    return dev::pollBegin(&d.tileStatusRead[dyn::tileIndex(d.in, tile, d.prodGrid)]);
+    return dev::pollBegin(&d.tileStatusRead[dyn::tileIndex(d.in, tile, d.prodGrid) * CUSYNC_SEM_STRIDE]);
   }
 
   // Wave-uniform wait: every lane of the calling wave passes the same tile.
   // No barrier; each wave that is going to read the tile calls this itself.
   __device__ __forceinline__ void waitWave(const cusync_dim3& tile) const {
     if (!needsWait(tile)) return;
-    const uint32_t idx = dyn::tileIndex(d.in, tile, d.prodGrid);
+    const uint32_t idx = dyn::tileIndex(d.in, tile, d.prodGrid) * CUSYNC_SEM_STRIDE;
     const bool ok = lineAligned ? dev::spinUntilAtLeastNoInvalidate(&d.tileStatusRead[idx], waitTarget())
                                 : dev::spinUntilAtLeast(&d.tileStatusRead[idx], waitTarget());
     if (!ok && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0)
@@ -205,7 +205,7 @@ struct DynStage {
     if (!isProducer()) return;
     __syncthreads();
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
-      const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid);
+      const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid) * CUSYNC_SEM_STRIDE;
       const uint32_t v = dyn::postValue(d.out);
       if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::releaseStore(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
       else dev::releaseAdd(&d.tileStatusWrite[idx], v);

@@ -214,7 +214,7 @@ public:
 #if CUSYNC_HAS_DEVICE
   // Current value of the semaphore guarding `tile`.
   CUSYNC_DEVICE uint32_t waitSemValue(dim3 tile) {
-    return dev::loadAcquire(&tileStatusRead_[waitTileIndex(tile)]);
+    return dev::loadAcquire(&tileStatusRead_[waitTileIndex(tile) * CUSYNC_SEM_STRIDE]);
   }
 
   // Blocks the workgroup until the producer has delivered `tile`.  Thread
@@ -260,7 +260,7 @@ CUSTAGE_METHOD(CuSyncError) wait(dim3& tile, uint32_t waitingThread, bool callSy
   if (flat == waitingThread) {
     const uint32_t need = (uint32_t)iter * inputPolicy_.waitValue(tile, prodGrid_);
     const uint32_t idx = inputPolicy_.tileIndex(tile, prodGrid_);
-    if (!dev::spinUntilAtLeast(&tileStatusRead_[idx], need)) dev::ticketAdd(spinTimeouts_, 1);
+    if (!dev::spinUntilAtLeast(&tileStatusRead_[idx * CUSYNC_SEM_STRIDE], need)) dev::ticketAdd(spinTimeouts_, 1);
   }
   if (callSync) __syncthreads();
   return CuSyncSuccess;
@@ -275,8 +275,8 @@ CUSTAGE_METHOD(CuSyncError) post(const dim3& tile, uint32_t postThread) {
   if (flat == postThread) {
     const uint32_t idx = outputPolicy_.tileIndex(tile, grid_);
     const uint32_t value = outputPolicy_.postValue(tile, grid_);
-    if (getNoAtomicAdd()) dev::releaseStore(&tileStatusWrite_[idx], value * (uint32_t)iter);
-    else dev::releaseAdd(&tileStatusWrite_[idx], value);
+    if (getNoAtomicAdd()) dev::releaseStore(&tileStatusWrite_[idx * CUSYNC_SEM_STRIDE], value * (uint32_t)iter);
+    else dev::releaseAdd(&tileStatusWrite_[idx * CUSYNC_SEM_STRIDE], value);
   }
   return CuSyncSuccess;
 }

@@ -76,6 +76,11 @@ typedef struct cusync_policy_desc {
  * ships (CS/tile-orders.h:52-75).  The prebuilt kernels then compute a ticket's tile instead of loading it. */
 enum { CUSYNC_STAGE_IDENTITY_ORDER = 1 };
 
+/* Semaphore i of a stage lives at tileStatus[i * CUSYNC_SEM_STRIDE]: each on its own 128-byte line, so that the
+ * waves polling one semaphore do not queue up behind those polling its neighbours (the reference packs them,
+ * CS/cusync.h:186-190).  cusync_stage_read_state returns them packed. */
+#define CUSYNC_SEM_STRIDE 32
+
 typedef struct cusync_stage_desc {
   cusync_dim3 grid;           /* grid_     : logical tile grid of this stage */
   cusync_dim3 prodGrid;       /* prodGrid_ : logical tile grid of its producer */
@@ -93,7 +98,7 @@ typedef struct cusync_stage_desc {
                                  kernels plus a count of workgroups that ran dry; all 0 between runs */
   uint32_t *kernelExecuted;   /* wait-kernel flag: == iter once every workgroup of the run has begun */
   uint32_t *spinTimeouts;     /* number of waits of this stage that gave up (0 in a healthy chain) */
-  uint32_t *tileStatusWrite;  /* semaphores this stage posts */
+  uint32_t *tileStatusWrite;  /* semaphores this stage posts, CUSYNC_SEM_STRIDE apart */
   uint32_t *tileStatusRead;   /* semaphores this stage waits on (its producer's) */
 } cusync_stage_desc;
 
