@@ -29,8 +29,8 @@ BATCHES = [1, 16, 64, 256, 512, 1024, 2048]
 PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes one GEMM launch of the B = 2048 step moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by
-# a plain copy of known size (profiles/gemm_dma_128x192x32_gpt3_mlp_b2048.md).
-TRAFFIC_BYTES_PER_LAUNCH = 877e6
+# a plain copy of known size (profiles/gemm_dma_gpt3_mlp_b2048.md).
+TRAFFIC_BYTES_PER_LAUNCH = 819e6
 
 
 def trimmed(times):
@@ -139,7 +139,7 @@ def main():
         k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
         flops_per_launch = 2.0 * B * HIDDEN * INNER
         achieved = flops_per_launch / (k_us * 1e-6) / 1e12
-        tm, tn, tk = api.tile_shape(tiles[0])
+        shapes = ["%dx%dx%d" % api.tile_shape(t) for t in tiles[:2]]
         # plain copy of known size: the scale for the FETCH_SIZE / WRITE_SIZE counters
         a = torch.zeros(64 << 20, dtype=torch.float16, device="cuda")      # 128 MiB read + 128 MiB written
         b = torch.empty_like(a)
@@ -148,8 +148,9 @@ def main():
         torch.cuda.synchronize()
         return {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
-                "kernel": "gemmDmaKernel/gemmKernel tile %dx%dx%d (mean of GEMM1 %.1f us and GEMM2 %.1f us, stream-ordered, "
-                          "%.1f GFLOP per launch)" % (tm, tn, tk, statistics.fmean(g1), statistics.fmean(g2), flops_per_launch / 1e9),
+                "kernel": "gemmDmaKernel, mean of the two launches of the step: GEMM1 tile %s %.1f us, GEMM2 tile %s %.1f us "
+                          "(stream-ordered, %.1f GFLOP per launch)" % (shapes[0], statistics.fmean(g1), shapes[1], statistics.fmean(g2),
+                                                                       flops_per_launch / 1e9),
                 }, trimmed(t_s)[0], tiles
 
     if args.profile_chain == "attention":

@@ -6,7 +6,8 @@
 // One workgroup (four wavefronts) owns 128 query rows of one head; each
 // wavefront owns 32 of them.  K and V are walked in blocks of 64 rows that go
 // from global memory straight into LDS (two stages, the next block loads while
-// the current one is multiplied).
+// the current one is multiplied; two workgroups share a CU.  Four stages with
+// one workgroup per CU were measured at 2048 rows x 12 heads: 89 us against 70).
 //
 // Everything is computed transposed so that the softmax needs no shuffles:
 //   S^T = K Q^T      (MFMA rows = kv, columns = q)
