@@ -277,7 +277,7 @@ def main():
     # ---- the timed step: B = args.batch under the better CuSync policy ----------
     cand = {}
     for name, sync in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE)):
-        ts, _ = protocol(B, sync, warm=5, timed=10)
+        ts, _ = protocol(B, sync, warm=10, timed=30)
         cand[name] = (trimmed(ts)[0], sync)
     policy = min(cand, key=lambda k: cand[k][0])
     m, h, y = make(B, cand[policy][1])
