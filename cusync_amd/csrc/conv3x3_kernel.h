@@ -30,6 +30,7 @@ namespace gemm {
 template<int BM_, int BN_, int WM_, int WN_, int STAGES_, int OCC_>
 struct Halo3x3Cfg {
   static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_, STAGES = STAGES_, OCC = OCC_;
+  static constexpr int THREADS = kThreads;
   static constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32, KS = BK / 16;
   static constexpr int B_ROW_BYTES = BK * 2, B_CPR = B_ROW_BYTES / 16;
   static constexpr int B_STAGE = BN * B_ROW_BYTES, B_LOADS = B_STAGE / 1024 / 4;

@@ -146,9 +146,9 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
     constexpr int PITCH = C::BN * 2 + 16;
     constexpr int ROWS = C::WM * 32;
     constexpr int CPR = C::BN / 8;
-    constexpr int STEPS = ROWS * CPR / kThreads;
+    constexpr int STEPS = ROWS * CPR / C::THREADS;
     static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
-    static_assert((ROWS * CPR) % kThreads == 0, "whole copy steps");
+    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
     {
       __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
 #pragma unroll
@@ -164,7 +164,7 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
       __syncthreads();
 #pragma unroll
       for (int s = 0; s < STEPS; s++) {
-        const uint32_t idx = s * kThreads + threadIdx.x;
+        const uint32_t idx = s * C::THREADS + threadIdx.x;
         const uint32_t lr = idx / CPR, c = idx % CPR;
         const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
         if (m < p.M && n < p.N)
@@ -181,12 +181,12 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
     return true;
   }
   // Partial sums live in the workspace in register order: value g of MFMA tile (i, j) of every thread is one
-  // contiguous 4 KiB run (256 threads x 16 bytes), so slices write and the finishing slice reads with fully
+  // contiguous run (16 bytes per thread), so slices write and the finishing slice reads with fully
   // coalesced accesses; the padding rows and columns of edge tiles are carried along.
   constexpr size_t kTileFloats = (size_t)C::BM * C::BN;
   const size_t sliceStride = (size_t)p.stage.d.grid.x * p.stage.d.grid.y * kTileFloats;
   float* mine = p.partials + ((size_t)t.y * p.stage.d.grid.x + t.x) * kTileFloats + (size_t)threadIdx.x * 4;
-  auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (kThreads * 4); };
+  auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (C::THREADS * 4); };
 #pragma unroll
   for (int i = 0; i < C::TM; i++)
 #pragma unroll

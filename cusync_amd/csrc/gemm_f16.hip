@@ -44,22 +44,23 @@ using namespace cusync::gemm;
 
 struct TileInfo {
   uint32_t bm, bn, bk;
+  uint32_t threads;
   size_t lds;
   void (*kernel[2])(GemmParams);   // [plain A, SwiGLU A]
   int residentPerCU;     // filled lazily
 };
 
 #define CUSYNC_TILE(BM, BN, BK, WM, WN) \
-  { BM, BN, BK, (size_t)TileCfg<BM, BN, BK, WM, WN>::LDS_BYTES, \
+  { BM, BN, BK, kThreads, (size_t)TileCfg<BM, BN, BK, WM, WN>::LDS_BYTES, \
     { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1 }
 
 // Direct-to-LDS tiles have no SwiGLU variant (that operand needs arithmetic on its way into LDS).
 #define CUSYNC_TILE_DMA(BM, BN, BK, WM, WN, ST, OCC) \
-  { BM, BN, BK, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC>::LDS_BYTES, \
+  { BM, BN, BK, DmaCfg<BM, BN, BK, WM, WN, ST, OCC>::THREADS, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC>::LDS_BYTES, \
     { gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC>>, nullptr }, -1 }
 
 TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
-  CUSYNC_TILE_DMA(256, 256, 32, 2, 2, 4, 1),   // CUSYNC_TILE_256x256x32: direct-to-LDS, 4 stages
+  CUSYNC_TILE_DMA(256, 256, 32, 4, 2, 4, 2),   // CUSYNC_TILE_256x256x32: direct-to-LDS, eight wavefronts of 64x128, 4 stages, one workgroup per CU
   CUSYNC_TILE(256, 128, 64, 2, 2),   // CUSYNC_TILE_256x128x64
   CUSYNC_TILE(128, 128, 64, 2, 2),   // CUSYNC_TILE_128x128x64
   CUSYNC_TILE(64, 128, 64, 1, 4),    // CUSYNC_TILE_64x128x64
@@ -71,7 +72,7 @@ TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
   CUSYNC_TILE_DMA(128, 256, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x256x32
   CUSYNC_TILE_DMA(128, 128, 32, 2, 2, 3, 3),   // CUSYNC_TILE_128x128x32: three workgroups per CU
   CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x192x32: 6144 and 12288 columns are 32 and 64 tiles
-  CUSYNC_TILE_DMA(256, 192, 32, 2, 2, 3, 1),   // CUSYNC_TILE_256x192x32
+  CUSYNC_TILE_DMA(256, 192, 32, 4, 2, 4, 2),   // CUSYNC_TILE_256x192x32: eight wavefronts of 64x96
 };
 
 std::mutex g_mutex;
@@ -99,7 +100,7 @@ int residentWorkgroups(int tile) {
       if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->kernel[v]),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds))) return 0;
       int n = 0;
-      if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel[v], kThreads, ti->lds))) return 0;
+      if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel[v], (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
     }
     ti->residentPerCU = perCU;
@@ -221,7 +222,7 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   p.mPad = s.grid.y * ti->bm;
   p.partials = (float*)a->workspace;
   p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
-  hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(kThreads), ti->lds, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }

@@ -41,17 +41,23 @@ struct DmaCfg {
   static constexpr int B_ROWS = BT ? BN : BK;
   static constexpr int A_CPR = A_ROW_BYTES / 16, B_CPR = B_ROW_BYTES / 16;   // 16-byte chunks per row
   static constexpr int A_STAGE = BM * A_ROW_BYTES, B_STAGE = B_ROWS * B_ROW_BYTES;
-  static constexpr int A_LOADS = A_STAGE / 1024 / 4, B_LOADS = B_STAGE / 1024 / 4;   // per wave per chunk
+  static constexpr int WAVES = WM * WN, THREADS = WAVES * 64;
+  // 1 KiB wave loads per chunk.  When B's do not divide among the waves the spare ones of the last waves
+  // go out of range into a 1 KiB dump behind the stages, so that every wave counts the same loads per chunk.
+  static constexpr int A_TOTAL = A_STAGE / 1024, B_TOTAL = B_STAGE / 1024;
+  static constexpr int A_LOADS = A_TOTAL / WAVES, B_LOADS = (B_TOTAL + WAVES - 1) / WAVES;   // per wave per chunk
   static constexpr int LOADS = A_LOADS + B_LOADS;
   static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES;
-  static constexpr int LDS_BYTES = STAGES * (A_STAGE + B_STAGE);
-  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static constexpr bool DUMP = B_TOTAL % WAVES != 0;
+  static constexpr int DUMP_OFFSET = STAGES * (A_STAGE + B_STAGE);
+  static constexpr int LDS_BYTES = DUMP_OFFSET + (DUMP ? 1024 : 0);
+  static_assert(WAVES == 4 || WAVES == 8, "four or eight wavefronts per workgroup");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile is made of 32x32 MFMA tiles");
   static_assert(A_CPR == 4 || A_CPR == 8, "BK is 32 or 64");
   static_assert(BT || B_CPR % 8 == 0, "a B row covers whole 128-byte bank sweeps");
   static_assert(BT || WTN % 32 == 0, "MFMA tiles of B start on 64-byte groups");
-  static_assert(A_STAGE % 4096 == 0 && B_STAGE % 4096 == 0, "whole 1 KiB loads per wave");
-  static_assert(LDS_BYTES * WAVES_PER_SIMD <= 160 * 1024, "fits the LDS of one CU");
+  static_assert(A_TOTAL % WAVES == 0 && B_STAGE % 1024 == 0, "whole 1 KiB loads per wave");
+  static_assert(LDS_BYTES * (WAVES_PER_SIMD * 4 / WAVES) <= 160 * 1024, "fits the LDS of one CU");
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
   static_assert(KS >= 2, "the loads of the next chunk ride on the LDS reads of k-step 1");
 };
@@ -77,7 +83,7 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
 }
 
 template<class C, int AMODE = kAPlain>
-__global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
+__global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
   constexpr bool conv = AMODE == kAConv;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   __shared__ uint32_t sTicket, sLast;
@@ -105,7 +111,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
 #pragma unroll
   for (int q = 0; q < C::B_LOADS; q++) {
     const uint32_t slot = (wave * C::B_LOADS + q) * 64 + lane;
-    bLoadRow[q] = slot / C::B_CPR;
+    bLoadRow[q] = slot / C::B_CPR;                 // >= B_ROWS for a spare load
     const uint32_t pos = slot % C::B_CPR;
     bLoadChunk[q] = C::BT ? pos ^ ((bLoadRow[q] / A_SWZ_DIV) & (C::B_CPR - 1)) : pos ^ (4 * (bLoadRow[q] & 1));
   }
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
 #pragma unroll
     for (int q = 0; q < C::B_LOADS; q++) {
       if constexpr (C::BT) bVoff0[q] = ((n0 + bLoadRow[q]) * p.ldb + bLoadChunk[q] * 8) * 2;     // rows past N fall outside the buffer
-      else bVoff0[q] = n0 + bLoadChunk[q] * 8 < p.N ? (bLoadRow[q] * p.ldb + n0 + bLoadChunk[q] * 8) * 2 : kOutOfRange;
+      else bVoff0[q] = (bLoadRow[q] < C::B_ROWS && n0 + bLoadChunk[q] * 8 < p.N) ? (bLoadRow[q] * p.ldb + n0 + bLoadChunk[q] * 8) * 2 : kOutOfRange;
     }
 
     // Convolution: the pixel each of this lane's A rows stands for.
@@ -266,7 +272,8 @@ __global__ __launch_bounds__(kThreads, C::WAVES_PER_SIMD) void gemmDmaKernel(Gem
       constexpr int Q = decltype(QP)::value;
       const uint32_t k0 = kBegin + kt * C::BK;
       if constexpr (Q < C::B_LOADS) {
-        const uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
+        uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
+        if constexpr (C::DUMP) { static_assert(!C::BT, "spare loads are resolved for row-major B only"); if (wave * C::B_LOADS + Q >= C::B_TOTAL) lds = ldsBase + C::DUMP_OFFSET; }
         uint32_t off;
         if constexpr (C::BT) off = k0 + bLoadChunk[Q] * 8 < kEnd ? bVoff0[Q] + k0 * 2 : kOutOfRange;
         else off = (bVoff0[Q] != kOutOfRange && k0 < kEnd) ? bVoff0[Q] + k0 * p.ldb * 2 : kOutOfRange;

@@ -12,6 +12,7 @@ namespace gemm {
 template<int BM_, int BN_, int BK_, int WM_, int WN_>
 struct TileCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+  static constexpr int THREADS = kThreads;
   static constexpr int WTM = BM / WM, WTN = BN / WN;       // wavefront tile
   static constexpr int TM = WTM / 32, TN = WTN / 32;       // MFMA tiles per wavefront
   static constexpr int PA = BK + 8;                         // LDS row pitch of A in halfs (16 B pad)

@@ -22,11 +22,11 @@ import sys
 from . import api
 
 # tile id -> (wave grid M x N, pipeline stages)
-WAVES = {api.TILE.T256x256x32: (2, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.TILE.T128x128x64: (2, 2, 2),
+WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.TILE.T128x128x64: (2, 2, 2),
          api.TILE.T64x128x64: (1, 4, 2), api.TILE.T32x128x64: (1, 4, 2), api.TILE.T128x256x64: (2, 2, 2),
          api.TILE.T256x64x64: (4, 1, 2), api.TILE.T128x64x64: (2, 2, 2), api.TILE.T256x128x32: (2, 2, 3),
          api.TILE.T128x256x32: (2, 2, 3), api.TILE.T128x128x32: (2, 2, 3), api.TILE.T128x192x32: (2, 2, 3),
-         api.TILE.T256x192x32: (2, 2, 3)}
+         api.TILE.T256x192x32: (4, 2, 4)}
 
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 

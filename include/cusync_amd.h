@@ -180,9 +180,11 @@ enum {
   CUSYNC_A_SWIGLU = 1          /* A[m,k] = silu(G[m,k]) * G[m,k + K]; G has K*2 valid columns */
 };
 
-/* Tile shapes the library was built with.  256x256x32, 256x128x32, 128x256x32 and
- * 128x128x32 move their operands from global memory straight into LDS and have no SwiGLU
- * variant; the others stage them through registers. */
+/* Tile shapes the library was built with.  The ...x32 shapes move their operands from
+ * global memory straight into LDS and have no SwiGLU variant; the others stage them
+ * through registers.  256x256x32 and 256x192x32 run eight wavefronts per workgroup and
+ * one workgroup per CU (such a producer and its consumer cannot share a CU, so a chain
+ * on them overlaps nothing); all others run four wavefronts. */
 enum {
   CUSYNC_TILE_256x256x32 = 0,
   CUSYNC_TILE_256x128x64 = 1,
