@@ -233,6 +233,16 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   return true;
 }
 
+// Half a pass: NM MFMAs with the R LDS reads of the next k-step's fragments spread between them.
+template<int NM, int R, int M = 0>
+__device__ __forceinline__ void schedHalf() {
+  if constexpr (M < NM) {
+    schedGroup<kSchedMfma, 1>();
+    schedGroup<kSchedDsRead, evenShare(R, NM, M)>();
+    schedHalf<NM, R, M + 1>();
+  }
+}
+
 template<int P> struct Parity { static constexpr int value = P; };
 
 // Calls f(Parity<0>{}), f(Parity<1>{}), ... f(Parity<N-1>{}): a loop whose index

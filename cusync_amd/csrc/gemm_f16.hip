@@ -55,12 +55,12 @@ struct TileInfo {
     { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1 }
 
 // Direct-to-LDS tiles have no SwiGLU variant (that operand needs arithmetic on its way into LDS).
-#define CUSYNC_TILE_DMA(BM, BN, BK, WM, WN, ST, OCC) \
-  { BM, BN, BK, DmaCfg<BM, BN, BK, WM, WN, ST, OCC>::THREADS, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC>::LDS_BYTES, \
-    { gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC>>, nullptr }, -1 }
+#define CUSYNC_TILE_DMA(...) \
+  { DmaCfg<__VA_ARGS__>::BM, DmaCfg<__VA_ARGS__>::BN, DmaCfg<__VA_ARGS__>::BK, DmaCfg<__VA_ARGS__>::THREADS, \
+    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1 }
 
 TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
-  CUSYNC_TILE_DMA(256, 256, 32, 4, 2, 4, 2),   // CUSYNC_TILE_256x256x32: direct-to-LDS, eight wavefronts of 64x128, 4 stages, one workgroup per CU
+  CUSYNC_TILE_DMA(256, 256, 32, 4, 2, 4, 2, false, true),   // CUSYNC_TILE_256x256x32: direct-to-LDS, eight wavefronts of 64x128, 4 stages, one workgroup per CU
   CUSYNC_TILE(256, 128, 64, 2, 2),   // CUSYNC_TILE_256x128x64
   CUSYNC_TILE(128, 128, 64, 2, 2),   // CUSYNC_TILE_128x128x64
   CUSYNC_TILE(64, 128, 64, 1, 4),    // CUSYNC_TILE_64x128x64
@@ -72,7 +72,7 @@ TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
   CUSYNC_TILE_DMA(128, 256, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x256x32
   CUSYNC_TILE_DMA(128, 128, 32, 2, 2, 3, 3),   // CUSYNC_TILE_128x128x32: three workgroups per CU
   CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x192x32: 6144 and 12288 columns are 32 and 64 tiles
-  CUSYNC_TILE_DMA(256, 192, 32, 4, 2, 4, 2),   // CUSYNC_TILE_256x192x32: eight wavefronts of 64x96
+  CUSYNC_TILE_DMA(256, 192, 32, 4, 2, 4, 2, false, true),   // CUSYNC_TILE_256x192x32: eight wavefronts of 64x96
 };
 
 std::mutex g_mutex;

@@ -22,6 +22,14 @@
 // chunk kt.  The loads are inline assembly on purpose: the compiler would
 // otherwise wait for every outstanding direct load before any LDS read, which
 // removes the overlap between prefetch and compute.
+//
+// Pipelined order (DmaCfg::PIPE, for workgroups that have a CU to themselves and
+// so nobody to fill their bubbles).  In the order above the first fragments of a
+// chunk can only be read after the barrier, and all wavefronts read them at the
+// same moment: the matrix pipes idle for an LDS round trip per chunk.  Here the
+// barrier sits between the two k-steps of chunk kt and already covers chunk
+// kt+1, so that the fragments of (kt+1, k-step 0) are read under the MFMAs of
+// (kt, k-step 1); the loads of chunk kt+STAGES-1 go into the stage of chunk kt-1.
 #pragma once
 
 #include "gemm_common.h"
@@ -29,8 +37,9 @@
 namespace cusync {
 namespace gemm {
 
-template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false>
+template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false, bool PIPE_ = false>
 struct DmaCfg {
+  static constexpr bool PIPE = PIPE_;                      // barrier in the middle of a chunk, fragments prefetched across chunks
   static constexpr bool BT = BT_;                          // B given as [N][K] (k contiguous), e.g. KRSC filters
   static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // register budget: 512 / this per lane
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
@@ -60,6 +69,7 @@ struct DmaCfg {
   static_assert(LDS_BYTES * (WAVES_PER_SIMD * 4 / WAVES) <= 160 * 1024, "fits the LDS of one CU");
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
   static_assert(KS >= 2, "the loads of the next chunk ride on the LDS reads of k-step 1");
+  static_assert(!PIPE || (KS == 2 && STAGES >= 3), "the pipelined order is written for two k-steps per chunk");
 };
 
 // One direct load: 64 lanes x 16 bytes from buffer `rsrc` at per-lane byte offset
@@ -366,6 +376,63 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
       __builtin_amdgcn_sched_barrier(0);
     };
 
+    // ---- pipelined order -----------------------------------------------------------
+    half8 pfa[2][C::TM], pfb[2][C::TN];
+    auto loadFragP = [&](auto SP, auto FP, auto SLOT, int kk) {
+      constexpr int S = decltype(SP)::value, F = decltype(FP)::value, slot = decltype(SLOT)::value;
+      if constexpr (F < C::TM) {
+        pfa[slot][F] = *reinterpret_cast<const half8*>(smem + S * C::A_STAGE + aFrag[kk] + F * 32 * C::A_ROW_BYTES);
+      } else {
+        constexpr int J = F - C::TM;
+        const char* sb = smem + C::STAGES * C::A_STAGE + S * C::B_STAGE;
+        if constexpr (C::BT) {
+          pfb[slot][J] = *reinterpret_cast<const half8*>(sb + bFragT[kk] + J * 32 * C::B_ROW_BYTES);
+        } else {
+          typedef short4v __attribute__((address_space(3))) * lds_ptr;
+          const char* q = sb + bFrag[J] + kk * 16 * C::B_ROW_BYTES;
+          short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
+          short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * C::B_ROW_BYTES));
+          half4 l4 = __builtin_bit_cast(half4, lo), h4 = __builtin_bit_cast(half4, hi);
+          pfb[slot][J] = __builtin_shufflevector(l4, h4, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      }
+    };
+    auto mfmaP = [&](auto SLOT) {
+      constexpr int slot = decltype(SLOT)::value;
+#pragma unroll
+      for (int i = 0; i < C::TM; i++)
+#pragma unroll
+        for (int j = 0; j < C::TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pfb[slot][j], pfa[slot][i], acc[i][j], 0, 0, 0);
+    };
+    auto stepP = [&](auto SP, uint32_t kt) {
+      constexpr int S = decltype(SP)::value;
+      constexpr int R = C::TM + C::TN;
+      constexpr int DS = C::TM + (C::BT ? 1 : 2) * C::TN;
+      // k-step 0 (fragments already in slot 0) while the fragments of k-step 1 arrive
+      staticFor<R>([&](auto FP) { loadFragP(SP, FP, Parity<1>{}, 1); });
+      mfmaP(Parity<0>{});
+      schedHalf<C::TM * C::TN, DS>();
+      __builtin_amdgcn_sched_barrier(0);
+      waitVmcnt<(C::STAGES - 3) * C::LOADS>();     // own part of chunk kt+1
+      __builtin_amdgcn_s_barrier();                // chunk kt+1 is in LDS for everyone; everyone is done with chunk kt-1
+      asm volatile("" ::: "memory");
+      const uint32_t ktLoad = kt + C::STAGES - 1;
+      if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
+      earlyPoll(kBegin + (ktLoad + 1) * C::BK);
+      __builtin_amdgcn_sched_barrier(0);
+      // k-step 1 while the first fragments of chunk kt+1 arrive and the loads of chunk ktLoad go out
+      staticFor<R>([&](auto FP) {
+        loadFragP(Parity<(S + 1) % C::STAGES>{}, FP, Parity<0>{}, 0);
+        staticFor<C::LOADS>([&](auto QP) {
+          if constexpr (decltype(QP)::value * R / C::LOADS == decltype(FP)::value) issueOne(Parity<(S + C::STAGES - 1) % C::STAGES>{}, QP, ktLoad);
+        });
+      });
+      mfmaP(Parity<1>{});
+      schedHalf<C::TM * C::TN, DS>();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+
     if (consumer) {
       cusync_dim3 w = {m0, 0, 1};
       if (stage.needsWait(w)) {
@@ -379,15 +446,31 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
     issueAll(Parity<0>{}, 0);
     if constexpr (C::STAGES > 2) { if (nk > 1) waitChunk(kBegin + C::BK); issueAll(Parity<1>{}, 1); }
     if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); issueAll(Parity<2>{}, 2); }
-    static_assert(C::STAGES >= 2 && C::STAGES <= 4, "prologue written for 2..4 stages");
+    if constexpr (C::STAGES > 4) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); issueAll(Parity<3>{}, 3); }
+    static_assert(C::STAGES >= 2 && C::STAGES <= 5, "prologue written for 2..5 stages");
     earlyPoll(kBegin + (C::STAGES - 1) * C::BK);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
 
-    for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
-      step(Parity<0>{}, kt);
-      if (kt + 1 < nk) step(Parity<1 % C::STAGES>{}, kt + 1);
-      if (C::STAGES > 2 && kt + 2 < nk) step(Parity<2 % C::STAGES>{}, kt + 2);
-      if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
+    if constexpr (C::PIPE) {
+      waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      staticFor<C::TM + C::TN>([&](auto FP) { loadFragP(Parity<0>{}, FP, Parity<0>{}, 0); });
+      for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
+        stepP(Parity<0>{}, kt);
+        if (kt + 1 < nk) stepP(Parity<1 % C::STAGES>{}, kt + 1);
+        if (C::STAGES > 2 && kt + 2 < nk) stepP(Parity<2 % C::STAGES>{}, kt + 2);
+        if (C::STAGES > 3 && kt + 3 < nk) stepP(Parity<3 % C::STAGES>{}, kt + 3);
+        if (C::STAGES > 4 && kt + 4 < nk) stepP(Parity<4 % C::STAGES>{}, kt + 4);
+      }
+    } else {
+      for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
+        step(Parity<0>{}, kt);
+        if (kt + 1 < nk) step(Parity<1 % C::STAGES>{}, kt + 1);
+        if (C::STAGES > 2 && kt + 2 < nk) step(Parity<2 % C::STAGES>{}, kt + 2);
+        if (C::STAGES > 3 && kt + 3 < nk) step(Parity<3 % C::STAGES>{}, kt + 3);
+        if (C::STAGES > 4 && kt + 4 < nk) step(Parity<4 % C::STAGES>{}, kt + 4);
+      }
     }
 
     // The loads issued for chunks past the end of K (zeros) may still be on their way into LDS, which the

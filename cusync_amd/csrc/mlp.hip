@@ -44,19 +44,17 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   else if (c.batch <= 64) small = CUSYNC_TILE_64x128x64;
   else small = CUSYNC_TILE_128x128x64;
   const bool big = c.batch > 128;
-  // measured on the GPT-3 shard: 128x128 wins up to 512 rows (more tiles to spread), 128x256 from 2048 on;
-  // where the width is a multiple of 192, 128x192 beats both above 512 rows (6144 and 12288 columns are 32
-  // and 64 tiles: whole rounds on 256 CUs at two workgroups each)
+  // Measured on the GPT-3 shard.  Where the width is a multiple of 192 (6144 and 12288 columns are 32 and
+  // 64 tiles: whole rounds on 256 CUs) the 192-wide direct-to-LDS tiles win from 256 rows on: 128x192 at two
+  // workgroups per CU up to 768 rows, 256x192 with a CU to itself above (8 % faster at 1024 and 2048 rows;
+  // at 512 rows it is as fast stream-ordered but leaves a consumer launched next to it nowhere to run).
+  // Other widths: 128x128 up to 1024 rows (more tiles to spread), 128x256 above.
   const uint32_t n1 = c.model == CUSYNC_MLP_LLAMA ? 2 * c.inner : c.inner, n2 = c.hidden;
+  const int wide = c.batch > 768 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  // (the per-batch tuner, cusync_amd/tuner.py, found the same tile best at 256 rows — with 4 and 2 k-slices —
-  // and 128x128 at 512 rows)
-  const bool wide = big && (c.batch <= 384 || c.batch > 768);
-  // GEMM1 keeps 128x256 above 1024 rows: at 2048 rows 128x192 makes 512 tiles, one per slot, and leaves a
-  // consumer launched next to it nowhere to start
-  if (wide && c.batch <= 1024 && n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
-  if (wide && n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
+  if (big && n1 % 192 == 0) a = wide;
+  if (big && n2 % 192 == 0 && !swiglu) b = wide;
   if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;

@@ -42,7 +42,7 @@ def candidates(batch, n1, n2):
     elif batch <= 512:
         tiles, splits = [api.TILE.T128x128x32, api.TILE.T128x192x32, api.TILE.T256x128x32, api.TILE.T128x256x32], [1, 2, 4]
     else:
-        tiles, splits = [api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1]
+        tiles, splits = [api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1]
     ok = lambda t, n: n % 192 == 0 or t not in (api.TILE.T128x192x32, api.TILE.T256x192x32)
     return [(t, s) for t in tiles for s in splits if ok(t, n1)], [(t, s) for t in tiles for s in splits if ok(t, n2)]
 
