@@ -297,6 +297,13 @@ def main():
     # stream-ordered on the same shape: baseline latency and the kernels' own durations
     roof, stream_us, _ = roofline_leg(B, args.warmup, max(10, args.steps))
     roof["traffic"] = TRAFFIC_BYTES_PER_LAUNCH
+    # what the matrix pipes alone sustain on this machine (register operands, no LDS, no memory): the clock
+    # drops under a device-wide MFMA load, further with random operands than with zeros
+    zero_tf, zero_mhz = api.probe_mfma_rate(False)
+    rand_tf, rand_mhz = api.probe_mfma_rate(True)
+    roof["mfma_alone"] = {"zero_operands_tflops": round(zero_tf, 1), "zero_operands_mhz": round(zero_mhz),
+                          "random_operands_tflops": round(rand_tf, 1), "random_operands_mhz": round(rand_mhz),
+                          "frac_of_random_operands_rate": round(roof["achieved"] / rand_tf, 4)}
 
     out = {
         "metric": "GPT-3 MLP shard latency (us) + % gain vs kernel-boundary sync, B=1..2048",

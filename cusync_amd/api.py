@@ -343,6 +343,13 @@ def sync_overhead_pair(blocks=1280, threads=128, warmup=10, iters=100):
     return a.value, b.value
 
 
+def probe_mfma_rate(random_data=True, iters=2000, launches=10):
+    """(TFLOP/s, shader clock in MHz) the matrix pipes sustain alone, on zero or random register operands."""
+    t, f = C.c_double(0), C.c_double(0)
+    check(_lib.load().cusync_probe_mfma_rate(1 if random_data else 0, iters, launches, C.byref(t), C.byref(f)), "probe_mfma_rate")
+    return t.value, f.value
+
+
 def sync_overhead_pingpong(partner, rounds=2000):
     """Nanoseconds per post -> wait -> post -> wait round trip between workgroup 0 and workgroup `partner`."""
     t = C.c_double(0)

@@ -417,6 +417,18 @@ cusync_error cusync_sync_overhead_pair(uint32_t blocks, uint32_t threads, int wa
  * workgroup 0's XCD and partner 1 does not.  No counterpart in the reference, whose GPUs have one L2. */
 cusync_error cusync_sync_overhead_pingpong(uint32_t partner, uint32_t rounds, double *ns_per_round_trip);
 
+/* ------------------------------------------------------------------------- */
+/* What the matrix pipes sustain on this machine                              */
+/* ------------------------------------------------------------------------- */
+
+/* Runs chains of v_mfma_f32_32x32x16_f16 on register operands (no LDS, no memory) on every SIMD of the device,
+ * `launches` untimed launches and then `launches` timed ones of `iters` x 16 MFMAs per wavefront, with all-zero
+ * (`random_data` = 0) or random operands, and reports the rate and the shader clock it ran at.  Under such a load
+ * the power management lowers the clock, more so the more bits toggle: the result is the ceiling of any fp16 GEMM
+ * on the machine, below the published 2.5 PFLOP/s.  No counterpart in the reference; bench.py prints it next to
+ * the roofline of the GEMM kernels. */
+cusync_error cusync_probe_mfma_rate(int random_data, uint32_t iters, int launches, double *tflops, double *clock_mhz);
+
 #ifdef __cplusplus
 }
 #endif

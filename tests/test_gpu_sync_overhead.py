@@ -26,3 +26,15 @@ def test_pingpong_rejects_bad_arguments():
         api.sync_overhead_pingpong(0)
     with pytest.raises(api.CuSyncError):
         api.sync_overhead_pingpong(64)
+
+
+@pytest.mark.gpu
+def test_mfma_rate_probe():
+    """The matrix pipes alone: plausible rates and clocks, and zero operands are not slower than random ones."""
+    zero_tf, zero_mhz = api.probe_mfma_rate(False, iters=1000, launches=5)
+    rand_tf, rand_mhz = api.probe_mfma_rate(True, iters=1000, launches=5)
+    print("MFMA alone: zeros %.0f TFLOP/s at %.0f MHz, random %.0f TFLOP/s at %.0f MHz" % (zero_tf, zero_mhz, rand_tf, rand_mhz), flush=True)
+    for tf, mhz in ((zero_tf, zero_mhz), (rand_tf, rand_mhz)):
+        assert 300.0 < tf < 2700.0            # cannot exceed the published dense rate
+        assert 400.0 < mhz < 2700.0
+    assert zero_tf > 0.9 * rand_tf
