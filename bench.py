@@ -30,7 +30,7 @@ PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes one GEMM launch of the B = 2048 step moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by
 # a plain copy of known size (profiles/gemm_dma_gpt3_mlp_b2048.md).
-TRAFFIC_BYTES_PER_LAUNCH = 819e6
+TRAFFIC_BYTES_PER_LAUNCH = 582e6
 
 
 def trimmed(times):
