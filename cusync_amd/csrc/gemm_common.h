@@ -213,20 +213,31 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   // into `acc`, makes the compiler spill in the main loop.  (Letting all slices wait for each other and add
   // up a share each was measured and is slower: every waiting slice ends with an acquire that empties its
   // XCD's L2 under the workgroups still streaming weights; the GPT-3 MLP at one row went from 108 to 156 us.)
+  // Narrow wavefront tiles have few loads per slice: several slices are fetched together (G of them, up to 16
+  // loads of 16 bytes per thread in flight), still added in index order.
+  constexpr int G = C::TN * 4 >= 16 ? 1 : 16 / (C::TN * 4);
 #pragma unroll
   for (int i = 0; i < C::TM; i++) {
     floatx4 sum[C::TN][4];
-    for (uint32_t z = 0; z < p.splitK; z++) {
-      const float* src = mine + z * sliceStride;
-      floatx4 v[C::TN][4];
+    for (uint32_t z = 0; z < p.splitK; z += G) {
+      floatx4 v[G][C::TN][4];
 #pragma unroll
-      for (int j = 0; j < C::TN; j++)
+      for (int q = 0; q < G; q++) {
+        if (z + q >= p.splitK) break;
+        const float* src = mine + (z + q) * sliceStride;
 #pragma unroll
-        for (int g = 0; g < 4; g++) v[j][g] = *reinterpret_cast<const floatx4*>(src + slot(i, j, g));
+        for (int j = 0; j < C::TN; j++)
 #pragma unroll
-      for (int j = 0; j < C::TN; j++)
+          for (int g = 0; g < 4; g++) v[q][j][g] = *reinterpret_cast<const floatx4*>(src + slot(i, j, g));
+      }
 #pragma unroll
-        for (int g = 0; g < 4; g++) sum[j][g] = z == 0 ? v[j][g] : sum[j][g] + v[j][g];
+      for (int q = 0; q < G; q++) {
+        if (z + q >= p.splitK) break;
+#pragma unroll
+        for (int j = 0; j < C::TN; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) sum[j][g] = (z + q == 0) ? v[q][j][g] : sum[j][g] + v[q][j][g];
+      }
     }
     storePass(i, [&](int j, int g) { return sum[j][g]; });
   }

@@ -199,7 +199,10 @@ enum {
   CUSYNC_TILE_128x128x32 = 10,
   CUSYNC_TILE_128x192x32 = 11,       /* direct-to-LDS; 6144 = 32 x 192, 12288 = 64 x 192: whole waves on 256 CUs */
   CUSYNC_TILE_256x192x32 = 12,
-  CUSYNC_TILE_COUNT = 13
+  CUSYNC_TILE_D32x128x64 = 13,       /* direct-to-LDS, 4 stages: few rows, bound by streaming the weights */
+  CUSYNC_TILE_D64x128x64 = 14,       /* direct-to-LDS, 3 stages */
+  CUSYNC_TILE_D64x192x64 = 15,       /* direct-to-LDS, 4 stages, a CU to itself: 32 or 64 column tiles times 8 or 4 k-slices are 256 */
+  CUSYNC_TILE_COUNT = 16
 };
 
 typedef struct cusync_gemm_args {
