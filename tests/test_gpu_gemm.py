@@ -196,7 +196,10 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
 
 @pytest.mark.parametrize("policy_kind,opts", [("tile", 0), ("tile", api.OPT.NO_ATOMIC_ADD | api.OPT.REORDER_TILE_LOADS), ("row", 0)])
 @pytest.mark.parametrize("tiles", [(api.TILE.T128x128x64, api.TILE.T128x128x64), (api.TILE.T32x128x64, api.TILE.T64x128x64),
-                                   (api.TILE.T256x128x64, api.TILE.T128x128x64)])
+                                   (api.TILE.T256x128x64, api.TILE.T128x128x64),
+                                   (api.TILE.T256x192x32, api.TILE.T256x192x32),      # eight wavefronts, pipelined order
+                                   (api.TILE.D32x128x64, api.TILE.D64x192x64),        # few-row direct-to-LDS tiles
+                                   (api.TILE.D64x192x64, api.TILE.T128x192x32)])
 def test_two_chained_gemms_config1(policy_kind, opts, tiles):
     # BASELINE config 1: M=256, N=K=1024, fp32 accumulate, inputs uniform from a seed
     print("chained", policy_kind, opts, tiles, flush=True)
@@ -223,10 +226,12 @@ def test_chained_gemms_with_few_workgroups():
 
 
 @pytest.mark.parametrize("policy_kind,opts", [("tile", api.OPT.NO_ATOMIC_ADD), ("row", 0)])
-def test_chained_gemms_with_split_k(policy_kind, opts):
+@pytest.mark.parametrize("tiles", [(api.TILE.T64x128x64, api.TILE.T128x128x32), (api.TILE.D32x128x64, api.TILE.D32x128x64),
+                                   (api.TILE.D64x192x64, api.TILE.T256x192x32)])
+def test_chained_gemms_with_split_k(policy_kind, opts, tiles):
     # split-K on both sides: only the slice that completes a tile posts it, and a consumer slice waits
     # for the producer tiles of its own K range only (CC/gemm/kernel/cusyncgemm.h:374-398)
-    a, b, d, c, e, ps, cs, want_sems = chained(256, 1024, 1024, api.TILE.T64x128x64, api.TILE.T128x128x32,
+    a, b, d, c, e, ps, cs, want_sems = chained(256, 1024, 1024, tiles[0], tiles[1],
                                                policy_kind, iters=2, opts=opts, split=(4, 2))
     assert_close(c, orc.gemm(a, b), "C")
     assert_close(e, orc.gemm(c, d), "E")
