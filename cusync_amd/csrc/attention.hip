@@ -16,6 +16,7 @@
 #include "../../include/cusync_amd.h"
 #include "rt_internal.h"
 #include "attention_kernel.h"
+#include "split_choice.h"
 
 namespace {
 
@@ -59,6 +60,9 @@ struct cusync_attn_layer {
   const void* wo;
   uint32_t E;                      // heads * head_dim
   int tile1, tile3;
+  int split1, split3;              // k-slices of the two projections
+  void* ws1;
+  void* ws3;                       // their split-K workspaces (null without slices)
   cusync_stage_desc st[3];         // QKV projection, attention, output projection
   hipStream_t stream[3];
   hipEvent_t eStart, eMid1, eMid2, eEnd;
@@ -148,23 +152,34 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   L->cfg = *cfg;
   L->wqkv = wqkv; L->wo = wo;
   L->E = cfg->heads * kHD;
-  // Same per-row-count choice as the MLP chain: 128x128 tiles while the grid would otherwise not
-  // cover the device, 128x256 from 2048 rows on.
-  const int small = cfg->seq <= 32 ? CUSYNC_TILE_32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
+  // Same per-row-count choice as the MLP chain.  Widths that are multiples of 192 (4608 = 24 x 192, 12288 =
+  // 64 x 192) take the 192-wide direct-to-LDS tiles: 64x192x64 up to 256 rows, where streaming the weights
+  // bounds the projections, 128x192 above (256x192, the MLP's choice from 1024 rows on, gains nothing here: the
+  // QKV projection has only 24 column tiles).  Other widths: tiles that follow the row count up to 128 rows,
+  // 128x128 up to 1024 rows, 128x256 above.
+  const int small = cfg->seq <= 32 ? CUSYNC_TILE_D32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  // widths that are multiples of 192 (4608 = 24 x 192, 12288 = 64 x 192) fill whole rounds with 128x192 tiles
-  const int wide = cfg->seq > 512 ? CUSYNC_TILE_128x192x32 : dflt;
+  const int wide = cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64 : CUSYNC_TILE_128x192x32;
   L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide : dflt;
   L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide : dflt;
+  L->ws1 = L->ws3 = nullptr;
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
     setError("attn layer: unknown tile id");
     delete L;
     return nullptr;
   }
-  const cusync_dim3 g1 = cusync_gemm_grid(L->tile1, cfg->seq, 3 * L->E, 1);
+  // few rows leave most CUs without a tile: k-slices as in the MLP chain
+  uint32_t bk1 = 0, bk3 = 0;
+  cusync_gemm_tile_shape(L->tile1, nullptr, nullptr, &bk1);
+  cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, &bk3);
+  const cusync_dim3 flat1 = cusync_gemm_grid(L->tile1, cfg->seq, 3 * L->E, 1);
+  const cusync_dim3 flat3 = cusync_gemm_grid(L->tile3, cfg->seq, cfg->hidden, 1);
+  L->split1 = cusync::gemm::pickSplit(0, flat1.x * flat1.y, cfg->hidden, bk1, cusync_gemm_max_resident(L->tile1));
+  L->split3 = cusync::gemm::pickSplit(0, flat3.x * flat3.y, L->E, bk3, cusync_gemm_max_resident(L->tile3));
+  const cusync_dim3 g1 = cusync_gemm_grid(L->tile1, cfg->seq, 3 * L->E, L->split1);
   const cusync_dim3 g2 = cusync_attention_grid(cfg->seq, cfg->heads);
-  const cusync_dim3 g3 = cusync_gemm_grid(L->tile3, cfg->seq, cfg->hidden, 1);
+  const cusync_dim3 g3 = cusync_gemm_grid(L->tile3, cfg->seq, cfg->hidden, L->split3);
 
   cusync_policy_desc sync1 = noSync(), sync2 = noSync();
   int opts = 0;
@@ -214,6 +229,19 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
     delete L;
     return nullptr;
   }
+  for (int which = 0; which < 2; which++) {
+    cusync_gemm_args a;
+    memset(&a, 0, sizeof a);
+    a.stage = L->st[which == 0 ? 0 : 2];
+    a.M = cfg->seq; a.N = which == 0 ? 3 * L->E : cfg->hidden; a.K = which == 0 ? cfg->hidden : L->E;
+    a.tile = which == 0 ? L->tile1 : L->tile3;
+    a.split_k = which == 0 ? L->split1 : L->split3;
+    const size_t bytes = cusync_gemm_workspace_size(&a);
+    if (bytes == 0) continue;
+    void* ws = nullptr;
+    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { delete L; return nullptr; }
+    (which == 0 ? L->ws1 : L->ws3) = ws;
+  }
   for (int i = 0; i < 3; i++)
     if (CUSYNC_HIP(hipStreamCreateWithFlags(&L->stream[i], hipStreamNonBlocking))) { delete L; return nullptr; }
   if (CUSYNC_HIP(hipEventCreate(&L->eStart)) || CUSYNC_HIP(hipEventCreate(&L->eMid1)) ||
@@ -227,6 +255,8 @@ void cusync_attn_layer_destroy(cusync_attn_layer* L) {
   for (int i = 0; i < 3; i++) cusync_stage_free(&L->st[i]);
   (void)hipEventDestroy(L->eStart); (void)hipEventDestroy(L->eMid1); (void)hipEventDestroy(L->eMid2); (void)hipEventDestroy(L->eEnd);
   for (int i = 0; i < 3; i++) (void)hipStreamDestroy(L->stream[i]);
+  if (L->ws1) (void)hipFree(L->ws1);
+  if (L->ws3) (void)hipFree(L->ws3);
   delete L;
 }
 
@@ -241,7 +271,7 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     a1.stage = L->st[0]; a1.M = S; a1.N = 3 * E; a1.K = H;
     a1.A = x; a1.lda = H; a1.B = L->wqkv; a1.ldb = 3 * E; a1.ldd = 3 * E;
     a1.D = (char*)qkv + (size_t)L->cfg.cached_rows * 3 * E * 2;       // behind the cache rows (attention.cu:289)
-    a1.tile = L->tile1; a1.split_k = 1;
+    a1.tile = L->tile1; a1.split_k = L->split1; a1.workspace = L->ws1;
     cusync_attention_args a2;
     memset(&a2, 0, sizeof a2);
     a2.stage = L->st[1]; a2.seq = S; a2.heads = L->cfg.heads; a2.head_dim = kHD;
@@ -249,7 +279,7 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     a2.cached_rows = L->cfg.cached_rows;
     a3.stage = L->st[2]; a3.M = S; a3.N = H; a3.K = E;
     a3.A = o; a3.lda = E; a3.B = L->wo; a3.ldb = H; a3.D = y; a3.ldd = H;
-    a3.tile = L->tile3; a3.split_k = 1;
+    a3.tile = L->tile3; a3.split_k = L->split3; a3.workspace = L->ws3;
 
     hipStream_t s0 = L->stream[0], s1 = overlapped ? L->stream[1] : s0, s2 = overlapped ? L->stream[2] : s0;
     cusync_error e;

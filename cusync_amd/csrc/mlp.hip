@@ -13,6 +13,7 @@
 
 #include "../../include/cusync_amd.h"
 #include "rt_internal.h"
+#include "split_choice.h"
 
 struct cusync_mlp {
   cusync_mlp_config cfg;
@@ -33,6 +34,7 @@ struct cusync_mlp {
 namespace {
 
 using cusync::rt::setError;
+using cusync::gemm::pickSplit;
 
 // Built-in choice of tile shapes per batch size for 256 CUs.  Above 128 rows the
 // direct-to-LDS tiles are used; below that the M extent follows the batch.  A SwiGLU consumer has
@@ -69,20 +71,6 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
   *t2 = c.tile2 >= 0 ? c.tile2 : b;
-}
-
-// k-slices for a GEMM of `tiles` output tiles: double while the launch stays
-// within one and a half workgroups per CU and every slice keeps at least eight
-// K chunks.  Small batches are bound by streaming the weights, and without
-// slices a 32-row problem occupies 48 workgroups on 256 CUs; beyond about 384
-// workgroups the cost of adding the slices' partial sums outweighs the gain
-// (measured: M=16, N=6144, K=12288 takes 121 / 49 / 52 / 72 us with 1 / 4 / 8 / 16 slices).
-int pickSplit(int requested, uint32_t tiles, uint32_t K, uint32_t bk, int resident) {
-  if (requested > 0) return requested;
-  const uint32_t target = (uint32_t)std::min(resident, 384);
-  int s = 1;
-  while (tiles * (uint32_t)s * 2 <= target && K / ((uint32_t)s * 2) >= 8 * bk) s *= 2;
-  return s;
 }
 
 cusync_policy_desc noSync() {
