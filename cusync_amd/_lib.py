@@ -56,12 +56,13 @@ class ConvChainConfig(C.Structure):
 
 class AttentionArgs(C.Structure):
     _fields_ = [("stage", StageDesc), ("seq", u32), ("heads", u32), ("head_dim", u32), ("cached_rows", u32), ("qkv", vp), ("ldqkv", u32),
-                ("out", vp), ("ldo", u32), ("scale", C.c_float), ("causal", i32), ("max_workgroups", i32)]
+                ("out", vp), ("ldo", u32), ("scale", C.c_float), ("causal", i32), ("max_workgroups", i32),
+                ("kv_split_blocks", u32), ("workspace", vp)]
 
 
 class AttnLayerConfig(C.Structure):
     _fields_ = [("seq", u32), ("hidden", u32), ("heads", u32), ("head_dim", u32), ("sync", i32),
-                ("tile1", i32), ("tile3", i32), ("opts", i32), ("causal", i32), ("cached_rows", u32)]
+                ("tile1", i32), ("tile3", i32), ("opts", i32), ("causal", i32), ("cached_rows", u32), ("kv_split_blocks", i32)]
 
 
 class MlpConfig(C.Structure):
@@ -122,6 +123,8 @@ SIGNATURES = {
     "cusync_conv_chain_tile": (C.c_int, [vp]),
     "cusync_attention_tile_shape": (C.c_int, [C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_attention_grid": (Dim3, [u32, u32]),
+    "cusync_attention_grid_split": (Dim3, [u32, u32, u32, u32]),
+    "cusync_attention_workspace_size": (sz, [C.POINTER(AttentionArgs)]),
     "cusync_attention_can_implement": (C.c_int, [C.POINTER(AttentionArgs)]),
     "cusync_attention_max_resident": (C.c_int, []),
     "cusync_attention_run": (C.c_int, [C.POINTER(AttentionArgs), vp]),

@@ -266,17 +266,26 @@ def attention_tile_shape():
     return m.value, n.value, k.value
 
 
-def attention_grid(seq, heads):
-    return _lib.load().cusync_attention_grid(seq, heads).tup()
+def attention_grid(seq, heads, cached_rows=0, kv_split_blocks=0):
+    """(heads, row tiles, splits of the key range)."""
+    return _lib.load().cusync_attention_grid_split(seq, heads, cached_rows, kv_split_blocks).tup()
 
 
-def attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, head_dim=128, scale=0.0, causal=True, max_workgroups=0, cached_rows=0):
+def attention_args(stage, seq, heads, qkv, ldqkv, out, ldo, head_dim=128, scale=0.0, causal=True, max_workgroups=0, cached_rows=0,
+                   kv_split_blocks=0, workspace=None):
     a = AttentionArgs()
+    a.kv_split_blocks, a.workspace = kv_split_blocks, workspace
     a.stage = stage.desc
     a.seq, a.heads, a.head_dim, a.cached_rows = seq, heads, head_dim, cached_rows
     a.qkv, a.ldqkv, a.out, a.ldo = qkv, ldqkv, out, ldo
     a.scale, a.causal, a.max_workgroups = scale, int(causal), max_workgroups
     return a
+
+
+def attention_workspace_size(seq, heads, cached_rows=0, kv_split_blocks=0):
+    a = AttentionArgs()
+    a.seq, a.heads, a.cached_rows, a.kv_split_blocks = seq, heads, cached_rows, kv_split_blocks
+    return _lib.load().cusync_attention_workspace_size(C.byref(a))
 
 
 def attention(stage, seq, heads, qkv, ldqkv, out, ldo, stream=None, **kw):
@@ -304,9 +313,9 @@ class AttnLayer:
     CuSync stages (the chain of src/ml-bench/transformer/attention.cu:702-830)."""
 
     def __init__(self, seq, hidden, heads, sync, wqkv_ptr, wo_ptr, head_dim=128, tile1=-1, tile3=-1, opts=-1, causal=True,
-                 cached_rows=0):
+                 cached_rows=0, kv_split_blocks=-1):
         self.L = _lib.load()
-        self.cfg = AttnLayerConfig(seq, hidden, heads, head_dim, sync, tile1, tile3, opts, int(causal), cached_rows)
+        self.cfg = AttnLayerConfig(seq, hidden, heads, head_dim, sync, tile1, tile3, opts, int(causal), cached_rows, kv_split_blocks)
         self.h = self.L.cusync_attn_layer_create(C.byref(self.cfg), wqkv_ptr, wo_ptr)
         if not self.h:
             raise RuntimeError("cusync_attn_layer_create failed: " + last_error())

@@ -63,6 +63,8 @@ struct cusync_attn_layer {
   int split1, split3;              // k-slices of the two projections
   void* ws1;
   void* ws3;                       // their split-K workspaces (null without slices)
+  uint32_t kvSplit;                // key/value blocks per attention workgroup, 0 = no split
+  void* ws2;                       // workspace of the split attention
   cusync_stage_desc st[3];         // QKV projection, attention, output projection
   hipStream_t stream[3];
   hipEvent_t eStart, eMid1, eMid2, eEnd;
@@ -82,6 +84,23 @@ cusync_dim3 cusync_attention_grid(uint32_t seq, uint32_t heads) {
   return g;
 }
 
+cusync_dim3 cusync_attention_grid_split(uint32_t seq, uint32_t heads, uint32_t cached_rows, uint32_t kv_split_blocks) {
+  cusync_dim3 g = cusync_attention_grid(seq, heads);
+  if (kv_split_blocks) {
+    const uint32_t blocks = (cached_rows + seq + kBKV - 1) / kBKV;
+    g.z = std::max(1u, (blocks + kv_split_blocks - 1) / kv_split_blocks);
+  }
+  return g;
+}
+
+size_t cusync_attention_workspace_size(const cusync_attention_args* a) {
+  if (!a || !a->kv_split_blocks) return 0;
+  const cusync_dim3 g = cusync_attention_grid_split(a->seq, a->heads, a->cached_rows, a->kv_split_blocks);
+  if (g.z <= 1) return 0;
+  const size_t tiles = (size_t)g.x * g.y;
+  return tiles * g.z * (64 + 2) * kThreads * sizeof(float) + tiles * sizeof(uint32_t);
+}
+
 cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
   if (!a) return CUSYNC_ERROR_NOT_INITIALIZED;
   if (!a->seq || !a->heads) { setError("attention: empty problem"); return CUSYNC_ERROR_NOT_INITIALIZED; }
@@ -90,9 +109,10 @@ cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
   if (a->ldqkv < 3 * E || a->ldqkv % 8 || a->ldo < E || a->ldo % 4) { setError("attention: row pitch too small or misaligned"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if ((uint64_t)(a->seq + a->cached_rows) * a->ldqkv * 2 >= 0x80000000ull) { setError("attention: QKV larger than 2 GiB is not addressable by one buffer descriptor"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if ((uintptr_t)a->qkv % 16 || (uintptr_t)a->out % 8 || !a->qkv || !a->out) { setError("attention: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  const cusync_dim3 g = cusync_attention_grid(a->seq, a->heads);
+  const cusync_dim3 g = cusync_attention_grid_split(a->seq, a->heads, a->cached_rows, a->kv_split_blocks);
   const cusync_stage_desc& s = a->stage;
-  if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("attention: stage grid does not match cusync_attention_grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("attention: stage grid does not match cusync_attention_grid / cusync_attention_grid_split"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (g.z > 1 && (!a->workspace || (uintptr_t)a->workspace % 16)) { setError("attention: a split key range needs a 16-byte aligned workspace of cusync_attention_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (!s.tileOrder || !s.tileCounter || !s.startCounter || !s.spinTimeouts || !s.xcdTickets) { setError("attention: stage not allocated"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (s.out.kind != CUSYNC_POLICY_NOSYNC && !s.tileStatusWrite) { setError("attention: producer stage without semaphores"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (s.in.kind != CUSYNC_POLICY_NOSYNC) {
@@ -137,6 +157,13 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.scaleLog2 = scale * 1.4426950408889634f;
   p.causal = a->causal ? 1 : 0;
   p.launched = launched;
+  if (s.grid.z > 1) {
+    const size_t tiles = (size_t)s.grid.x * s.grid.y;
+    p.chunk = a->kv_split_blocks;
+    p.partO = (float*)a->workspace;
+    p.partStat = p.partO + tiles * s.grid.z * 64 * kThreads;
+    p.arrivals = (uint32_t*)(p.partStat + tiles * s.grid.z * 2 * kThreads);
+  }
   hipLaunchKernelGGL(attentionKernel, dim3(launched), dim3(kThreads), kLdsBytes, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
@@ -162,7 +189,13 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   const int wide = cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64 : CUSYNC_TILE_128x192x32;
   L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide : dflt;
   L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide : dflt;
-  L->ws1 = L->ws3 = nullptr;
+  L->ws1 = L->ws3 = L->ws2 = nullptr;
+  // Key ranges of 16 blocks (1024 rows) or more are cut in two.  Measured alone at 12 heads: 1024 rows 40 -> 35 us,
+  // 2048 rows 73 -> 65 us; finer cuts lose again (four: 71 us, eight: 124 us) — the kernel is bound by the softmax
+  // arithmetic of a CU rather than by its longest workgroup, and every cut adds a tile's fixed cost (Q fragments,
+  // first block, a pass over the partial results).
+  const uint32_t kvBlocks = (cfg->cached_rows + cfg->seq + kBKV - 1) / kBKV;
+  L->kvSplit = cfg->kv_split_blocks >= 0 ? (uint32_t)cfg->kv_split_blocks : kvBlocks >= 16 ? (kvBlocks + 1) / 2 : 0u;
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
     setError("attn layer: unknown tile id");
@@ -178,7 +211,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   L->split1 = cusync::gemm::pickSplit(0, flat1.x * flat1.y, cfg->hidden, bk1, cusync_gemm_max_resident(L->tile1));
   L->split3 = cusync::gemm::pickSplit(0, flat3.x * flat3.y, L->E, bk3, cusync_gemm_max_resident(L->tile3));
   const cusync_dim3 g1 = cusync_gemm_grid(L->tile1, cfg->seq, 3 * L->E, L->split1);
-  const cusync_dim3 g2 = cusync_attention_grid(cfg->seq, cfg->heads);
+  const cusync_dim3 g2 = cusync_attention_grid_split(cfg->seq, cfg->heads, cfg->cached_rows, L->kvSplit);
   const cusync_dim3 g3 = cusync_gemm_grid(L->tile3, cfg->seq, cfg->hidden, L->split3);
 
   cusync_policy_desc sync1 = noSync(), sync2 = noSync();
@@ -242,6 +275,13 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
     if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { delete L; return nullptr; }
     (which == 0 ? L->ws1 : L->ws3) = ws;
   }
+  {
+    cusync_attention_args a;
+    memset(&a, 0, sizeof a);
+    a.seq = cfg->seq; a.heads = cfg->heads; a.cached_rows = cfg->cached_rows; a.kv_split_blocks = L->kvSplit;
+    const size_t bytes = cusync_attention_workspace_size(&a);
+    if (bytes && (CUSYNC_HIP(hipMalloc(&L->ws2, bytes)) || CUSYNC_HIP(hipMemset(L->ws2, 0, bytes)))) { delete L; return nullptr; }
+  }
   for (int i = 0; i < 3; i++)
     if (CUSYNC_HIP(hipStreamCreateWithFlags(&L->stream[i], hipStreamNonBlocking))) { delete L; return nullptr; }
   if (CUSYNC_HIP(hipEventCreate(&L->eStart)) || CUSYNC_HIP(hipEventCreate(&L->eMid1)) ||
@@ -257,6 +297,7 @@ void cusync_attn_layer_destroy(cusync_attn_layer* L) {
   for (int i = 0; i < 3; i++) (void)hipStreamDestroy(L->stream[i]);
   if (L->ws1) (void)hipFree(L->ws1);
   if (L->ws3) (void)hipFree(L->ws3);
+  if (L->ws2) (void)hipFree(L->ws2);
   delete L;
 }
 
@@ -277,6 +318,7 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     a2.stage = L->st[1]; a2.seq = S; a2.heads = L->cfg.heads; a2.head_dim = kHD;
     a2.qkv = qkv; a2.ldqkv = 3 * E; a2.out = o; a2.ldo = E; a2.scale = 0.0f; a2.causal = L->cfg.causal;
     a2.cached_rows = L->cfg.cached_rows;
+    a2.kv_split_blocks = L->kvSplit; a2.workspace = L->ws2;
     a3.stage = L->st[2]; a3.M = S; a3.N = H; a3.K = E;
     a3.A = o; a3.lda = E; a3.B = L->wo; a3.ldb = H; a3.D = y; a3.ldd = H;
     a3.tile = L->tile3; a3.split_k = L->split3; a3.workspace = L->ws3;

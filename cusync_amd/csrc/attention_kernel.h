@@ -20,6 +20,13 @@
 // to fp16, already are the B operand of the second product: register e of a
 // lane in half-wave h stands for kv position 16u + 8(e/4) + 4h + e%4 of k-step
 // u, and the V^T fragment is read (LDS transpose read) in that same order.
+//
+// Long key ranges can be split (AttnParams::chunk key/value blocks per workgroup, grid z = split
+// index): a workgroup that walks all 32 blocks of the last rows of a 2048-row causal problem
+// alone is what the whole kernel waits for.  Each split leaves its unnormalised O^T, row maxima
+// and row sums in a workspace (register order, so all accesses are coalesced); the split that
+// arrives last at the tile's counter rescales and adds them in split order — the result does
+// not depend on arrival order — normalises, stores, re-arms the counter and posts the tile.
 #pragma once
 
 #include "gemm_kernel_dma.h"
@@ -44,11 +51,15 @@ struct AttnParams {
   float scaleLog2;                   // softmax scale * log2(e)
   uint32_t causal;
   uint32_t launched;
+  uint32_t chunk;                    // key/value blocks per split; 0: one workgroup walks the whole range
+  float* partO;                      // [heads][row tiles][splits][64][256] unnormalised O^T, register order
+  float* partStat;                   // [heads][row tiles][splits][2][256] row maximum, row sum
+  uint32_t* arrivals;                // [heads][row tiles] splits finished; 0 between launches
 };
 
 __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  __shared__ uint32_t sTicket;
+  __shared__ uint32_t sTicket, sLast;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -123,6 +134,15 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     const uint32_t qEnd = min(q0 + (uint32_t)kBQ, p.S);
     const uint32_t nkv = p.causal ? p.cached + qEnd : total;
     const uint32_t nblk = (nkv + kBKV - 1) / kBKV;
+    const uint32_t splits = p.chunk ? (nblk + p.chunk - 1) / p.chunk : 1;
+    if (t.z >= splits) {                               // this row tile needs fewer splits than the grid has
+      if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);
+      if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+      __syncthreads();
+      continue;
+    }
+    const uint32_t jBegin = p.chunk ? t.z * p.chunk : 0;
+    const uint32_t jEnd = p.chunk ? min(nblk, jBegin + p.chunk) : nblk;
     const uint32_t qw = q0 + 32 * wave;                 // first query row of this wave
     const uint32_t myq = qw + (lane & 31);
     // positions are rows of qkv: query i sits at cached + i and, when causal, sees keys 0 .. cached + i
@@ -157,8 +177,8 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     for (int s = 0; s < 8; s++)
       qf[s] = __builtin_bit_cast(half8, loadChunk(rReg, myq < p.S ? ((p.cached + myq) * p.ldq + head * kHD + 16 * s + 8 * hi) * 2 : kOutOfRange));
 
-    waitKV(0);
-    issue(0, 0);
+    waitKV(jBegin);
+    issue(jBegin, 0);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
 
     float rowMax = kMasked, rowSum = 0.0f;      // rowSum: this half-wave's share
@@ -168,12 +188,12 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) o[tt][r] = 0.0f;
 
-    for (uint32_t j = 0; j < nblk; j++) {
-      const uint32_t st = j & 1;
+    for (uint32_t j = jBegin; j < jEnd; j++) {
+      const uint32_t st = (j - jBegin) & 1;
       waitVmcnt<0>();
       __builtin_amdgcn_s_barrier();       // block j is in LDS for everyone; everyone is done with block j-1
       asm volatile("" ::: "memory");
-      if (j + 1 < nblk) { waitKV(j + 1); issue(j + 1, st ^ 1); }
+      if (j + 1 < jEnd) { waitKV(j + 1); issue(j + 1, st ^ 1); }
       if (p.causal && j * kBKV > p.cached + qw + 31) continue;       // wholly in this wave's future (wave-uniform)
 
       const char* ks = smem + st * 2 * kStageBytes;
@@ -246,10 +266,58 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     }
 
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
-    // Normalise and store: register r of tile tt is head-dim 32tt + 8(r/4) + 4hi + r%4 of query myq.
     rowSum += __shfl_xor(rowSum, 32);
+    bool completed = true;
+    if (splits > 1) {
+      // leave this split's share in the workspace; the last split to arrive puts the tile together
+      const size_t slot = ((size_t)head * stage.d.grid.y + t.y) * stage.d.grid.z;
+      float* po = p.partO + (slot + t.z) * (64 * kThreads) + tid * 4;
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+          *reinterpret_cast<floatx4*>(po + (tt * 4 + g) * (kThreads * 4)) = floatx4{o[tt][4 * g], o[tt][4 * g + 1], o[tt][4 * g + 2], o[tt][4 * g + 3]};
+      float* ps = p.partStat + (slot + t.z) * (2 * kThreads) + tid;
+      ps[0] = rowMax;
+      ps[kThreads] = rowSum;
+      __syncthreads();
+      uint32_t* counter = p.arrivals + head * stage.d.grid.y + t.y;
+      if (tid == 0) {
+        const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = before == splits - 1;
+        if (last) cusync::dev::storeRelaxed(counter, 0);
+        sLast = last;
+      }
+      __syncthreads();
+      completed = sLast != 0;
+      if (completed) {
+        cusync::dev::acquireFence();
+        float m = kMasked;
+        for (uint32_t z = 0; z < splits; z++) m = fmaxf(m, p.partStat[(slot + z) * (2 * kThreads) + tid]);
+        rowSum = 0.0f;
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) o[tt][r] = 0.0f;
+        for (uint32_t z = 0; z < splits; z++) {
+          const float* qs = p.partStat + (slot + z) * (2 * kThreads) + tid;
+          const float w = __builtin_amdgcn_exp2f(qs[0] - m);
+          rowSum += w * qs[kThreads];
+          const float* qo = p.partO + (slot + z) * (64 * kThreads) + tid * 4;
+#pragma unroll
+          for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const floatx4 v = *reinterpret_cast<const floatx4*>(qo + (tt * 4 + g) * (kThreads * 4));
+#pragma unroll
+              for (int e = 0; e < 4; e++) o[tt][4 * g + e] += w * v[e];
+            }
+        }
+      }
+    }
+    // Normalise and store: register r of tile tt is head-dim 32tt + 8(r/4) + 4hi + r%4 of query myq.
     const float inv = 1.0f / rowSum;
-    if (myq < p.S) {
+    if (completed && myq < p.S) {
       half_t* dst = p.out + (size_t)myq * p.ldo + head * kHD + 4 * hi;
 #pragma unroll
       for (int tt = 0; tt < 4; tt++)
@@ -265,7 +333,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
     cusync_dim3 done = {q0, head * kHD, 0};
-    if (stage.isProducer()) stage.post(done);
+    if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();
   }
 }

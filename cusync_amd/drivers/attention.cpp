@@ -41,7 +41,7 @@ int main(int argc, char** argv) {
     cusync_attn_layer_config c;
     memset(&c, 0, sizeof c);
     c.seq = (uint32_t)batch; c.hidden = hidden; c.heads = heads; c.head_dim = 128; c.sync = mode;
-    c.tile1 = c.tile3 = -1; c.opts = -1; c.causal = 1; c.cached_rows = (uint32_t)seqlen;
+    c.tile1 = c.tile3 = -1; c.opts = -1; c.causal = 1; c.cached_rows = (uint32_t)seqlen; c.kv_split_blocks = -1;
     cusync_attn_layer* l = cusync_attn_layer_create(&c, wqkv, wo);
     if (!l) { fprintf(stderr, "cusync_attn_layer_create failed: %s\n", cusync_rt_last_error()); exit(EXIT_FAILURE); }
     DRV_CHECK(cusync_attn_layer_run(l, x, qkv, o, y, warmup, nullptr, nullptr));

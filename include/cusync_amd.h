@@ -320,12 +320,19 @@ typedef struct cusync_attention_args {
   float scale;                 /* softmax scale; 0 selects 1/sqrt(head_dim) */
   int32_t causal;              /* 1: query i sees keys 0..i */
   int32_t max_workgroups;      /* 0 = as many as stay resident */
+  uint32_t kv_split_blocks;    /* 0: one workgroup walks all keys of its rows; n: at most n key/value blocks (of 64 rows) per
+                                  workgroup, grid = cusync_attention_grid_split, partial results combined through `workspace` */
+  void *workspace;             /* kv_split_blocks > 0: cusync_attention_workspace_size bytes, zeroed once by the caller */
 } cusync_attention_args;
 
 /* Rows per output tile (128), columns per output tile (= head_dim) and key/value rows per inner step. */
 int cusync_attention_tile_shape(uint32_t *tileM, uint32_t *tileN, uint32_t *blockKV);
 /* Logical grid (heads, row tiles, 1); an output tile is posted as {row, head*head_dim, 0}. */
 cusync_dim3 cusync_attention_grid(uint32_t seq, uint32_t heads);
+/* Grid with the key range split: (heads, row tiles, splits of the longest row tile).  Row tiles that see fewer keys
+ * (causal) leave their surplus splits empty; a tile is posted once, by the split that completes it. */
+cusync_dim3 cusync_attention_grid_split(uint32_t seq, uint32_t heads, uint32_t cached_rows, uint32_t kv_split_blocks);
+size_t cusync_attention_workspace_size(const cusync_attention_args *args);
 cusync_error cusync_attention_can_implement(const cusync_attention_args *args);
 int cusync_attention_max_resident(void);
 /* As a consumer (input policy RowSync, TileSync or ConsecutiveSync over the QKV projection's tiles) the
@@ -344,6 +351,7 @@ typedef struct cusync_attn_layer_config {
   int32_t causal;
   uint32_t cached_rows;        /* key/value cache rows in front of the `seq` new ones (the reference's --seqlen with
                                   --batch new rows, TB/attention.cu:265-276); qkv then has cached_rows + seq rows */
+  int32_t kv_split_blocks;     /* key/value blocks per attention workgroup: -1 = built-in choice, 0 = no split */
 } cusync_attn_layer_config;
 
 typedef struct cusync_attn_layer cusync_attn_layer;

@@ -239,3 +239,64 @@ def test_attention_layer_with_cache(S, cached):
     for sync in (api.SYNC.ROW, api.SYNC.TILE, api.SYNC.STRIDED):
         for got, want, name in zip(outs[sync], outs[api.SYNC.STREAM], ("QKV", "O", "Y")):
             assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (sync, name)
+
+
+# ---- key range split over several workgroups --------------------------------------------------------------
+
+def run_attention_split(qkv, cached, heads, causal, blocks, launches=2, max_workgroups=0):
+    import torch
+    L = _lib.load()
+    S = qkv.shape[0] - cached
+    dq = to_dev(qkv)
+    do = empty_dev((S, heads * 128), fill=float("nan"))
+    grid = api.attention_grid(S, heads, cached, blocks)
+    ws_bytes = api.attention_workspace_size(S, heads, cached, blocks)
+    ws = torch.zeros(max(16, ws_bytes), dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    st = api.Stage(grid, (1, 1, 1), api.no_sync(), api.no_sync())
+    for _ in range(launches):           # the second launch finds the arrival counters re-armed
+        do.fill_(float("nan"))
+        torch.cuda.synchronize()
+        rc = api.attention(st, S, heads, dq.data_ptr(), qkv.shape[1], do.data_ptr(), heads * 128, causal=causal, cached_rows=cached,
+                           kv_split_blocks=blocks, workspace=ws.data_ptr(), max_workgroups=max_workgroups)
+        assert rc == api.ERR.SUCCESS, api.last_error()
+        assert L.cusync_rt_device_sync() == 0, api.last_error()
+    assert st.read_state().tile_counter == 0
+    st.destroy()
+    return to_host(do), grid
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("S,cached,heads,blocks", [(300, 0, 2, 1), (512, 0, 3, 2), (1000, 0, 1, 3), (129, 200, 2, 2), (16, 500, 1, 4),
+                                                   (2048, 0, 2, 8), (64, 0, 1, 8)])
+def test_attention_split_key_range(S, cached, heads, blocks, causal):
+    print("attention split", S, cached, heads, blocks, causal, flush=True)
+    qkv = normal_f16((cached + S, 3 * heads * 128), 21, std=1.0)
+    got, grid = run_attention_split(qkv, cached, heads, causal, blocks)
+    kv_blocks = -(-(cached + S) // 64)
+    assert grid == (heads, (S + 127) // 128, max(1, -(-kv_blocks // blocks)))
+    assert_close(got, orc.attention_kv(qkv, cached, heads, 128, causal), "O")
+    # few workgroups: splits of one tile run one after the other, the last one still puts the tile together
+    got2, _ = run_attention_split(qkv, cached, heads, causal, blocks, launches=1, max_workgroups=2)
+    assert np.array_equal(got.view(np.uint16), got2.view(np.uint16))      # the result does not depend on arrival order
+
+
+def test_attention_split_closed_form():
+    # Q = 0: row i of O is the mean of V rows 0..i, however the key range is cut
+    S, heads = 700, 1
+    rng = np.random.default_rng(6)
+    qkv = normal_f16((S, 3 * 128), 22, std=1.0)
+    qkv[:, :128] = 0
+    v = rng.integers(-4, 5, (S, 128)).astype(np.float16)
+    qkv[:, 256:] = v
+    got, _ = run_attention_split(qkv, 0, heads, True, 2)
+    want = np.cumsum(v.astype(np.float64), axis=0) / np.arange(1, S + 1)[:, None]
+    assert np.max(np.abs(got.astype(np.float32) - want)) < 4e-3
+
+
+def test_attention_split_needs_workspace():
+    st = api.Stage(api.attention_grid(512, 1, 0, 2), (1, 1, 1), api.no_sync(), api.no_sync())
+    dq = to_dev(normal_f16((512, 384), 23)); do = empty_dev((512, 128))
+    a = api.attention_args(st, 512, 1, dq.data_ptr(), 384, do.data_ptr(), 128, kv_split_blocks=2, workspace=None)
+    assert _lib.load().cusync_attention_can_implement(C.byref(a)) != api.ERR.SUCCESS
+    st.destroy()
