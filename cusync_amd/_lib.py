@@ -51,7 +51,7 @@ class Conv2dArgs(C.Structure):
 
 class ConvChainConfig(C.Structure):
     _fields_ = [("N", u32), ("H", u32), ("W", u32), ("C", u32), ("layers", u32), ("sync", i32), ("tile", i32),
-                ("opts", i32), ("relu", i32)]
+                ("opts", i32), ("relu", i32), ("fused", i32)]
 
 
 class AttentionArgs(C.Structure):

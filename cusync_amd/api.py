@@ -228,10 +228,10 @@ class ConvChain:
     """Handle over cusync_conv_chain_*: `layers` dependent 3x3 convolutions, stream-ordered or one CuSync
     stage per layer (src/ml-bench/volta_conv2d/resnet.cu, vgg.cu)."""
 
-    def __init__(self, N, H, W, Cc, weight_ptrs, sync, tile=-1, opts=-1, relu=True):
+    def __init__(self, N, H, W, Cc, weight_ptrs, sync, tile=-1, opts=-1, relu=True, fused=False):
         self.L = _lib.load()
         self.layers = len(weight_ptrs)
-        self.cfg = ConvChainConfig(N, H, W, Cc, self.layers, sync, tile, opts, int(relu))
+        self.cfg = ConvChainConfig(N, H, W, Cc, self.layers, sync, tile, opts, int(relu), int(fused))
         arr = (C.c_void_p * self.layers)(*weight_ptrs)
         self.h = self.L.cusync_conv_chain_create(C.byref(self.cfg), arr)
         if not self.h:

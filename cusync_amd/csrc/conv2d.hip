@@ -33,11 +33,12 @@ struct ConvTile {
   size_t lds;
   void (*kernel)(GemmParams);
   int residentPerCU;
+  void (*chainKernel)(ConvChainParams);     // several layers in one launch; halo tiles only
 };
 
 #define CUSYNC_CONV_TILE(BM, BN, BK, WM, WN, ST, OCC) \
   { BM, BN, BK, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>::LDS_BYTES, \
-    gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>, kAConv>, -1 }
+    gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>, kAConv>, -1, nullptr }
 
 using HaloA = Halo3x3Cfg<256, 64, 4, 1, 4, 2>;     // 64 output channels per tile: four waves of 64 x 64 stacked
 using HaloB = Halo3x3Cfg<128, 128, 2, 2, 3, 1>;    // 128 output channels per tile
@@ -47,8 +48,8 @@ ConvTile g_convTiles[CUSYNC_CONV_TILE_COUNT] = {
   CUSYNC_CONV_TILE(128, 128, 32, 2, 2, 4, 2),   // CUSYNC_CONV_TILE_128x128x32
   CUSYNC_CONV_TILE(256, 64, 32, 4, 1, 3, 2),    // CUSYNC_CONV_TILE_256x64x32
   // the halo tiles: 3x3 / pad 1 / stride 1 only; LDS size depends on the image width and channels
-  { HaloA::BM, HaloA::BN, HaloA::BK, 0, convHalo3x3Kernel<HaloA>, -1 },   // CUSYNC_CONV_TILE_HALO_256x64x64
-  { HaloB::BM, HaloB::BN, HaloB::BK, 0, convHalo3x3Kernel<HaloB>, -1 },   // CUSYNC_CONV_TILE_HALO_128x128x64
+  { HaloA::BM, HaloA::BN, HaloA::BK, 0, convHalo3x3Kernel<HaloA>, -1, convHalo3x3ChainKernel<HaloA> },   // CUSYNC_CONV_TILE_HALO_256x64x64
+  { HaloB::BM, HaloB::BN, HaloB::BK, 0, convHalo3x3Kernel<HaloB>, -1, convHalo3x3ChainKernel<HaloB> },   // CUSYNC_CONV_TILE_HALO_128x128x64
 };
 
 bool isHalo(int tile) { return tile == CUSYNC_CONV_TILE_HALO_256x64x64 || tile == CUSYNC_CONV_TILE_HALO_128x128x64; }
@@ -86,6 +87,14 @@ int residentConv(ConvTile* ti, size_t lds) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, halo ? (int)kMaxLds : (int)lds))) return 0;
     int n = 0;
     if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel, kThreads, lds))) return 0;
+    if (ti->chainKernel) {
+      // the chain kernel is the same code in a loop: it gets the same LDS allowance and must fit as often
+      int m = 0;
+      if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->chainKernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds)) ||
+          CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, ti->chainKernel, kThreads, lds))) return 0;
+      n = std::min(n, m);
+    }
     ti->residentPerCU = n;
     if (halo) g_haloLds[idx] = (uint32_t)lds;
   }
@@ -93,6 +102,32 @@ int residentConv(ConvTile* ti, size_t lds) {
 }
 
 uint32_t outExtent(uint32_t in, uint32_t filter, uint32_t pad, uint32_t stride) { return (in + 2 * pad - filter) / stride + 1; }
+
+// Kernel parameters of one convolution launched with `launched` workgroups.
+GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t launched) {
+  const cusync_stage_desc& s = a->stage;
+  GemmParams p = {};
+  p.stage.d = s;
+  p.cvN = a->N; p.cvH = a->H; p.cvW = a->W; p.cvC = a->C;
+  p.cvP = outExtent(a->H, a->R, a->pad, a->stride);
+  p.cvQ = outExtent(a->W, a->S, a->pad, a->stride);
+  p.cvR = a->R; p.cvS = a->S; p.cvPad = a->pad; p.cvStride = a->stride;
+  p.M = a->N * p.cvP * p.cvQ; p.N = a->K; p.K = a->R * a->S * a->C;
+  p.A = (const half_t*)a->x; p.lda = a->C;
+  p.B = (const half_t*)a->w; p.ldb = p.K;
+  p.D = (half_t*)a->y; p.ldd = a->K;
+  p.epilogue = a->epilogue;
+  p.a_mode = CUSYNC_A_PLAIN;
+  p.launched = launched;
+  p.splitK = 1;
+  p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
+  p.mPad = s.grid.y * ti->bm;
+  // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
+  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
+                        (a->C * 2) % 128 == 0 &&
+                        (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
+  return p;
+}
 
 }  // namespace
 
@@ -176,26 +211,7 @@ cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   uint32_t launched = std::min<uint32_t>(tiles, (uint32_t)resident);
   if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
 
-  GemmParams p = {};
-  p.stage.d = s;
-  p.cvN = a->N; p.cvH = a->H; p.cvW = a->W; p.cvC = a->C;
-  p.cvP = outExtent(a->H, a->R, a->pad, a->stride);
-  p.cvQ = outExtent(a->W, a->S, a->pad, a->stride);
-  p.cvR = a->R; p.cvS = a->S; p.cvPad = a->pad; p.cvStride = a->stride;
-  p.M = a->N * p.cvP * p.cvQ; p.N = a->K; p.K = a->R * a->S * a->C;
-  p.A = (const half_t*)a->x; p.lda = a->C;
-  p.B = (const half_t*)a->w; p.ldb = p.K;
-  p.D = (half_t*)a->y; p.ldd = a->K;
-  p.epilogue = a->epilogue;
-  p.a_mode = CUSYNC_A_PLAIN;
-  p.launched = launched;
-  p.splitK = 1;
-  p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
-  p.mPad = s.grid.y * ti->bm;
-  // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
-  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
-                        (a->C * 2) % 128 == 0 &&
-                        (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
+  GemmParams p = convParams(a, ti, launched);
   hipLaunchKernelGGL(ti->kernel, dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
@@ -247,6 +263,12 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
                   : cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_256x64x32;
   uint32_t tm = 0, tn = 0;
   if (cusync_conv2d_tile_shape(c->cfg.tile, &tm, &tn, nullptr)) { setError("conv chain: unknown tile id"); delete c; return nullptr; }
+  if (c->cfg.fused && cfg->sync != CUSYNC_SYNC_STREAM &&
+      (!isHalo(c->cfg.tile) || cfg->layers > (uint32_t)kMaxFusedLayers || !haloEligible(c->cfg.tile, cfg->W, cfg->C, 3, 3, 1, 1))) {
+    setError("conv chain: one launch for all layers needs a halo tile that fits and at most 8 layers");
+    delete c;
+    return nullptr;
+  }
   const cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);
   if (g.x == 0 || g.y == 0) { setError("conv chain: empty shape"); delete c; return nullptr; }
 
@@ -311,20 +333,54 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
   if (!c || !x || !ys) return CUSYNC_ERROR_NOT_INITIALIZED;
   const uint32_t n = c->cfg.layers;
   const bool overlapped = c->cfg.sync != CUSYNC_SYNC_STREAM;
+  auto layerArgs = [&](uint32_t i) {
+    cusync_conv2d_args a;
+    memset(&a, 0, sizeof a);
+    a.stage = c->st[i];
+    a.N = c->cfg.N; a.H = c->cfg.H; a.W = c->cfg.W; a.C = c->cfg.C; a.K = c->cfg.C;
+    a.R = a.S = 3; a.pad = 1; a.stride = 1;
+    a.x = i == 0 ? x : ys[i - 1];
+    a.w = c->w[i];
+    a.y = ys[i];
+    a.epilogue = (c->cfg.relu && i + 1 < n) ? CUSYNC_EPILOGUE_RELU : CUSYNC_EPILOGUE_NONE;
+    a.tile = c->cfg.tile;
+    return a;
+  };
+  if (overlapped && c->cfg.fused) {
+    // all layers in one launch on the first stream
+    ConvTile* ti = convTile(c->cfg.tile);
+    const size_t lds = haloLds(c->cfg.tile, c->cfg.W, c->cfg.C);
+    const int resident = residentConv(ti, lds);
+    if (resident <= 0) { cusync::rt::setError("conv chain: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
+    const cusync_dim3& g = c->st[0].grid;
+    const uint32_t launched = std::min<uint32_t>(g.x * g.y * g.z, (uint32_t)resident);
+    for (int r = 0; r < runs; r++) {
+      ConvChainParams cp = {};
+      cp.layers = n;
+      for (uint32_t i = 0; i < n; i++) {
+        const cusync_conv2d_args a = layerArgs(i);
+        const cusync_error e = cusync_conv2d_can_implement(&a);
+        if (e != CUSYNC_SUCCESS) return e;
+        cp.layer[i] = convParams(&a, ti, launched);
+      }
+      if (CUSYNC_HIP(hipEventRecord(c->ev[0], c->stream[0]))) return CUSYNC_ERROR_DEVICE;
+      hipLaunchKernelGGL(ti->chainKernel, dim3(launched), dim3(kThreads), lds, c->stream[0], cp);
+      if (CUSYNC_HIP(hipGetLastError()) || CUSYNC_HIP(hipEventRecord(c->ev[n], c->stream[0])) ||
+          CUSYNC_HIP(hipEventSynchronize(c->ev[n]))) return CUSYNC_ERROR_DEVICE;
+      float ms = 0;
+      if (times_us) {
+        if (CUSYNC_HIP(hipEventElapsedTime(&ms, c->ev[0], c->ev[n]))) return CUSYNC_ERROR_DEVICE;
+        times_us[r] = (double)ms * 1000.0;
+      }
+      for (uint32_t i = 0; i < n; i++) c->st[i].iter += 1;
+    }
+    return CUSYNC_SUCCESS;
+  }
   for (int r = 0; r < runs; r++) {
     if (CUSYNC_HIP(hipEventRecord(c->ev[0], c->stream[0]))) return CUSYNC_ERROR_DEVICE;
     for (uint32_t i = 0; i < n; i++) {
       hipStream_t s = c->stream[overlapped ? i : 0];
-      cusync_conv2d_args a;
-      memset(&a, 0, sizeof a);
-      a.stage = c->st[i];
-      a.N = c->cfg.N; a.H = c->cfg.H; a.W = c->cfg.W; a.C = c->cfg.C; a.K = c->cfg.C;
-      a.R = a.S = 3; a.pad = 1; a.stride = 1;
-      a.x = i == 0 ? x : ys[i - 1];
-      a.w = c->w[i];
-      a.y = ys[i];
-      a.epilogue = (c->cfg.relu && i + 1 < n) ? CUSYNC_EPILOGUE_RELU : CUSYNC_EPILOGUE_NONE;
-      a.tile = c->cfg.tile;
+      const cusync_conv2d_args a = layerArgs(i);
       cusync_error e;
       if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
       if ((e = cusync_conv2d_run(&a, s)) != CUSYNC_SUCCESS) return e;

@@ -44,8 +44,9 @@ struct Halo3x3Cfg {
   }
 };
 
+// One layer: all tiles of stage p.stage that this workgroup draws.
 template<class C>
-__global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams p) {
+__device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   __shared__ uint32_t sTicket, sLast;
 
@@ -208,6 +209,32 @@ __global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams
     cusync_dim3 done = {m0, n0, 0};
     if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();
+  }
+}
+
+template<class C>
+__global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams p) {
+  convHalo3x3Layer<C>(p);
+}
+
+// A chain of layers in ONE launch: every workgroup works through the tiles of layer 0 it can draw, then those
+// of layer 1, and so on; a tile of layer l+1 waits on the semaphores of layer l exactly as it does when the
+// layers are separate launches.  No wait kernel and no second launch sit between a producer and its consumer
+// (on this device the first dispatch on another stream starts 15-20 us after the producer did, about as long
+// as a whole 3x3 layer of the ResNet shapes takes).  Forward progress: the launch has no more workgroups than
+// stay resident, and a workgroup only moves on to layer l+1 when layer l has no tile left to hand out, so every
+// tile a consumer tile waits for is already in the hands of a running workgroup.
+constexpr int kMaxFusedLayers = 8;
+struct ConvChainParams {
+  GemmParams layer[kMaxFusedLayers];
+  uint32_t layers;
+};
+
+template<class C>
+__global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3ChainKernel(ConvChainParams cp) {
+  for (uint32_t l = 0; l < cp.layers; l++) {
+    convHalo3x3Layer<C>(cp.layer[l]);
+    __syncthreads();        // everyone has read the last ticket of this layer before the next one's is written
   }
 }
 

@@ -285,6 +285,9 @@ typedef struct cusync_conv_chain_config {
   int32_t tile;                /* CUSYNC_CONV_TILE_*, -1 = built-in choice */
   int32_t opts;                /* extra CUSYNC_OPT_* bits, -1 = none */
   int32_t relu;                /* 1: ReLU after every layer but the last */
+  int32_t fused;               /* 1 (sync ROW or TILE, halo tiles, at most 8 layers): all layers in ONE launch whose workgroups
+                                  work through layer 0, then layer 1, ... with the same semaphores between them; no wait
+                                  kernel and no second launch between a producer and its consumer */
 } cusync_conv_chain_config;
 
 typedef struct cusync_conv_chain cusync_conv_chain;

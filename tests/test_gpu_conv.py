@@ -283,3 +283,31 @@ def test_conv_chain_all_sync_modes(shape, layers):
     for sync in (api.SYNC.ROW, api.SYNC.TILE):
         for i in range(layers):
             assert np.array_equal(outs[sync][i].view(np.uint16), ys[i].view(np.uint16)), (sync, i)
+
+
+@pytest.mark.parametrize("shape,layers", [((4, 20, 20, 64), 2), ((32, 56, 56, 64), 2), ((32, 28, 28, 128), 2),
+                                          ((2, 24, 24, 64), 4), ((16, 56, 56, 64), 4), ((8, 28, 28, 128), 8)])
+@pytest.mark.parametrize("sync", [api.SYNC.ROW, api.SYNC.TILE])
+def test_conv_chain_in_one_launch(shape, layers, sync):
+    # all layers in one launch: same semaphores, same results bit for bit as the stream-ordered chain
+    print("conv chain, one launch", shape, layers, sync, flush=True)
+    x, ws, want, _, _, _ = run_chain(*shape, layers, api.SYNC.STREAM, runs=1)
+    _, _, got, states, tile, _ = run_chain(*shape, layers, sync, runs=3, fused=True)
+    tm, tn, _ = api.conv2d_tile_shape(tile)
+    for i, st in enumerate(states):
+        assert st.spin_timeouts == 0 and st.tile_counter == 0 and st.start_counter == 0
+        if i + 1 < layers:
+            d = st.desc
+            p = orc.Policy(d.out.kind, d.out.order, d.out.tileM, d.out.tileN, d.out.waitValue, d.out.postValue,
+                           d.out.gridN, d.out.stride, d.out.R, d.out.S, d.out.H)
+            assert np.array_equal(st.sems, orc.expected_sems_gemm(p, st.grid, tm, tn, 3, d.opts))
+    for i in range(layers):
+        assert np.array_equal(got[i].view(np.uint16), want[i].view(np.uint16)), i
+
+
+def test_conv_chain_in_one_launch_rejects():
+    import torch
+    w = [to_dev(he_filters(64, 3, 3, 64, 1)) for _ in range(2)]
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError):      # the implicit-GEMM tiles have no chain kernel
+        api.ConvChain(4, 20, 20, 64, [t.data_ptr() for t in w], api.SYNC.ROW, tile=api.CONV_TILE.T256x64x32, fused=True)
