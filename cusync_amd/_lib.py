@@ -68,7 +68,7 @@ class AttnLayerConfig(C.Structure):
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
                 ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
-                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32)]
+                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32), ("one_launch", i32)]
 
 
 # every symbol include/cusync_amd.h declares: name -> (restype, argtypes)
@@ -110,6 +110,7 @@ SIGNATURES = {
     "cusync_gemm_can_implement": (C.c_int, [C.POINTER(GemmArgs)]),
     "cusync_gemm_workspace_size": (sz, [C.POINTER(GemmArgs)]),
     "cusync_gemm_max_resident": (C.c_int, [C.c_int]),
+    "cusync_gemm_chain_run": (C.c_int, [C.POINTER(GemmArgs), C.c_int, vp]),
     "cusync_gemm_run": (C.c_int, [C.POINTER(GemmArgs), vp]),
     "cusync_conv2d_tile_shape": (C.c_int, [C.c_int, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_conv2d_grid": (Dim3, [C.c_int, u32, u32, u32, u32, u32, u32, u32, u32]),

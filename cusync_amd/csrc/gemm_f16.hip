@@ -48,16 +48,17 @@ struct TileInfo {
   size_t lds;
   void (*kernel[2])(GemmParams);   // [plain A, SwiGLU A]
   int residentPerCU;     // filled lazily
+  void (*chainKernel)(GemmChainParams);   // several dependent GEMMs in one launch; direct-to-LDS tiles only
 };
 
 #define CUSYNC_TILE(BM, BN, BK, WM, WN) \
   { BM, BN, BK, kThreads, (size_t)TileCfg<BM, BN, BK, WM, WN>::LDS_BYTES, \
-    { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1 }
+    { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1, nullptr }
 
 // Direct-to-LDS tiles have no SwiGLU variant (that operand needs arithmetic on its way into LDS).
 #define CUSYNC_TILE_DMA(...) \
   { DmaCfg<__VA_ARGS__>::BM, DmaCfg<__VA_ARGS__>::BN, DmaCfg<__VA_ARGS__>::BK, DmaCfg<__VA_ARGS__>::THREADS, \
-    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1 }
+    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1, gemmDmaChainKernel<DmaCfg<__VA_ARGS__>> }
 
 TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
   CUSYNC_TILE_DMA(256, 256, 32, 4, 2, 4, 2, false, true),   // CUSYNC_TILE_256x256x32: direct-to-LDS, eight wavefronts of 64x128, 4 stages, one workgroup per CU
@@ -104,6 +105,13 @@ int residentWorkgroups(int tile) {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds))) return 0;
       int n = 0;
       if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel[v], (int)ti->threads, ti->lds))) return 0;
+      perCU = std::min(perCU, n);
+    }
+    if (ti->chainKernel) {
+      int n = 0;
+      if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->chainKernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds)) ||
+          CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->chainKernel, (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
     }
     ti->residentPerCU = perCU;
@@ -187,24 +195,9 @@ static size_t partialBytes(const cusync_gemm_args* a, const TileInfo* ti) {
   return (size_t)a->split_k * g.y * g.x * ti->bm * ti->bn * sizeof(float);
 }
 
-size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {
-  TileInfo* ti = a ? tileInfo(a->tile) : nullptr;
-  if (!ti || a->split_k <= 1) return 0;
-  const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
-  return partialBytes(a, ti) + (size_t)g.x * g.y * sizeof(uint32_t);
-}
-
-cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
-  cusync_error e = cusync_gemm_can_implement(a);
-  if (e != CUSYNC_SUCCESS) return e;
-  TileInfo* ti = tileInfo(a->tile);
-  const int resident = residentWorkgroups(a->tile);
-  if (resident <= 0) { cusync::rt::setError("gemm: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
+// Kernel parameters of one GEMM launched with `launched` workgroups.
+static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint32_t launched) {
   const cusync_stage_desc& s = a->stage;
-  const uint32_t tiles = s.grid.x * s.grid.y * s.grid.z;
-  uint32_t launched = std::min<uint32_t>(tiles, (uint32_t)resident);
-  if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
-
   GemmParams p;
   p.stage.d = s;
   // Producer tiles are whole 128-byte lines of A when the row pitch, the base and
@@ -225,7 +218,56 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   p.mPad = s.grid.y * ti->bm;
   p.partials = (float*)a->workspace;
   p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
+  return p;
+}
+
+size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {
+  TileInfo* ti = a ? tileInfo(a->tile) : nullptr;
+  if (!ti || a->split_k <= 1) return 0;
+  const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
+  return partialBytes(a, ti) + (size_t)g.x * g.y * sizeof(uint32_t);
+}
+
+cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
+  cusync_error e = cusync_gemm_can_implement(a);
+  if (e != CUSYNC_SUCCESS) return e;
+  TileInfo* ti = tileInfo(a->tile);
+  const int resident = residentWorkgroups(a->tile);
+  if (resident <= 0) { cusync::rt::setError("gemm: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
+  const cusync_stage_desc& s = a->stage;
+  const uint32_t tiles = s.grid.x * s.grid.y * s.grid.z;
+  uint32_t launched = std::min<uint32_t>(tiles, (uint32_t)resident);
+  if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
+
+  const GemmParams p = gemmParams(a, ti, launched);
   hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
+  if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_gemm_chain_run(const cusync_gemm_args* args, int count, void* stream) {
+  using cusync::rt::setError;
+  if (!args || count < 1 || count > kMaxChainedGemms) { setError("gemm chain: 1 to 4 GEMMs"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  TileInfo* ti = tileInfo(args[0].tile);
+  if (!ti || !ti->chainKernel) { setError("gemm chain: needs a direct-to-LDS tile"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  const int resident = residentWorkgroups(args[0].tile);
+  if (resident <= 0) { setError("gemm: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
+  uint32_t launched = (uint32_t)resident;
+  for (int i = 0; i < count; i++) {
+    const cusync_gemm_args& a = args[i];
+    if (a.tile != args[0].tile) { setError("gemm chain: all GEMMs must use the same tile"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (a.a_mode != CUSYNC_A_PLAIN) { setError("gemm chain: plain A operands only"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    const cusync_error e = cusync_gemm_can_implement(&a);
+    if (e != CUSYNC_SUCCESS) return e;
+    if (a.stage.in.kind != CUSYNC_POLICY_NOSYNC && i == 0) { setError("gemm chain: the first GEMM cannot wait on a stage outside the launch"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    // never more workgroups than any of the GEMMs has tiles: a workgroup without a tile of GEMM i would run ahead
+    launched = std::min<uint32_t>(launched, a.stage.grid.x * a.stage.grid.y * a.stage.grid.z);
+    if (a.max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a.max_workgroups);
+  }
+  GemmChainParams cp = {};
+  cp.count = (uint32_t)count;
+  for (int i = 0; i < count; i++) cp.gemm[i] = gemmParams(&args[i], ti, launched);
+  hipLaunchKernelGGL(ti->chainKernel, dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, cp);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }

@@ -92,8 +92,9 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
   return r;
 }
 
-template<class C, int AMODE = kAPlain>
-__global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
+// One GEMM: all tiles of stage p.stage that this workgroup draws.
+template<class C, int AMODE>
+__device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   constexpr bool conv = AMODE == kAConv;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   __shared__ uint32_t sTicket, sLast;
@@ -484,6 +485,32 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
     cusync_dim3 done = {m0, n0, t.z};
     if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();
+  }
+}
+
+template<class C, int AMODE = kAPlain>
+__global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
+  gemmDmaTiles<C, AMODE>(p);
+}
+
+// Dependent GEMMs of one tile shape in ONE launch: every workgroup works through the tiles of the first
+// GEMM it can draw, then those of the second, and so on; a tile of a later GEMM waits on the semaphores
+// of the one before exactly as it does when they are separate launches.  No kernel boundary, wait
+// kernel or second launch sits between producer and consumer, which is what a chain of short GEMMs
+// (few rows: 30 us in the kernel, 10 us around it) pays most for.  Forward progress: the launch has
+// no more workgroups than stay resident, and a workgroup only moves on when the GEMM it is on has no
+// tile left to hand out, so every tile a consumer tile waits for is in the hands of a running workgroup.
+constexpr int kMaxChainedGemms = 4;
+struct GemmChainParams {
+  GemmParams gemm[kMaxChainedGemms];
+  uint32_t count;
+};
+
+template<class C>
+__global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaChainKernel(GemmChainParams cp) {
+  for (uint32_t g = 0; g < cp.count; g++) {
+    gemmDmaTiles<C, kAPlain>(cp.gemm[g]);
+    __syncthreads();        // everyone has read the last ticket of this GEMM before the next one's is written
   }
 }
 

@@ -177,6 +177,16 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       return nullptr;
   }
   if (cfg->opts >= 0) opts |= cfg->opts;
+  if (cfg->one_launch && sync != CUSYNC_SYNC_STREAM) {
+    uint32_t bk = 0;
+    cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk);
+    const bool direct = bk == 32 || m->tile1 >= CUSYNC_TILE_D32x128x64;      // the direct-to-LDS tiles
+    if (m->tile1 != m->tile2 || !direct || m->aMode2 != CUSYNC_A_PLAIN) {
+      setError("mlp: one launch for both GEMMs needs the same direct-to-LDS tile for both and a plain A operand");
+      delete m;
+      return nullptr;
+    }
+  }
 
   memset(&m->prod, 0, sizeof m->prod);
   memset(&m->cons, 0, sizeof m->cons);
@@ -235,8 +245,14 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     cusync_gemm_args a2 = gemmArgs(m, 1, x, h, y);
     cusync_error e;
     if (CUSYNC_HIP(hipEventRecord(m->eStart, m->sProd))) return CUSYNC_ERROR_DEVICE;
-    if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) return e;
-    if (overlapped) {
+    if (overlapped && m->cfg.one_launch) {
+      // both GEMMs in one launch: same stages and semaphores, no wait kernel, no second launch
+      const cusync_gemm_args both[2] = {a1, a2};
+      if ((e = cusync_gemm_chain_run(both, 2, m->sProd)) != CUSYNC_SUCCESS) return e;
+      if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sProd))) return CUSYNC_ERROR_DEVICE;
+    } else if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) {
+      return e;
+    } else if (overlapped) {
       if ((e = cusync_invoke_wait_kernel(&m->prod, m->sCons)) != CUSYNC_SUCCESS) return e;
       if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;
       if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sCons))) return CUSYNC_ERROR_DEVICE;

@@ -233,6 +233,13 @@ size_t cusync_gemm_workspace_size(const cusync_gemm_args *args);
 int cusync_gemm_max_resident(int tile);
 /* run(stream) (cusyncgemm.h:525-563).  args->stage.iter selects the run. */
 cusync_error cusync_gemm_run(const cusync_gemm_args *args, void *stream);
+/* `count` (1..4) dependent GEMMs of one direct-to-LDS tile shape in ONE launch: every workgroup works through the
+ * tiles of args[0] it can draw, then those of args[1], ...; a tile of args[i] waits on the semaphores args[i-1]
+ * posts, exactly as in separate launches (the stages are created and paired the same way), but no kernel boundary,
+ * wait kernel or second launch sits in between.  No counterpart in the reference, whose consumer is always a launch
+ * of its own; here a first dispatch on another stream starts 15-20 us after the producer did, which chains of
+ * short kernels cannot afford.  args[0] must not wait on a stage outside the launch. */
+cusync_error cusync_gemm_chain_run(const cusync_gemm_args *args, int count, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Sync-aware NHWC forward convolution as an implicit GEMM (replaces           */
@@ -393,6 +400,8 @@ typedef struct cusync_mlp_config {
   int32_t split_k1, split_k2;  /* k-slices per GEMM (--split-k1/--split-k2, TB/mlp.cu:880-931); 0 = pick so that
                                   the launch fills the device */
   int32_t max_wg1, max_wg2;    /* workgroups per launch of each GEMM; 0 = built-in choice, -1 = as many as stay resident */
+  int32_t one_launch;          /* 1 (with a CuSync mode): both GEMMs in one launch, cusync_gemm_chain_run; needs the same
+                                  direct-to-LDS tile for both and a plain A operand in GEMM2 */
 } cusync_mlp_config;
 
 typedef struct cusync_mlp cusync_mlp;   /* opaque */

@@ -139,3 +139,28 @@ def test_strided_sync_rejects_unaligned_split():
     with pytest.raises(RuntimeError, match="inner % tileN"):
         api.Mlp(api.MODEL.LLAMA, 256, 8192, 2752, api.SYNC.STRIDED, w.data_ptr(), w.data_ptr(),
                 tile1=api.TILE.T256x128x64)
+
+
+@pytest.mark.parametrize("batch", [1, 16, 64, 256, 512, 1024, 2048])
+@pytest.mark.parametrize("sync", [api.SYNC.ROW, api.SYNC.TILE])
+def test_gpt3_mlp_in_one_launch(batch, sync):
+    # both GEMMs in one launch: same stages and semaphores, results bit for bit those of the stream-ordered pair
+    print("gpt3 one launch", batch, sync, flush=True)
+    _, _, _, h0, y0, _, _, tiles0, _ = run_mlp(api.MODEL.GPT3, batch, sync=api.SYNC.STREAM, runs=1, **GPT3)
+    x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.GPT3, batch, sync=sync, runs=3, one_launch=True, **GPT3)
+    assert tiles == tiles0
+    assert cons.spin_timeouts == 0
+    assert prod.tile_counter == 0 and cons.tile_counter == 0
+    assert np.array_equal(prod.sems, expected_sems(prod, tiles, 3))
+    assert np.array_equal(h.view(np.uint16), h0.view(np.uint16))
+    assert np.array_equal(y.view(np.uint16), y0.view(np.uint16))
+
+
+def test_mlp_in_one_launch_rejects():
+    w1, w2, dw1, dw2 = weights(api.MODEL.GPT3, 12288, 6144)
+    with pytest.raises(RuntimeError):       # two different tiles cannot share a launch
+        api.Mlp(api.MODEL.GPT3, 256, 12288, 6144, api.SYNC.ROW, dw1.data_ptr(), dw2.data_ptr(),
+                tile1=api.TILE.T128x192x32, tile2=api.TILE.T128x128x32, one_launch=True)
+    with pytest.raises(RuntimeError):       # the register-staged tiles have no chain kernel
+        api.Mlp(api.MODEL.GPT3, 256, 12288, 6144, api.SYNC.ROW, dw1.data_ptr(), dw2.data_ptr(),
+                tile1=api.TILE.T128x128x64, tile2=api.TILE.T128x128x64, one_launch=True)
