@@ -159,6 +159,13 @@ def load():
             "cusync_amd: %s is missing — the HIP library has not been built "
             "(run `make -C cusync_amd/csrc` or __graft_entry__.build()). "
             "There is no CPU fallback." % LIB_PATH)
+    # PyTorch ships a HIP runtime of its own.  Whichever copy is loaded first serves the whole process, and the
+    # tensors handed to this library come from PyTorch's: let it load first (measured the other way round: the
+    # occupancy query answers 0 workgroups per CU for every kernel that needs more than 64 KB of LDS).
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
     for name, (res, args) in SIGNATURES.items():
         f = getattr(L, name)          # AttributeError if the symbol is not exported

@@ -198,7 +198,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     uint32_t bVoff0[C::B_LOADS];
 #pragma unroll
     for (int q = 0; q < C::B_LOADS; q++) {
-      if constexpr (C::BT) bVoff0[q] = ((n0 + bLoadRow[q]) * p.ldb + bLoadChunk[q] * 8) * 2;     // rows past N fall outside the buffer
+      if constexpr (C::BT) bVoff0[q] = bLoadRow[q] < C::B_ROWS ? ((n0 + bLoadRow[q]) * p.ldb + bLoadChunk[q] * 8) * 2 : kOutOfRange;     // rows past N fall outside the buffer
       else bVoff0[q] = (bLoadRow[q] < C::B_ROWS && n0 + bLoadChunk[q] * 8 < p.N) ? (bLoadRow[q] * p.ldb + n0 + bLoadChunk[q] * 8) * 2 : kOutOfRange;
     }
 
@@ -284,9 +284,9 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       const uint32_t k0 = kBegin + kt * C::BK;
       if constexpr (Q < C::B_LOADS) {
         uint32_t lds = ldsBase + C::STAGES * C::A_STAGE + S * C::B_STAGE + (wave * C::B_LOADS + Q) * 1024;
-        if constexpr (C::DUMP) { static_assert(!C::BT, "spare loads are resolved for row-major B only"); if (wave * C::B_LOADS + Q >= C::B_TOTAL) lds = ldsBase + C::DUMP_OFFSET; }
+        if constexpr (C::DUMP) { if (wave * C::B_LOADS + Q >= C::B_TOTAL) lds = ldsBase + C::DUMP_OFFSET; }
         uint32_t off;
-        if constexpr (C::BT) off = k0 + bLoadChunk[Q] * 8 < kEnd ? bVoff0[Q] + k0 * 2 : kOutOfRange;
+        if constexpr (C::BT) off = (bVoff0[Q] != kOutOfRange && k0 + bLoadChunk[Q] * 8 < kEnd) ? bVoff0[Q] + k0 * 2 : kOutOfRange;
         else off = (bVoff0[Q] != kOutOfRange && k0 < kEnd) ? bVoff0[Q] + k0 * p.ldb * 2 : kOutOfRange;
         loadToLds(rB, __builtin_amdgcn_readfirstlane(lds), off);
       } else {
