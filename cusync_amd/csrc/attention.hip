@@ -186,9 +186,14 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   // 128x128 up to 1024 rows, 128x256 above.
   const int small = cfg->seq <= 32 ? CUSYNC_TILE_D32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  const int wide = cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64 : CUSYNC_TILE_128x192x32;
-  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide : dflt;
-  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide : dflt;
+  // 128x192: with a CU to itself, four stages and the pipelined order while the GEMM has about one tile per CU
+  // (QKV projection, 24 column tiles: up to 1024 rows; output projection, 64: up to 512), else two per CU
+  auto wide = [&](uint32_t aloneUpTo) {
+    return cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64
+           : cfg->seq <= aloneUpTo ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_128x192x32;
+  };
+  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide(1024) : dflt;
+  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide(512) : dflt;
   L->ws1 = L->ws3 = L->ws2 = nullptr;
   // Key ranges of 16 blocks (1024 rows) or more are cut in two.  Measured alone at 12 heads: 1024 rows 40 -> 35 us,
   // 2048 rows 73 -> 65 us; finer cuts lose again (four: 71 us, eight: 124 us) — the kernel is bound by the softmax

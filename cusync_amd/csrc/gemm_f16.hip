@@ -79,6 +79,7 @@ TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
   CUSYNC_TILE_DMA(32, 128, 64, 1, 4, 4, 2),     // CUSYNC_TILE_D32x128x64: 60 KB of loads in flight per workgroup
   CUSYNC_TILE_DMA(64, 128, 64, 1, 4, 3, 2),     // CUSYNC_TILE_D64x128x64
   CUSYNC_TILE_DMA(64, 192, 64, 2, 2, 4, 1),     // CUSYNC_TILE_D64x192x64: 96 KB of loads in flight per CU
+  CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 4, 2, false, true),   // CUSYNC_TILE_128x192x32_ALONE: 80 KB of LDS, so one workgroup per CU
 };
 
 std::mutex g_mutex;

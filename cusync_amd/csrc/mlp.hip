@@ -47,16 +47,17 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   else small = CUSYNC_TILE_128x128x64;
   const bool big = c.batch > 128;
   // Measured on the GPT-3 shard.  Where the width is a multiple of 192 (6144 and 12288 columns are 32 and
-  // 64 tiles: whole rounds on 256 CUs) the 192-wide direct-to-LDS tiles win from 256 rows on: 128x192 at two
-  // workgroups per CU up to 768 rows, 256x192 with a CU to itself above (8 % faster at 1024 and 2048 rows;
-  // at 512 rows it is as fast stream-ordered but leaves a consumer launched next to it nowhere to run).
+  // 64 tiles: whole rounds on 256 CUs) the 192-wide direct-to-LDS tiles win from 256 rows on.  GEMM1: 256x192
+  // with a CU to itself (8 % faster than 128x192 at two workgroups per CU at 1024 and 2048 rows; below that the
+  // k-slices fill the device).  GEMM2: the same from 513 rows on; up to 512 rows, where it has at most one 128-row
+  // tile per CU, 128x192 with four stages in the pipelined order (384 rows: 258 -> 225 us, 512 rows: 254 -> 235 us
+  // for the pair against 128x192 at two workgroups per CU for both).
   // Other widths: 128x128 up to 1024 rows (more tiles to spread), 128x256 above.
   const uint32_t n1 = c.model == CUSYNC_MLP_LLAMA ? 2 * c.inner : c.inner, n2 = c.hidden;
-  const int wide = c.batch > 768 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  if (big && n1 % 192 == 0) a = wide;
-  if (big && n2 % 192 == 0 && !swiglu) b = wide;
+  if (big && n1 % 192 == 0) a = CUSYNC_TILE_256x192x32;
+  if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 512 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32_ALONE;
   // Up to 256 rows the GEMMs are bound by streaming the weights: direct-to-LDS tiles with 60-96 KB of loads
   // in flight per workgroup (measured: 104 -> 85 us at 1-32 rows, 127 -> 101 us at 64, 187 -> 158 us at 256).
   // 64x192 makes 32 or 64 column tiles, which 8 or 4 k-slices turn into one workgroup per CU.
@@ -71,6 +72,8 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
     a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
   *t2 = c.tile2 >= 0 ? c.tile2 : b;
+  // both GEMMs in one launch share a kernel: the consumer takes the producer's tile
+  if (c.one_launch && sync != CUSYNC_SYNC_STREAM && c.tile2 < 0 && !swiglu) *t2 = *t1;
 }
 
 cusync_policy_desc noSync() {

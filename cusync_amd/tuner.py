@@ -27,7 +27,7 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
          api.TILE.T256x64x64: (4, 1, 2), api.TILE.T128x64x64: (2, 2, 2), api.TILE.T256x128x32: (2, 2, 3),
          api.TILE.T128x256x32: (2, 2, 3), api.TILE.T128x128x32: (2, 2, 3), api.TILE.T128x192x32: (2, 2, 3),
          api.TILE.T256x192x32: (4, 2, 4), api.TILE.D32x128x64: (1, 4, 4), api.TILE.D64x128x64: (1, 4, 3),
-         api.TILE.D64x192x64: (2, 2, 4)}
+         api.TILE.D64x192x64: (2, 2, 4), api.TILE.T128x192x32_ALONE: (2, 2, 4)}
 
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 
@@ -41,10 +41,10 @@ def candidates(batch, n1, n2):
     elif batch <= 128:
         tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x128x64, api.TILE.T128x128x32], [1, 2, 4, 8]
     elif batch <= 512:
-        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x128x32, api.TILE.T128x192x32, api.TILE.T256x128x32, api.TILE.T128x256x32], [1, 2, 4]
+        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4]
     else:
         tiles, splits = [api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
-    ok = lambda t, n: n % 192 == 0 or t not in (api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.D64x192x64)
+    ok = lambda t, n: n % 192 == 0 or t not in (api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE)
     return [(t, s) for t in tiles for s in splits if ok(t, n1)], [(t, s) for t in tiles for s in splits if ok(t, n2)]
 
 

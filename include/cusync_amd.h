@@ -202,7 +202,8 @@ enum {
   CUSYNC_TILE_D32x128x64 = 13,       /* direct-to-LDS, 4 stages: few rows, bound by streaming the weights */
   CUSYNC_TILE_D64x128x64 = 14,       /* direct-to-LDS, 3 stages */
   CUSYNC_TILE_D64x192x64 = 15,       /* direct-to-LDS, 4 stages, a CU to itself: 32 or 64 column tiles times 8 or 4 k-slices are 256 */
-  CUSYNC_TILE_COUNT = 16
+  CUSYNC_TILE_128x192x32_ALONE = 16, /* 128x192x32 with 4 stages in the pipelined order and a CU to itself: for GEMMs of about one tile per CU */
+  CUSYNC_TILE_COUNT = 17
 };
 
 typedef struct cusync_gemm_args {

@@ -146,8 +146,11 @@ def test_strided_sync_rejects_unaligned_split():
 def test_gpt3_mlp_in_one_launch(batch, sync):
     # both GEMMs in one launch: same stages and semaphores, results bit for bit those of the stream-ordered pair
     print("gpt3 one launch", batch, sync, flush=True)
-    _, _, _, h0, y0, _, _, tiles0, _ = run_mlp(api.MODEL.GPT3, batch, sync=api.SYNC.STREAM, runs=1, **GPT3)
     x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.GPT3, batch, sync=sync, runs=3, one_launch=True, **GPT3)
+    assert tiles[0] == tiles[1]            # one kernel for both
+    # the same tiles and k-slices as two stream-ordered launches
+    _, _, _, h0, y0, _, _, tiles0, _ = run_mlp(api.MODEL.GPT3, batch, sync=api.SYNC.STREAM, runs=1, tile1=tiles[0], tile2=tiles[1],
+                                               split_k1=tiles[2], split_k2=tiles[3], **GPT3)
     assert tiles == tiles0
     assert cons.spin_timeouts == 0
     assert prod.tile_counter == 0 and cons.tile_counter == 0
