@@ -68,7 +68,7 @@ class AttnLayerConfig(C.Structure):
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
                 ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
-                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32), ("one_launch", i32)]
+                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32), ("one_launch", i32), ("swiglu_in_gemm2", i32)]
 
 
 # every symbol include/cusync_amd.h declares: name -> (restype, argtypes)

@@ -14,6 +14,7 @@
 #include "../../include/cusync_amd.h"
 #include "rt_internal.h"
 #include "split_choice.h"
+#include "gemm_common.h"
 
 struct cusync_mlp {
   cusync_mlp_config cfg;
@@ -29,12 +30,108 @@ struct cusync_mlp {
   cusync_stage_desc prod, cons;
   hipStream_t sProd, sCons;
   hipEvent_t eStart, eMid, eEnd;
+  // LLaMA with the activation as a stage of its own between the GEMMs: silu(gate) * up, once per element
+  bool actStage;
+  void* act;                         // [batch][inner] fp16, GEMM2's A operand
+  cusync_stage_desc mid;
+  hipStream_t sMid;
 };
 
 namespace {
 
 using cusync::rt::setError;
 using cusync::gemm::pickSplit;
+using cusync::gemm::half_t;
+using cusync::gemm::uint4v;
+
+// ---- silu(gate) * up as a CuSync stage ------------------------------------------------------------
+// A = silu(G[:, 0:d]) * G[:, d:2d] in tiles of 128 x 128.  As a consumer of GEMM1 a tile waits for the
+// producer tiles that hold its gate and its up columns (under StridedSync both map to one semaphore
+// that counts to two); as a producer for GEMM2 it posts the tile.  Fused into GEMM2's A loader the
+// same arithmetic is repeated once per column tile of GEMM2 (64 times for the LLaMA shard) and makes
+// that kernel three times slower; here every element is computed once.
+constexpr uint32_t kActM = 128, kActN = 128, kActThreads = 256;
+
+struct ActParams {
+  cusync::DynStage stage;
+  uint32_t M, d;                 // rows, columns of A (= inner)
+  const half_t* G; uint32_t ldg; // gate | up, [M][ldg]
+  half_t* A; uint32_t lda;
+  uint32_t launched;
+};
+
+__global__ __launch_bounds__(kActThreads) void swigluStageKernel(ActParams p) {
+  __shared__ uint32_t sTicket;
+  const cusync::DynStage& stage = p.stage;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t numTiles = stage.numTiles();
+  const bool consumer = stage.isConsumer();
+  const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
+  // the row policies mark their waits with z = 1, the tile policies with z = 0
+  const uint32_t zWait = consumer && stage.d.in.kind == CUSYNC_POLICY_ROWSYNC ? 1 : 0;
+  uint32_t dryXcds = 0, nextRaw = 0;
+  const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
+  const bool noDraws = stage.allStatic(p.launched);
+  for (uint32_t round = 0;; round++) {
+    if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
+    __syncthreads();
+    const uint32_t ticket = sTicket;
+    if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+    if (ticket >= numTiles) break;
+    const cusync_dim3 t = stage.ticketToTile(ticket);
+    const uint32_t m0 = t.y * kActM, c0 = t.x * kActN;
+    const uint32_t mEnd = min(m0 + kActM, p.M), cEnd = min(c0 + kActN, p.d);
+    if (consumer) {
+      if (tid < 64) {          // one wavefront waits for everybody
+        for (uint32_t r = m0; r < mEnd; r = (r / tmq + 1) * tmq)
+          for (uint32_t half = 0; half < 2; half++)
+            for (uint32_t c = (half * p.d + c0) / tnq * tnq; c < half * p.d + cEnd; c += tnq) {
+              cusync_dim3 w = {r, c, zWait};
+              stage.waitWave(w);
+              if (zWait) break;             // a row policy guards whole rows: one wait per row block
+            }
+      }
+      __syncthreads();
+    }
+    if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the tile
+#pragma unroll
+    for (uint32_t i = 0; i < kActM * kActN / 8 / kActThreads; i++) {
+      const uint32_t idx = i * kActThreads + tid;
+      const uint32_t m = m0 + idx / (kActN / 8), c = c0 + (idx % (kActN / 8)) * 8;
+      if (m < p.M && c < p.d) {
+        const uint4v g = *reinterpret_cast<const uint4v*>(p.G + (size_t)m * p.ldg + c);
+        const uint4v u = *reinterpret_cast<const uint4v*>(p.G + (size_t)m * p.ldg + p.d + c);
+        *reinterpret_cast<uint4v*>(p.A + (size_t)m * p.lda + c) = cusync::gemm::swigluChunk(g, u);
+      }
+    }
+    cusync_dim3 done = {m0, c0, 0};
+    if (stage.isProducer()) stage.post(done);
+    else __syncthreads();
+  }
+}
+
+int g_actResident = 0;
+
+cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
+  if (g_actResident == 0) {
+    int dev = 0, perCU = 0;
+    hipDeviceProp_t prop;
+    if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev)) ||
+        CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, swigluStageKernel, (int)kActThreads, 0))) return CUSYNC_ERROR_DEVICE;
+    g_actResident = std::max(1, std::min(perCU, 4)) * prop.multiProcessorCount;
+  }
+  const cusync_stage_desc& s = m->mid;
+  ActParams p = {};
+  p.stage.d = s;
+  p.stage.lineAligned = false;       // every wait is followed by an L2 invalidation: tiles of 128 columns of a 2d-wide matrix are not whole lines for every d
+  p.M = m->cfg.batch; p.d = m->cfg.inner;
+  p.G = (const half_t*)h; p.ldg = m->ldh;
+  p.A = (half_t*)m->act; p.lda = m->cfg.inner;
+  p.launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)g_actResident);
+  hipLaunchKernelGGL(swigluStageKernel, dim3(p.launched), dim3(kActThreads), 0, (hipStream_t)stream, p);
+  if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  return CUSYNC_SUCCESS;
+}
 
 // Built-in choice of tile shapes per batch size for 256 CUs.  Above 128 rows the
 // direct-to-LDS tiles are used; below that the M extent follows the batch.  A SwiGLU consumer has
@@ -103,7 +200,7 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
   } else {
     a.stage = m->cons;
     a.N = m->n2; a.K = m->k2;
-    a.A = h; a.lda = m->ldh;
+    a.A = m->actStage ? m->act : h; a.lda = m->actStage ? m->k2 : m->ldh;
     a.B = m->w2; a.ldb = m->n2;
     a.D = y; a.ldd = m->n2;
     a.epilogue = CUSYNC_EPILOGUE_NONE;
@@ -130,10 +227,16 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->n2 = cfg->hidden;
   m->ldh = m->n1;
   m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : CUSYNC_EPILOGUE_NONE;
-  m->aMode2 = (llama && cfg->activation) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  const bool swiglu = llama && cfg->activation;
+  // up to 128 rows the third launch costs more than the repeated arithmetic (64 rows: 87 against 82 us)
+  m->actStage = swiglu && (cfg->swiglu_in_gemm2 < 0 || (cfg->swiglu_in_gemm2 == 0 && cfg->batch > 128));
+  m->aMode2 = (swiglu && !m->actStage) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  m->act = nullptr;
+  m->sMid = nullptr;
+  memset(&m->mid, 0, sizeof m->mid);
 
   int sync = cfg->sync;
-  if (llama && sync == CUSYNC_SYNC_TILE && m->aMode2 == CUSYNC_A_SWIGLU && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
+  if (swiglu && sync == CUSYNC_SYNC_TILE && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
   pickTiles(*cfg, sync, m->aMode2 == CUSYNC_A_SWIGLU, &m->tile1, &m->tile2);
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
@@ -184,11 +287,21 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     uint32_t bk = 0;
     cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk);
     const bool direct = bk == 32 || m->tile1 >= CUSYNC_TILE_D32x128x64;      // the direct-to-LDS tiles
-    if (m->tile1 != m->tile2 || !direct || m->aMode2 != CUSYNC_A_PLAIN) {
+    if (m->tile1 != m->tile2 || !direct || m->aMode2 != CUSYNC_A_PLAIN || m->actStage) {
       setError("mlp: one launch for both GEMMs needs the same direct-to-LDS tile for both and a plain A operand");
       delete m;
       return nullptr;
     }
+  }
+
+  // the edge into GEMM2 when the activation is a stage of its own: its 128 x 128 tiles under the same kind of policy
+  cusync_policy_desc pol2 = pol;
+  const cusync_dim3 gAct = {(cfg->inner + kActN - 1) / kActN, (cfg->batch + kActM - 1) / kActM, 1};
+  if (m->actStage && sync != CUSYNC_SYNC_STREAM) {
+    pol2 = noSync();
+    pol2.order = CUSYNC_ORDER_TRANSPOSE_XY; pol2.postValue = 1;
+    if (sync == CUSYNC_SYNC_ROW) { pol2.kind = CUSYNC_POLICY_ROWSYNC; pol2.tileM = kActM; pol2.tileN = 1; pol2.waitValue = gAct.x; }
+    else { pol2.kind = CUSYNC_POLICY_TILESYNC; pol2.tileM = kActM; pol2.tileN = kActN; pol2.waitValue = 1; }
   }
 
   memset(&m->prod, 0, sizeof m->prod);
@@ -196,17 +309,31 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->prod.grid = g1; m->prod.tileSize = {1, 1, 1}; m->prod.iter = 1; m->prod.opts = opts;
   m->prod.in = noSync(); m->prod.out = pol;
   m->cons.grid = g2; m->cons.tileSize = {1, 1, 1}; m->cons.iter = 1; m->cons.opts = opts;
-  m->cons.in = pol; m->cons.out = noSync();
+  m->cons.in = m->actStage ? pol2 : pol; m->cons.out = noSync();
   if (cusync_stage_create(&m->prod, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS ||
       cusync_stage_create(&m->cons, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) {
     delete m;
     return nullptr;
   }
-  if (sync != CUSYNC_SYNC_STREAM &&
-      cusync_set_producer_consumer_pair(&m->prod, &m->cons) != CUSYNC_SUCCESS) {
-    setError("mlp: pairing the stages failed");
-    delete m;
-    return nullptr;
+  if (m->actStage) {
+    m->mid.grid = gAct; m->mid.tileSize = {1, 1, 1}; m->mid.iter = 1; m->mid.opts = opts;
+    m->mid.in = pol; m->mid.out = pol2;
+    if (cusync_stage_create(&m->mid, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS ||
+        CUSYNC_HIP(hipMalloc(&m->act, (size_t)cfg->batch * cfg->inner * sizeof(half_t))) ||
+        CUSYNC_HIP(hipStreamCreateWithFlags(&m->sMid, hipStreamNonBlocking))) {
+      delete m;
+      return nullptr;
+    }
+  }
+  if (sync != CUSYNC_SYNC_STREAM) {
+    const bool ok = m->actStage ? cusync_set_producer_consumer_pair(&m->prod, &m->mid) == CUSYNC_SUCCESS &&
+                                  cusync_set_producer_consumer_pair(&m->mid, &m->cons) == CUSYNC_SUCCESS
+                                : cusync_set_producer_consumer_pair(&m->prod, &m->cons) == CUSYNC_SUCCESS;
+    if (!ok) {
+      setError("mlp: pairing the stages failed");
+      delete m;
+      return nullptr;
+    }
   }
   for (int which = 0; which < 2; which++) {
     cusync_gemm_args a = gemmArgs(m, which, nullptr, nullptr, nullptr);
@@ -232,6 +359,11 @@ void cusync_mlp_destroy(cusync_mlp* m) {
   (void)hipStreamSynchronize(m->sCons);
   cusync_stage_free(&m->prod);
   cusync_stage_free(&m->cons);
+  if (m->actStage) {
+    if (m->sMid) { (void)hipStreamSynchronize(m->sMid); (void)hipStreamDestroy(m->sMid); }
+    cusync_stage_free(&m->mid);
+    if (m->act) (void)hipFree(m->act);
+  }
   if (m->ws1) (void)hipFree(m->ws1);
   if (m->ws2) (void)hipFree(m->ws2);
   (void)hipEventDestroy(m->eStart); (void)hipEventDestroy(m->eMid); (void)hipEventDestroy(m->eEnd);
@@ -256,11 +388,18 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     } else if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) {
       return e;
     } else if (overlapped) {
-      if ((e = cusync_invoke_wait_kernel(&m->prod, m->sCons)) != CUSYNC_SUCCESS) return e;
+      if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a wait kernel per edge
+        if ((e = cusync_invoke_wait_kernel(&m->prod, m->sMid)) != CUSYNC_SUCCESS) return e;
+        if ((e = runActStage(m, h, m->sMid)) != CUSYNC_SUCCESS) return e;
+        if ((e = cusync_invoke_wait_kernel(&m->mid, m->sCons)) != CUSYNC_SUCCESS) return e;
+      } else if ((e = cusync_invoke_wait_kernel(&m->prod, m->sCons)) != CUSYNC_SUCCESS) {
+        return e;
+      }
       if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;
       if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sCons))) return CUSYNC_ERROR_DEVICE;
     } else {
       if (CUSYNC_HIP(hipEventRecord(m->eMid, m->sProd))) return CUSYNC_ERROR_DEVICE;
+      if (m->actStage && (e = runActStage(m, h, m->sProd)) != CUSYNC_SUCCESS) return e;     // counted with GEMM2
       if ((e = cusync_gemm_run(&a2, m->sProd)) != CUSYNC_SUCCESS) return e;
       if (CUSYNC_HIP(hipEventRecord(m->eEnd, m->sProd))) return CUSYNC_ERROR_DEVICE;
     }
@@ -268,6 +407,7 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     // The consumer finishing implies every producer tile was posted, but the
     // producer kernel itself must have retired before its stage is reused.
     if (overlapped && CUSYNC_HIP(hipStreamSynchronize(m->sProd))) return CUSYNC_ERROR_DEVICE;
+    if (overlapped && m->actStage && CUSYNC_HIP(hipStreamSynchronize(m->sMid))) return CUSYNC_ERROR_DEVICE;
     float ms = 0;
     if (times_us) {
       if (CUSYNC_HIP(hipEventElapsedTime(&ms, m->eStart, m->eEnd))) return CUSYNC_ERROR_DEVICE;
@@ -283,6 +423,7 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     }
     m->prod.iter += 1;     // incrementIter on both stages, mlp.cu:709-712
     m->cons.iter += 1;
+    m->mid.iter += 1;
   }
   return CUSYNC_SUCCESS;
 }
@@ -293,6 +434,7 @@ cusync_error cusync_mlp_run(cusync_mlp* m, const void* x, void* h, void* y, int 
 
 const cusync_stage_desc* cusync_mlp_stage(const cusync_mlp* m, int which) {
   if (!m) return nullptr;
+  if (which == 2) return m->actStage ? &m->mid : nullptr;
   return which == 0 ? &m->prod : &m->cons;
 }
 

@@ -403,6 +403,11 @@ typedef struct cusync_mlp_config {
   int32_t max_wg1, max_wg2;    /* workgroups per launch of each GEMM; 0 = built-in choice, -1 = as many as stay resident */
   int32_t one_launch;          /* 1 (with a CuSync mode): both GEMMs in one launch, cusync_gemm_chain_run; needs the same
                                   direct-to-LDS tile for both and a plain A operand in GEMM2 */
+  int32_t swiglu_in_gemm2;     /* LLaMA with activation: where silu(gate)*up is computed.  -1: in a stage of its own between
+                                  the GEMMs (a third kernel and stream, every element once; GEMM2 then runs the
+                                  direct-to-LDS tiles).  1: in GEMM2's A loader as the data passes (one kernel fewer,
+                                  but repeated for every column tile of GEMM2: 357 against 128 us at 2048 rows).
+                                  0: built-in choice, the stage of its own above 128 rows */
 } cusync_mlp_config;
 
 typedef struct cusync_mlp cusync_mlp;   /* opaque */
@@ -422,7 +427,7 @@ cusync_error cusync_mlp_run(cusync_mlp *mlp, const void *x, void *h, void *y, in
 cusync_error cusync_mlp_run_split(cusync_mlp *mlp, const void *x, void *h, void *y, int runs,
                                   double *times_us, double *gemm1_us, double *gemm2_us);
 /* Device state of the two stages for tests (see cusync_stage_read_state). */
-const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer, 1 consumer */);
+const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer (GEMM1), 1 consumer (GEMM2), 2 the activation stage or NULL */);
 int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
 int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 

@@ -106,16 +106,18 @@ def test_gpt3_without_activation_matches_reference_check_build():
     check_against_oracle(api.MODEL.GPT3, x, w1, w2, h, y, inner=6144, activation=0)
 
 
+@pytest.mark.parametrize("in_gemm2", [-1, 1])
 @pytest.mark.parametrize("inner", [2752, 2816])
 @pytest.mark.parametrize("batch", [1, 64, 256, 1024])
-def test_llama_mlp(inner, batch):
-    print("llama", inner, batch, flush=True)
+def test_llama_mlp(inner, batch, in_gemm2):
+    # silu(gate) * up either as a stage of its own between the GEMMs or in GEMM2's A loader
+    print("llama", inner, batch, in_gemm2, flush=True)
     outs = {}
     # StridedSync constrains the tile width (gate|up split on a tile boundary); the other modes are run with
     # the same tiles and k-slices so that all three execute the same kernels and must agree bit for bit
     same = {}
     for sync in (api.SYNC.STRIDED, api.SYNC.STREAM, api.SYNC.ROW):
-        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2, **same)
+        x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2, swiglu_in_gemm2=in_gemm2, **same)
         same = dict(tile1=tiles[0], tile2=tiles[1], split_k1=tiles[2], split_k2=tiles[3])
         outs[sync] = (h, y)
         assert cons.spin_timeouts == 0
