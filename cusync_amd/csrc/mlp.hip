@@ -149,10 +149,13 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
   // k-slices fill the device).  GEMM2: the same from 513 rows on; up to 512 rows, where it has at most one 128-row
   // tile per CU, 128x192 with four stages in the pipelined order (384 rows: 258 -> 225 us, 512 rows: 254 -> 235 us
   // for the pair against 128x192 at two workgroups per CU for both).
-  // Other widths: 128x128 up to 1024 rows (more tiles to spread), 128x256 above.
+  // Other widths (the LLaMA shard: 5504 and 8192 columns; the kernels mask the ragged last column tile): 128x192
+  // alone on its CU up to 1024 rows, above that 256x192 for GEMM1 and 256x256 for GEMM2 (at 2048 rows 232 and 256
+  // tiles: one round).  Measured against 128x128 / 128x256 at two workgroups per CU: 172 -> 147 us at 512 rows,
+  // 232 -> 211 at 1024, 356 -> 304 at 2048.
   const uint32_t n1 = c.model == CUSYNC_MLP_LLAMA ? 2 * c.inner : c.inner, n2 = c.hidden;
-  int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 512 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
+  int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
+  int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x256x32;
   if (big && n1 % 192 == 0) a = CUSYNC_TILE_256x192x32;
   if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 512 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32_ALONE;
   // Up to 256 rows the GEMMs are bound by streaming the weights: direct-to-LDS tiles with 60-96 KB of loads
@@ -165,8 +168,14 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* 
     if (n1 % 192 == 0) a = CUSYNC_TILE_D64x192x64;
     if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_D64x192x64;
   }
-  if (sync == CUSYNC_SYNC_STRIDED && c.inner % 128 != 0)
-    a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
+  // StridedSync needs the gate|up split on a column-tile boundary of GEMM1: 128- or 256-wide tiles where the
+  // 192-wide ones do not divide `inner`, 64-wide ones where nothing else does (2752 = 43 * 64)
+  if (sync == CUSYNC_SYNC_STRIDED) {
+    uint32_t tn = 0;
+    cusync_gemm_tile_shape(c.tile1 >= 0 ? c.tile1 : a, nullptr, &tn, nullptr);
+    if (c.inner % 128 != 0) a = c.batch <= 128 ? CUSYNC_TILE_128x64x64 : CUSYNC_TILE_256x64x64;
+    else if (tn == 0 || c.inner % tn != 0) a = c.batch <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
+  }
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
   *t2 = c.tile2 >= 0 ? c.tile2 : b;
   // both GEMMs in one launch share a kernel: the consumer takes the producer's tile
