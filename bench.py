@@ -80,7 +80,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=50,
+                    help="untimed steps before the timed ones; after a light load the device needs about 30 steps of\n"
+                         "this size before its clock settles")
     ap.add_argument("--batch", type=int, default=2048, help="B of the timed step")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-batch table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -151,7 +153,7 @@ def main():
                 "kernel": "gemmDmaKernel, mean of the two launches of the step: GEMM1 tile %s %.1f us, GEMM2 tile %s %.1f us "
                           "(stream-ordered, %.1f GFLOP per launch)" % (shapes[0], statistics.fmean(g1), shapes[1], statistics.fmean(g2),
                                                                        flops_per_launch / 1e9),
-                }, trimmed(t_s)[0], tiles
+                }, statistics.fmean(t_s), tiles
 
     if args.profile_chain == "attention":
         heads, e, seq = 12, 12 * 128, 2048
@@ -347,8 +349,11 @@ def main():
         "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "GPT-3 175B MLP 1/8 shard, B=%d: X[B,12288] x W1[12288,6144] +GeLU -> x W2[6144,12288]" % B,
                    "policy": policy, "tiles": list(tiles), "device": dev["arch"], "cus": dev["cus"]},
+        # the same two GEMMs stream-ordered, same warm-up and step count, plain mean like `value`
         "stream_ordered_us": round(stream_us, 2),
         "gain_pct": round(100 - statistics.fmean(step_times) / stream_us * 100, 2),
+        "step_us": {"median": round(statistics.median(step_times), 2), "min": round(min(step_times), 2),
+                    "max": round(max(step_times), 2)},
         "tflops": round(mlp_flops(B) / statistics.fmean(step_times) / 1e6, 1),
         "roofline": roof,
         "per_batch": per_batch,

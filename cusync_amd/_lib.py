@@ -97,6 +97,7 @@ SIGNATURES = {
     "cusync_stage_create": (C.c_int, [C.POINTER(StageDesc), C.c_int]),
     "cusync_set_producer_consumer_pair": (C.c_int, [C.POINTER(StageDesc), C.POINTER(StageDesc)]),
     "cusync_invoke_wait_kernel": (C.c_int, [C.POINTER(StageDesc), vp]),
+    "cusync_invoke_wait_kernel_after": (C.c_int, [C.POINTER(StageDesc), vp, vp]),
     "cusync_wait_kernel": (C.c_int, [vp, u32, vp]),
     "cusync_stage_read_state": (C.c_int, [C.POINTER(StageDesc), vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_policy_tile_index": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),

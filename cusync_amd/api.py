@@ -137,7 +137,11 @@ class Stage:
         g = self.desc.grid
         return g.x * g.y * g.z
 
-    def invokeWaitKernel(self, stream):
+    def invokeWaitKernel(self, stream, after=None):
+        """`after`: an event recorded on the producer's stream right before the
+        producer's launch; the wait kernel is then dispatched behind it."""
+        if after is not None:
+            return self.L.cusync_invoke_wait_kernel_after(C.byref(self.desc), stream, after)
         return self.L.cusync_invoke_wait_kernel(C.byref(self.desc), stream)
 
     def incrementIter(self):

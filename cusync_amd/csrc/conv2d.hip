@@ -382,7 +382,10 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
       hipStream_t s = c->stream[overlapped ? i : 0];
       const cusync_conv2d_args a = layerArgs(i);
       cusync_error e;
-      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
+      // overlapped: ev[i] marks the launch of layer i on its stream, and the wait kernel for layer i - 1 goes
+      // behind ev[i - 1] (ahead of that launch its wave would hold a CU one of the producer's workgroups needs)
+      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel_after(&c->st[i - 1], s, c->ev[i - 1])) != CUSYNC_SUCCESS) return e;
+      if (overlapped && i > 0 && i + 1 < n && CUSYNC_HIP(hipEventRecord(c->ev[i], s))) return CUSYNC_ERROR_DEVICE;
       if ((e = cusync_conv2d_run(&a, s)) != CUSYNC_SUCCESS) return e;
       if ((!overlapped || i + 1 == n) && CUSYNC_HIP(hipEventRecord(c->ev[i + 1], s))) return CUSYNC_ERROR_DEVICE;
     }

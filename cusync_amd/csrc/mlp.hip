@@ -397,11 +397,14 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     } else if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) {
       return e;
     } else if (overlapped) {
+      // each wait kernel goes behind the event recorded right before its producer's launch: ahead of it, its wave
+      // would hold a CU that one of the producer's workgroups needs (see cusync_invoke_wait_kernel_after)
       if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a wait kernel per edge
-        if ((e = cusync_invoke_wait_kernel(&m->prod, m->sMid)) != CUSYNC_SUCCESS) return e;
+        if ((e = cusync_invoke_wait_kernel_after(&m->prod, m->sMid, m->eStart)) != CUSYNC_SUCCESS) return e;
+        if (CUSYNC_HIP(hipEventRecord(m->eMid, m->sMid))) return CUSYNC_ERROR_DEVICE;
         if ((e = runActStage(m, h, m->sMid)) != CUSYNC_SUCCESS) return e;
-        if ((e = cusync_invoke_wait_kernel(&m->mid, m->sCons)) != CUSYNC_SUCCESS) return e;
-      } else if ((e = cusync_invoke_wait_kernel(&m->prod, m->sCons)) != CUSYNC_SUCCESS) {
+        if ((e = cusync_invoke_wait_kernel_after(&m->mid, m->sCons, m->eMid)) != CUSYNC_SUCCESS) return e;
+      } else if ((e = cusync_invoke_wait_kernel_after(&m->prod, m->sCons, m->eStart)) != CUSYNC_SUCCESS) {
         return e;
       }
       if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;

@@ -181,6 +181,14 @@ cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc* prod, void* stre
   return cusync_wait_kernel(prod->kernelExecuted, (uint32_t)prod->iter, stream);
 }
 
+cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void* stream, void* launch_event) {
+  if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
+  if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
+  if (launch_event && RT(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)launch_event, 0))) return CUSYNC_ERROR_DEVICE;
+  return cusync_wait_kernel(prod->kernelExecuted, (uint32_t)prod->iter, stream);
+}
+
 cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems, cusync_dim3* tile_order,
                                      uint32_t* tile_counter, uint32_t* start_counter,
                                      uint32_t* kernel_executed, uint32_t* spin_timeouts) {

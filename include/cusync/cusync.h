@@ -155,10 +155,18 @@ public:
 
   // Holds `stream` back until the producer kernel of the current run is on the
   // device (src/include/cusync/cusync.h:203-209).
-  CuSyncError invokeWaitKernel(void* stream) {
+  // `launchEvent` (optional, not in the reference): a hipEvent_t recorded on the
+  // producer's stream right before the producer's launch.  `stream` then waits
+  // for it first, so that the wait kernel's wave cannot reach the device ahead of
+  // the producer's workgroups and hold a CU one of them needs.
+  CuSyncError invokeWaitKernel(void* stream, void* launchEvent = nullptr) {
     if (!isProducer()) return CuSyncErrorNotProducer;
     if (getAvoidWaitKernel()) return CuSyncSuccess;
     if (kernelExecuted_ == nullptr) return CuSyncErrorNotInitialized;
+    if (launchEvent != nullptr) {
+      const cusync_stage_desc d = desc();
+      return (CuSyncError)cusync_invoke_wait_kernel_after(&d, stream, launchEvent);
+    }
     return (CuSyncError)cusync_wait_kernel(kernelExecuted_, (uint32_t)iter, stream);
   }
 

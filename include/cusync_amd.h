@@ -150,6 +150,18 @@ cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc *prod, cu
  * enqueues a one-wave kernel on `stream` that returns once the producer's flag
  * has reached desc->iter.  No-op with AVOID_WAIT_KERNEL. */
 cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc *prod, void *stream);
+/* Same, but `stream` first waits for `launch_event` (a hipEvent_t the caller
+ * recorded on the producer's stream immediately before launching the producer's
+ * kernel; NULL = no ordering).  The two streams are separate hardware queues and
+ * the wait kernel's wave can reach the GPU before the producer's workgroups do.
+ * It then holds registers on one CU until every producer workgroup has started;
+ * a producer whose workgroups need whole CUs and fill the machine cannot place
+ * its last workgroup there, the flag is not raised until another workgroup
+ * retires, and that run of the chain is one producer tile longer.  Behind the
+ * event the wait kernel is dispatched after the producer's launch has begun.
+ * No counterpart in the reference, which launches the wait kernel unordered
+ * (src/ml-bench/transformer/mlp.cu:683-699). */
+cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc *prod, void *stream, void *launch_event);
 /* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
 cusync_error cusync_wait_kernel(uint32_t *semaphore, uint32_t value, void *stream);
 /* Reads back device state for tests (the reference reaches it through the

@@ -149,8 +149,9 @@ def test_gemm_can_implement_rejects():
     prod.destroy()
 
 
-def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1)):
-    """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`."""
+def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1), ordered=False):
+    """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`.  `ordered`: the wait kernel
+    goes behind an event recorded on the producer's stream right before the producer's launch."""
     import torch
     L = _lib.load()
     a = uniform_f16((M, K), seed)
@@ -177,19 +178,23 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
     a2 = api.gemm_args(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2, split_k=split[1], max_workgroups=max_wg)
     ws = [torch.zeros(max(16, L.cusync_gemm_workspace_size(C.byref(x))), dtype=torch.uint8, device="cuda") for x in (a1, a2)]
     torch.cuda.synchronize()
+    ev = C.c_void_p()
+    assert L.cusync_rt_event_create(C.byref(ev)) == 0
     for _ in range(iters):
         dc.fill_(float("nan")); de.fill_(float("nan"))
         torch.cuda.synchronize()
+        if ordered:
+            assert L.cusync_rt_event_record(ev, s1) == 0
         assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1, stream=s1,
                         max_workgroups=max_wg, split_k=split[0], workspace=ws[0].data_ptr()) == api.ERR.SUCCESS, api.last_error()
-        assert prod.invokeWaitKernel(s2) == api.ERR.SUCCESS
+        assert prod.invokeWaitKernel(s2, after=ev if ordered else None) == api.ERR.SUCCESS
         assert api.gemm(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2, stream=s2,
                         max_workgroups=max_wg, split_k=split[1], workspace=ws[1].data_ptr()) == api.ERR.SUCCESS, api.last_error()
         assert L.cusync_rt_device_sync() == 0, api.last_error()
         prod.incrementIter(); cons.incrementIter()
     ps, cs = prod.read_state(), cons.read_state()
     want_sems = orc.expected_sems_gemm(opol, g1, tm, tn, iters, opts)
-    L.cusync_rt_stream_destroy(s1); L.cusync_rt_stream_destroy(s2)
+    L.cusync_rt_stream_destroy(s1); L.cusync_rt_stream_destroy(s2); L.cusync_rt_event_destroy(ev)
     prod.destroy(); cons.destroy()
     return a, b, d, to_host(dc), to_host(de), ps, cs, want_sems
 
@@ -223,6 +228,21 @@ def test_chained_gemms_with_few_workgroups():
     assert_close(c, orc.gemm(a, b), "C")
     assert_close(e, orc.gemm(c, d), "E")
     assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3
+
+
+@pytest.mark.parametrize("policy_kind", ["tile", "row"])
+def test_chained_gemms_wait_kernel_behind_launch_event(policy_kind):
+    # cusync_invoke_wait_kernel_after: same results and semaphore end state as the unordered wait kernel
+    print("chained, ordered wait kernel", policy_kind, flush=True)
+    M, N, K = 512, 1536, 1024
+    tile = api.TILE.T256x192x32
+    a, b, d, c, e, ps, cs, want_sems = chained(M, N, K, tile, tile, policy_kind, iters=3, ordered=True)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0
+    assert np.array_equal(ps.sems, want_sems)
+    assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
+    assert ps.kernel_executed == 3
 
 
 @pytest.mark.parametrize("policy_kind,opts", [("tile", api.OPT.NO_ATOMIC_ADD), ("row", 0)])
