@@ -115,16 +115,16 @@ def main():
     w1, w2, x_all = (torch.from_numpy(a).cuda() for a in (w1_host, w2_host, x_host))
     torch.cuda.synchronize()
 
-    def make(batch, sync, one_launch=False):
+    def make(batch, sync, one_launch=False, repack=False):
         h = torch.empty((batch, INNER), dtype=torch.float16, device="cuda")
         y = torch.empty((batch, HIDDEN), dtype=torch.float16, device="cuda")
         torch.cuda.synchronize()
         m = api.Mlp(api.MODEL.GPT3, batch, HIDDEN, INNER, sync, w1.data_ptr(), w2.data_ptr(),
-                    tile1=args.tile1, tile2=args.tile2, one_launch=one_launch)
+                    tile1=args.tile1, tile2=args.tile2, one_launch=one_launch, repack_weights=repack)
         return m, h, y
 
-    def protocol(batch, sync, warm=10, timed=20, split=False, one_launch=False):
-        m, h, y = make(batch, sync, one_launch)
+    def protocol(batch, sync, warm=10, timed=20, split=False, one_launch=False, repack=False):
+        m, h, y = make(batch, sync, one_launch, repack)
         x = x_all[:batch]
         m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=warm)
         out = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=timed, split=split)
@@ -205,6 +205,10 @@ def main():
             t_t, _ = protocol(b, api.SYNC.TILE)
             # RowSync with both GEMMs in one launch (same stages and semaphores, no wait kernel, no second launch)
             one = trimmed(protocol(b, api.SYNC.ROW, one_launch=True)[0])[0] if tiles[0] == tiles[1] else None
+            # the same chain reading copies of the weights whose rows are 256 bytes longer (cusync_mlp_config.
+            # repack_weights): a column tile's k rows then spread over all memory channels instead of one class
+            s_rp = trimmed(protocol(b, api.SYNC.STREAM, repack=True)[0])[0]
+            r_rp = trimmed(protocol(b, api.SYNC.ROW, repack=True)[0])[0]
             s, s_sd = trimmed(t_s)
             r, r_sd = trimmed(t_r)
             t, t_sd = trimmed(t_t)
@@ -216,6 +220,8 @@ def main():
                 "rowsync_us": round(r, 2), "rowsync_std": round(r_sd, 2), "rowsync_gain_pct": round(100 - r / s * 100, 2),
                 "tilesync_us": round(t, 2), "tilesync_std": round(t_sd, 2), "tilesync_gain_pct": round(100 - t / s * 100, 2),
                 "rowsync_one_launch_us": None if one is None else round(one, 2),
+                "repacked_weights": {"stream_us": round(s_rp, 2), "rowsync_us": round(r_rp, 2),
+                                     "roofline_frac": round(ideal_us(b) / min(s_rp, r_rp), 4)},
                 "best_tflops": round(mlp_flops(b) / best / 1e6, 1),
                 "bound": "mfma" if mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12) > mlp_bytes(b) / (PEAK_HBM_GBS * 1e9) else "hbm",
                 "roofline_frac": round(ideal_us(b) / best, 4),
@@ -270,6 +276,11 @@ def main():
                     sys.exit("bench.py: LLaMA consumer waits timed out — results invalid")
                 row[name + "_us"] = round(trimmed(t)[0], 2)
                 row[name + "_tiles"] = list(m.tiles())
+                m.destroy()
+            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW)):      # W2's rows are 16 KiB
+                m = api.Mlp(api.MODEL.LLAMA, b, lh, li, sync, lw1.data_ptr(), lw2.data_ptr(), repack_weights=True)
+                m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
+                row[name + "_repacked_us"] = round(trimmed(m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20))[0], 2)
                 m.destroy()
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "stridedsync_us"))
             row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)

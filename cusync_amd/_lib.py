@@ -68,7 +68,7 @@ class AttnLayerConfig(C.Structure):
 class MlpConfig(C.Structure):
     _fields_ = [("model", i32), ("batch", u32), ("hidden", u32), ("inner", u32), ("sync", i32),
                 ("tile1", i32), ("tile2", i32), ("opts", i32), ("activation", i32),
-                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32), ("one_launch", i32), ("swiglu_in_gemm2", i32)]
+                ("split_k1", i32), ("split_k2", i32), ("max_wg1", i32), ("max_wg2", i32), ("one_launch", i32), ("swiglu_in_gemm2", i32), ("repack_weights", i32)]
 
 
 # every symbol include/cusync_amd.h declares: name -> (restype, argtypes)
@@ -140,6 +140,7 @@ SIGNATURES = {
     "cusync_probe_mfma_rate": (C.c_int, [C.c_int, u32, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_mlp_create": (vp, [C.POINTER(MlpConfig), vp, vp]),
     "cusync_mlp_destroy": (None, [vp]),
+    "cusync_mlp_reload_weights": (C.c_int, [vp]),
     "cusync_mlp_run": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double)]),
     "cusync_mlp_run_split": (C.c_int, [vp, vp, vp, vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_mlp_stage": (C.POINTER(StageDesc), [vp, C.c_int]),

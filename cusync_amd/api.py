@@ -377,13 +377,17 @@ class Mlp:
     """Handle over cusync_mlp_* (the reference's libmlp C surface, src/ml-bench/transformer/mlp-lib.cu:555-618)."""
 
     def __init__(self, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=-1, tile2=-1, opts=-1, activation=1,
-                 split_k1=0, split_k2=0, max_wg1=0, max_wg2=0, one_launch=False, swiglu_in_gemm2=0):
+                 split_k1=0, split_k2=0, max_wg1=0, max_wg2=0, one_launch=False, swiglu_in_gemm2=0, repack_weights=False):
         self.L = _lib.load()
         self.cfg = MlpConfig(model, batch, hidden, inner, sync, tile1, tile2, opts, activation, split_k1, split_k2,
-                             max_wg1, max_wg2, int(one_launch), int(swiglu_in_gemm2))
+                             max_wg1, max_wg2, int(one_launch), int(swiglu_in_gemm2), int(repack_weights))
         self.h = self.L.cusync_mlp_create(C.byref(self.cfg), w1_ptr, w2_ptr)
         if not self.h:
             raise RuntimeError("cusync_mlp_create failed: " + last_error())
+
+    def reload_weights(self):
+        """With repack_weights: copies the caller's weights into the handle's padded buffers again."""
+        return self.L.cusync_mlp_reload_weights(self.h)
 
     @classmethod
     def from_db(cls, entry, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, activation=1):

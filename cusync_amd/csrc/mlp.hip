@@ -26,6 +26,8 @@ struct cusync_mlp {
   void* ws2;
   uint32_t n1, k1, n2, k2;          // GEMM1 is [batch,k1]x[k1,n1], GEMM2 is [batch,k2]x[k2,n2]
   uint32_t ldh;                      // row pitch of the intermediate
+  void* w1p; void* w2p;              // repack_weights: padded copies of the weights, owned
+  uint32_t ldw1, ldw2;               // row pitch of the weights the GEMMs read
   int epilogue1, aMode2;
   cusync_stage_desc prod, cons;
   hipStream_t sProd, sCons;
@@ -35,6 +37,10 @@ struct cusync_mlp {
   void* act;                         // [batch][inner] fp16, GEMM2's A operand
   cusync_stage_desc mid;
   hipStream_t sMid;
+  ~cusync_mlp() {
+    if (w1p) (void)hipFree(w1p);
+    if (w2p) (void)hipFree(w2p);
+  }
 };
 
 namespace {
@@ -51,6 +57,12 @@ using cusync::gemm::uint4v;
 // same arithmetic is repeated once per column tile of GEMM2 (64 times for the LLaMA shard) and makes
 // that kernel three times slower; here every element is computed once.
 constexpr uint32_t kActM = 128, kActN = 128, kActThreads = 256;
+
+// dst[row][0..vecs) = src[row][0..vecs) in 16-byte pieces; dst rows are dstPitch pieces apart
+__global__ __launch_bounds__(256) void repackRowsKernel(const uint4v* src, uint4v* dst, uint32_t vecs, uint32_t dstPitch) {
+  const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+  if (c < vecs) dst[(size_t)blockIdx.y * dstPitch + c] = src[(size_t)blockIdx.y * vecs + c];
+}
 
 struct ActParams {
   cusync::DynStage stage;
@@ -201,7 +213,7 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
     a.stage = m->prod;
     a.N = m->n1; a.K = m->k1;
     a.A = x; a.lda = m->k1;
-    a.B = m->w1; a.ldb = m->n1;
+    a.B = m->w1p ? m->w1p : m->w1; a.ldb = m->ldw1;
     a.D = h; a.ldd = m->ldh;
     a.epilogue = m->epilogue1;
     a.a_mode = CUSYNC_A_PLAIN;
@@ -210,7 +222,7 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
     a.stage = m->cons;
     a.N = m->n2; a.K = m->k2;
     a.A = m->actStage ? m->act : h; a.lda = m->actStage ? m->k2 : m->ldh;
-    a.B = m->w2; a.ldb = m->n2;
+    a.B = m->w2p ? m->w2p : m->w2; a.ldb = m->ldw2;
     a.D = y; a.ldd = m->n2;
     a.epilogue = CUSYNC_EPILOGUE_NONE;
     a.a_mode = m->aMode2;
@@ -235,6 +247,19 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->k2 = cfg->inner;
   m->n2 = cfg->hidden;
   m->ldh = m->n1;
+  m->w1p = m->w2p = nullptr;
+  m->ldw1 = m->n1; m->ldw2 = m->n2;
+  if (cfg->repack_weights) {
+    // rows 256 bytes longer than the data: consecutive k rows of a column tile then fall into consecutive
+    // channel classes (address bits 8..11) instead of all into one
+    m->ldw1 = m->n1 + 128; m->ldw2 = m->n2 + 128;
+    if (CUSYNC_HIP(hipMalloc(&m->w1p, (size_t)m->k1 * m->ldw1 * sizeof(half_t))) ||
+        CUSYNC_HIP(hipMalloc(&m->w2p, (size_t)m->k2 * m->ldw2 * sizeof(half_t))) ||
+        cusync_mlp_reload_weights(m) != CUSYNC_SUCCESS) {
+      delete m;
+      return nullptr;
+    }
+  }
   m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : CUSYNC_EPILOGUE_NONE;
   const bool swiglu = llama && cfg->activation;
   // up to 128 rows the third launch costs more than the repeated arithmetic (64 rows: 87 against 82 us)
@@ -360,6 +385,26 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     return nullptr;
   }
   return m;
+}
+
+cusync_error cusync_mlp_reload_weights(cusync_mlp* m) {
+  if (!m) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (!m->w1p) return CUSYNC_SUCCESS;
+  // a kernel, not a copy-engine transfer: the GEMMs of the last run may have left lines of the padded buffers
+  // in the L2s, and only a kernel boundary on the device is sure to drop them
+  hipStream_t s = nullptr;
+  if (CUSYNC_HIP(hipDeviceSynchronize())) return CUSYNC_ERROR_DEVICE;
+  const struct { const void* src; void* dst; uint32_t rows, cols, pitch; } job[2] = {
+      {m->w1, m->w1p, m->k1, m->n1, m->ldw1}, {m->w2, m->w2p, m->k2, m->n2, m->ldw2}};
+  for (const auto& j : job) {
+    if (j.cols % 8 != 0) { setError("mlp: repack_weights needs rows of whole 16-byte pieces"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    const uint32_t vecs = j.cols / 8;
+    const dim3 grid((vecs + 255) / 256, j.rows, 1);
+    hipLaunchKernelGGL(repackRowsKernel, grid, dim3(256), 0, s, (const uint4v*)j.src, (uint4v*)j.dst, vecs, j.pitch / 8);
+    if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  }
+  if (CUSYNC_HIP(hipDeviceSynchronize())) return CUSYNC_ERROR_DEVICE;
+  return CUSYNC_SUCCESS;
 }
 
 void cusync_mlp_destroy(cusync_mlp* m) {

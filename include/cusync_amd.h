@@ -420,6 +420,13 @@ typedef struct cusync_mlp_config {
                                   direct-to-LDS tiles).  1: in GEMM2's A loader as the data passes (one kernel fewer,
                                   but repeated for every column tile of GEMM2: 357 against 128 us at 2048 rows).
                                   0: built-in choice, the stage of its own above 128 rows */
+  int32_t repack_weights;      /* 1: create() copies w1 and w2 into buffers of its own whose row pitch is 256 bytes longer
+                                  than the row, and the GEMMs read those (call cusync_mlp_reload_weights after changing
+                                  the caller's copies).  The shards' rows are multiples of 4 KiB, so a column tile of the
+                                  caller's layout keeps address bits 8..11 fixed over all its k rows and draws on one
+                                  class of memory channels only, one of which delivers a quarter less: at few rows,
+                                  where the GEMMs stream the weights, the slowest tiles decide (24 against 18.5 us).
+                                  0: read the caller's arrays in place (the reference's behaviour). */
 } cusync_mlp_config;
 
 typedef struct cusync_mlp cusync_mlp;   /* opaque */
@@ -428,6 +435,8 @@ typedef struct cusync_mlp cusync_mlp;   /* opaque */
  * w1: [hidden, inner] (GPT-3) or [hidden, 2*inner] gate|up (LLaMA); w2: [inner, hidden]. */
 cusync_mlp *cusync_mlp_create(const cusync_mlp_config *cfg, const void *w1, const void *w2);
 void cusync_mlp_destroy(cusync_mlp *mlp);
+/* With repack_weights: copies the caller's w1 / w2 (the pointers given to create) into the padded buffers again. */
+cusync_error cusync_mlp_reload_weights(cusync_mlp *mlp);
 /* runLLAMA / runCuSyncLLAMA (TB/mlp-lib.cu:569-576, 611-618): `runs` back-to-back
  * passes x -> h -> y.  h is the intermediate [batch, inner] (GPT-3) or
  * [batch, 2*inner] (LLaMA).  If times_us != NULL it receives one elapsed time

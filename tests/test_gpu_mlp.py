@@ -169,3 +169,50 @@ def test_mlp_in_one_launch_rejects():
     with pytest.raises(RuntimeError):       # the register-staged tiles have no chain kernel
         api.Mlp(api.MODEL.GPT3, 256, 12288, 6144, api.SYNC.ROW, dw1.data_ptr(), dw2.data_ptr(),
                 tile1=api.TILE.T128x128x64, tile2=api.TILE.T128x128x64, one_launch=True)
+
+
+@pytest.mark.parametrize("model,inner,batch,sync", [(api.MODEL.GPT3, 6144, 16, api.SYNC.STREAM), (api.MODEL.GPT3, 6144, 256, api.SYNC.ROW),
+                                                    (api.MODEL.GPT3, 6144, 2048, api.SYNC.TILE), (api.MODEL.LLAMA, 2752, 64, api.SYNC.ROW),
+                                                    (api.MODEL.LLAMA, 2752, 1024, api.SYNC.TILE)])
+def test_mlp_with_repacked_weights(model, inner, batch, sync):
+    # repack_weights: the GEMMs read padded copies of the weights; same arithmetic, so bit-identical outputs
+    print("repacked weights", model, inner, batch, sync, flush=True)
+    hidden = 12288 if model == api.MODEL.GPT3 else 8192
+    x, w1, w2, h0, y0, _, _, tiles0, _ = run_mlp(model, batch, hidden, inner, sync)
+    _, _, _, h1, y1, prod, cons, tiles1, _ = run_mlp(model, batch, hidden, inner, sync, repack_weights=True)
+    assert tiles0 == tiles1
+    assert np.array_equal(h0, h1) and np.array_equal(y0, y1)
+    assert cons.spin_timeouts == 0
+    check_against_oracle(model, x, w1, w2, h1, y1, inner)
+
+
+def test_mlp_repacked_weights_reload():
+    # the handle keeps its own copies: a change of the caller's weights shows only after reload_weights()
+    import torch
+    batch, hidden, inner = 32, GPT3["hidden"], GPT3["inner"]
+    w1, w2, dw1, dw2 = weights(api.MODEL.GPT3, hidden, inner)
+    mine1, mine2 = dw1.clone(), dw2.clone()
+    x = uniform_f16((batch, hidden), 1)
+    dx = to_dev(x)
+    dh, dy = empty_dev((batch, inner)), empty_dev((batch, hidden))
+    torch.cuda.synchronize()
+    mlp = api.Mlp(api.MODEL.GPT3, batch, hidden, inner, api.SYNC.ROW, mine1.data_ptr(), mine2.data_ptr(), repack_weights=True)
+    mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    y_first = to_host(dy)
+    mine2.neg_()
+    torch.cuda.synchronize()
+    mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    assert np.array_equal(to_host(dy), y_first)
+    assert mlp.reload_weights() == api.ERR.SUCCESS
+    mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    y_reloaded = to_host(dy)
+    # same arithmetic as a handle that reads the changed weights in place
+    fresh = api.Mlp(api.MODEL.GPT3, batch, hidden, inner, api.SYNC.ROW, mine1.data_ptr(), mine2.data_ptr())
+    fresh.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    fresh.destroy()
+    assert np.array_equal(y_reloaded, to_host(dy))
+    assert not np.array_equal(y_reloaded, y_first)
+    assert_close(y_reloaded, -y_first, "Y with W2 negated")
+    assert mlp.stage_state(1).spin_timeouts == 0
+    mlp.destroy()
+    check_against_oracle(api.MODEL.GPT3, x, w1, w2, to_host(dh), y_first, inner)
