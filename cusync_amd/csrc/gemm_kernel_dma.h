@@ -219,7 +219,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // ---- consumer side (same protocol as the staged kernel) ------------------
     uint32_t nextColTile = kBegin / tnq;
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
-    uint32_t polledTile = 0xffffffffu, polledValue = 0;
+    uint32_t readyEnd = 0;        // column tiles of the producer below this one are known to be posted (one row block)
     auto waitRows = [&](uint32_t col, uint32_t z) {
       for (uint32_t r = m0; r < mEnd; r = (r / tmq + 1) * tmq) {
         cusync_dim3 w = {r, col, z};
@@ -261,17 +261,10 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       }
       const uint32_t kLast = min(k0 + (uint32_t)C::BK, kEnd) - 1;
       for (; nextColTile <= kLast / tnq; nextColTile++) {
-        if (oneRowBlock && nextColTile == polledTile && cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) continue;
-        waitRows(nextColTile * tnq, 0);
+        if (nextColTile < readyEnd) continue;            // seen posted by an earlier look-ahead
+        if (oneRowBlock) readyEnd = nextColTile + stage.waitWaveAhead(m0, nextColTile * tnq, tnq, (kEnd - 1) / tnq - nextColTile + 1);
+        else waitRows(nextColTile * tnq, 0);
       }
-    };
-    auto earlyPoll = [&](uint32_t k0) {
-      if (conv || !oneRowBlock || k0 >= kEnd) return;
-      const uint32_t ct = k0 / tnq;
-      if (ct < nextColTile || ct == polledTile) return;
-      polledTile = ct;
-      cusync_dim3 w = {m0, ct * tnq, 0};
-      polledValue = stage.peekBegin(w);
     };
 
     // Direct load number q (B loads first, then A) of chunk kt into stage S.
@@ -371,7 +364,6 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       asm volatile("" ::: "memory");
       const uint32_t ktLoad = kt + C::STAGES - 1;
       if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
-      earlyPoll(kBegin + (ktLoad + 1) * C::BK);
       __builtin_amdgcn_sched_barrier(0);
       compute(SP, Parity<(S + C::STAGES - 1) % C::STAGES>{}, ktLoad);
       __builtin_amdgcn_sched_barrier(0);
@@ -420,7 +412,6 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       asm volatile("" ::: "memory");
       const uint32_t ktLoad = kt + C::STAGES - 1;
       if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
-      earlyPoll(kBegin + (ktLoad + 1) * C::BK);
       __builtin_amdgcn_sched_barrier(0);
       // k-step 1 while the first fragments of chunk kt+1 arrive and the loads of chunk ktLoad go out
       staticFor<R>([&](auto FP) {
@@ -449,7 +440,6 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); issueAll(Parity<2>{}, 2); }
     if constexpr (C::STAGES > 4) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); issueAll(Parity<3>{}, 3); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 5, "prologue written for 2..5 stages");
-    earlyPoll(kBegin + (C::STAGES - 1) * C::BK);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
 
     if constexpr (C::PIPE) {

@@ -200,6 +200,34 @@ struct DynStage {
       dev::ticketAdd(d.spinTimeouts, 1);
   }
 
+  // Wave-uniform wait for tile {row, col, 0} that looks ahead: the first poll reads, one per lane, the
+  // semaphores of up to `count` (at most 16) tiles {row, col + i * colStep, 0} in one round trip and
+  // returns how many of them, counted from the first, are posted.  If the first is not, the wave spins on
+  // that one alone (sixteen lanes polling for as long as the producer needs would be sixteen times the
+  // traffic on the semaphores) and returns 1.  A consumer that is several tiles behind its producer
+  // then polls once per sixteen tiles instead of once per tile; every poll is a round trip to memory
+  // that the loads already in flight have to drain behind.
+  __device__ __forceinline__ uint32_t waitWaveAhead(uint32_t row, uint32_t col, uint32_t colStep, uint32_t count) const {
+    const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint32_t n = count < 16u ? count : 16u;
+    const cusync_dim3 mine = {row, col + (lane < n ? lane : 0u) * colStep, 0};
+    const bool polls = lane < n && needsWait(mine);
+    const uint32_t target = waitTarget();
+    uint32_t v = 0xffffffffu;
+    if (polls) v = dev::loadRelaxed(&d.tileStatusRead[dyn::tileIndex(d.in, mine, d.prodGrid) * CUSYNC_SEM_STRIDE]);
+    const uint64_t pending = __ballot(v < target);
+    uint32_t ready = pending ? (uint32_t)__builtin_ctzll(pending) : n;
+    if (ready > n) ready = n;
+    if (ready == 0) {
+      const cusync_dim3 first = {row, col, 0};
+      waitWave(first);           // spins, fences, counts a time-out
+      return 1;
+    }
+    if (lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    else dev::acquireFence();
+    return ready;
+  }
+
   // Workgroup-wide post; contains a barrier, call from all threads.
   __device__ __forceinline__ void post(const cusync_dim3& tile) const {
     if (!isProducer()) return;
