@@ -109,10 +109,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   auto waitRows = [&](uint32_t rowBegin, uint32_t rowEnd, uint32_t col) {
     if (!consumer) return;
     const uint32_t c = col / tnq * tnq;
-    for (uint32_t r = rowBegin; r < rowEnd; r = (r / tmq + 1) * tmq) {
-      cusync_dim3 w = {r, c, zWait};
-      stage.waitWave(w);
-    }
+    if (rowBegin < rowEnd) stage.waitWaveRows(rowBegin, rowEnd - 1, tmq, c, zWait);
   };
 
   // Thread 0 keeps the ticket state: the start count is issued first and settled after the

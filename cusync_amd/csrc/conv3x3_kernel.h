@@ -124,11 +124,11 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     if (consumer) {
       const uint32_t lo = m0 > W + 1 ? m0 - (W + 1) : 0, hiRow = min(m0 + C::BM + W, p.M - 1);
       if (stage.d.in.kind == CUSYNC_POLICY_ROWSYNC) {
-        for (uint32_t r = lo; r <= hiRow; r = (r / tmq + 1) * tmq) { cusync_dim3 w = {r, 0, 1}; stage.waitWave(w); }
+        stage.waitWaveRows(lo, hiRow, tmq, 0, 1);
       } else {
         const uint32_t perTile = stage.d.in.kind == CUSYNC_POLICY_CONV2DTILESYNC ? 9 * tnq : tnq;
         for (uint32_t ct = 0; ct < Cc / tnq; ct++)
-          for (uint32_t r = lo; r <= hiRow; r = (r / tmq + 1) * tmq) { cusync_dim3 w = {r, ct * perTile, 0}; stage.waitWave(w); }
+          stage.waitWaveRows(lo, hiRow, tmq, ct * perTile, 0);
       }
     }
 

@@ -220,12 +220,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     uint32_t nextColTile = kBegin / tnq;
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
     uint32_t readyEnd = 0;        // column tiles of the producer below this one are known to be posted (one row block)
-    auto waitRows = [&](uint32_t col, uint32_t z) {
-      for (uint32_t r = m0; r < mEnd; r = (r / tmq + 1) * tmq) {
-        cusync_dim3 w = {r, col, z};
-        stage.waitWave(w);
-      }
-    };
+    auto waitRows = [&](uint32_t col, uint32_t z) { stage.waitWaveRows(m0, mEnd - 1, tmq, col, z); };
     // Convolution fed by another convolution: the rows of the producer's output
     // this tile reads are its own pixels plus the filter's halo, and a K chunk
     // (r, s, c0..) lies in the producer's column tile c0 / tileN.  Each column
@@ -244,10 +239,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     auto cvWaitRows = [&](uint32_t policyCol, uint32_t z) {
       uint32_t lo, hi;
       cvRowRange(lo, hi);
-      for (uint32_t r = lo; r <= hi; r = (r / tmq + 1) * tmq) {
-        cusync_dim3 w = {r, policyCol, z};
-        stage.waitWave(w);
-      }
+      stage.waitWaveRows(lo, hi, tmq, policyCol, z);
     };
     auto waitChunk = [&](uint32_t k0) {
       if (!chunkSync) return;

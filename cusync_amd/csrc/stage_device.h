@@ -200,6 +200,34 @@ struct DynStage {
       dev::ticketAdd(d.spinTimeouts, 1);
   }
 
+  // Wave-uniform wait for every tile {r, col, z} whose rows meet rowLo..rowHi (row blocks of tileM rows):
+  // one lane per row block, so that all their semaphores are read in the same round trips instead of one
+  // after the other.  A lane stops polling once its tile is posted.
+  __device__ __forceinline__ void waitWaveRows(uint32_t rowLo, uint32_t rowHi, uint32_t tileM, uint32_t col, uint32_t z) const {
+    if (!isConsumer()) return;
+    const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint32_t b0 = rowLo / tileM, blocks = rowHi / tileM - b0 + 1;
+    const uint32_t target = waitTarget();
+    bool timedOut = false;
+    for (uint32_t base = 0; base < blocks; base += 64) {
+      const uint32_t i = base + lane;
+      const cusync_dim3 mine = {(b0 + (i < blocks ? i : 0u)) * tileM, col, z};
+      bool pending = i < blocks && needsWait(mine);
+      const uint32_t* sem = &d.tileStatusRead[dyn::tileIndex(d.in, mine, d.prodGrid) * CUSYNC_SEM_STRIDE];
+      uint32_t polls = 0, naps = 1;
+      for (;;) {
+        if (pending && dev::loadRelaxed(sem) >= target) pending = false;
+        if (__ballot(pending) == 0) break;
+        if (++polls >= CUSYNC_SPIN_LIMIT) { timedOut = true; break; }
+        for (uint32_t n = 0; n < naps; n++) __builtin_amdgcn_s_sleep(16);
+        if (naps < CUSYNC_MAX_NAPS) naps <<= 1;
+      }
+    }
+    if (lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    else dev::acquireFence();
+    if (timedOut && lane == 0) dev::ticketAdd(d.spinTimeouts, 1);
+  }
+
   // Wave-uniform wait for tile {row, col, 0} that looks ahead: the first poll reads, one per lane, the
   // semaphores of up to `count` (at most 16) tiles {row, col + i * colStep, 0} in one round trip and
   // returns how many of them, counted from the first, are posted.  If the first is not, the wave spins on
