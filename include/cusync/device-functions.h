@@ -35,13 +35,14 @@ CUSYNC_DEVICE void acquireFence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "ag
 // post, a stage wired to the wrong producer) must not hold the GPU forever:
 // after this many polls the wait gives up and reports failure.  One poll is a
 // trip to the coherent level of the memory system plus a sleep that grows to
-// about two microseconds, so the default allows a second or two.
+// about one microsecond, so the default allows a second or two.
 #ifndef CUSYNC_SPIN_LIMIT
 #define CUSYNC_SPIN_LIMIT (1u << 20)
 #endif
-// Longest sleep between two polls, in units of 1024 clocks (about 0.43 us).
+// Longest sleep between two polls, in units of 1024 clocks (about 0.43 us).  Eight (3.5 us) cost the
+// chains 2-3 us per handover against two; one brought nothing more.
 #ifndef CUSYNC_MAX_NAPS
-#define CUSYNC_MAX_NAPS 8
+#define CUSYNC_MAX_NAPS 2
 #endif
 
 // First half of a poll by a whole wave: only the first active lane touches
@@ -59,7 +60,7 @@ CUSYNC_DEVICE uint32_t pollFinish(uint32_t begun) { return __builtin_amdgcn_read
 CUSYNC_DEVICE uint32_t pollOnce(const volatile uint32_t* addr) { return pollFinish(pollBegin(addr)); }
 
 // Polls *addr until it is >= want; returns false if the poll budget ran out.
-// Sleeps between polls and doubles the sleep up to a few microseconds: a
+// Sleeps between polls and doubles the sleep up to about a microsecond: a
 // semaphore is one address, and hundreds of waves polling it back to back would
 // saturate the memory channel it lives on and slow the very producer they are
 // waiting for.
