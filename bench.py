@@ -209,6 +209,7 @@ def main():
             # repack_weights): a column tile's k rows then spread over all memory channels instead of one class
             s_rp = trimmed(protocol(b, api.SYNC.STREAM, repack=True)[0])[0]
             r_rp = trimmed(protocol(b, api.SYNC.ROW, repack=True)[0])[0]
+            one_rp = trimmed(protocol(b, api.SYNC.ROW, one_launch=True, repack=True)[0])[0] if tiles[0] == tiles[1] else None
             s, s_sd = trimmed(t_s)
             r, r_sd = trimmed(t_r)
             t, t_sd = trimmed(t_t)
@@ -221,7 +222,8 @@ def main():
                 "tilesync_us": round(t, 2), "tilesync_std": round(t_sd, 2), "tilesync_gain_pct": round(100 - t / s * 100, 2),
                 "rowsync_one_launch_us": None if one is None else round(one, 2),
                 "repacked_weights": {"stream_us": round(s_rp, 2), "rowsync_us": round(r_rp, 2),
-                                     "roofline_frac": round(ideal_us(b) / min(s_rp, r_rp), 4)},
+                                     "rowsync_one_launch_us": None if one_rp is None else round(one_rp, 2),
+                                     "roofline_frac": round(ideal_us(b) / min(v for v in (s_rp, r_rp, one_rp) if v), 4)},
                 "best_tflops": round(mlp_flops(b) / best / 1e6, 1),
                 "bound": "mfma" if mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12) > mlp_bytes(b) / (PEAK_HBM_GBS * 1e9) else "hbm",
                 "roofline_frac": round(ideal_us(b) / best, 4),
