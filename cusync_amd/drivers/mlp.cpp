@@ -3,6 +3,10 @@
 //
 //   mlp --model gpt3|llama --batch <rows> [--check true|false] [--split-k1 n] [--split-k2 n]
 //       [--policy baseline|cusync|both] [--sync rowsync|tilesync|stridedsync] [--runs n]
+//       [--repack-weights true|false] [--one-launch true|false]
+//
+// --repack-weights: both chains read padded copies of the weights kept by the handle
+// (cusync_mlp_config.repack_weights); --one-launch: the CuSync chain runs both GEMMs in one launch.
 //
 // Output: "START-BASELINE:", one JSON object per timed run {"Total", "matmul1Time", "matmul2Time"} in
 // microseconds, "END-BASELINE:", then the same between START-OVERLAPPED: / END-OVERLAPPED: with {"Total"}
@@ -16,7 +20,8 @@ int main(int argc, char** argv) {
   const long batch = drv::getInt(args, "batch", 0);
   if ((model != "gpt3" && model != "llama") || batch <= 0) {
     fprintf(stderr, "usage: mlp --model gpt3|llama --batch <int> [--check true|false] [--split-k1 <int>] [--split-k2 <int>] "
-                    "[--policy baseline|cusync|both] [--sync rowsync|tilesync|stridedsync] [--runs <int>]\n");
+                    "[--policy baseline|cusync|both] [--sync rowsync|tilesync|stridedsync] [--runs <int>] "
+                    "[--repack-weights true|false] [--one-launch true|false]\n");
     return EXIT_FAILURE;
   }
   const bool check = drv::getBool(args, "check", false);
@@ -46,6 +51,8 @@ int main(int argc, char** argv) {
     c.tile1 = c.tile2 = -1; c.opts = -1;
     c.activation = llama ? 0 : 1;        // the reference's LLaMA chain multiplies the gate half as is (mlp.cu:785-792)
     c.split_k1 = (int)drv::getInt(args, "split-k1", 0); c.split_k2 = (int)drv::getInt(args, "split-k2", 0);
+    c.repack_weights = drv::getBool(args, "repack-weights", false) ? 1 : 0;
+    c.one_launch = (mode != CUSYNC_SYNC_STREAM && drv::getBool(args, "one-launch", false)) ? 1 : 0;
     cusync_mlp* m = cusync_mlp_create(&c, w1, w2);
     if (!m) { fprintf(stderr, "cusync_mlp_create failed: %s\n", cusync_rt_last_error()); exit(EXIT_FAILURE); }
     DRV_CHECK(cusync_mlp_run(m, x, h, y, warmup, nullptr));

@@ -39,6 +39,13 @@ def test_mlp_driver(model, batch, sync):
     assert "check: passed" in out
 
 
+def test_mlp_driver_repacked_weights_one_launch():
+    out = run("mlp", "--model", "gpt3", "--batch", "16", "--check", "true", "--sync", "rowsync", "--runs", "3",
+              "--repack-weights", "true", "--one-launch", "true")
+    over, _ = between(out, "START-OVERLAPPED:", "END-OVERLAPPED:")
+    assert len(over) == 3 and "check: passed" in out
+
+
 def test_mlp_driver_usage_error():
     p = subprocess.run([os.path.join(BIN, "mlp"), "--model", "bert"], capture_output=True, text=True, timeout=60)
     assert p.returncode != 0 and "usage" in p.stderr
