@@ -148,8 +148,15 @@ def main():
         for _ in range(3):
             torch.add(a, 1, out=b)
         torch.cuda.synchronize()
-        return {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+        # few rows: a launch streams its weight matrix once and that bounds it (algorithmic bytes: the operands once)
+        bytes_per_launch = 2.0 * (HIDDEN * INNER + B * HIDDEN + B * INNER)
+        hbm_bound = bytes_per_launch / (PEAK_HBM_GBS * 1e9) > flops_per_launch / (PEAK_FP16_TFLOPS * 1e12)
+        gbs = bytes_per_launch / (k_us * 1e-6) / 1e9
+        head = ({"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
+                if hbm_bound else
+                {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                 "frac": round(achieved / PEAK_FP16_TFLOPS, 4)})
+        return {**head, "traffic": None,
                 "kernel": "gemmDmaKernel, mean of the two launches of the step: GEMM1 tile %s %.1f us, GEMM2 tile %s %.1f us "
                           "(stream-ordered, %.1f GFLOP per launch)" % (shapes[0], statistics.fmean(g1), shapes[1], statistics.fmean(g2),
                                                                        flops_per_launch / 1e9),
@@ -343,14 +350,15 @@ def main():
 
     # stream-ordered on the same shape: baseline latency and the kernels' own durations
     roof, stream_us, _ = roofline_leg(B, args.warmup, max(10, args.steps))
-    roof["traffic"] = TRAFFIC_BYTES_PER_LAUNCH
+    roof["traffic"] = TRAFFIC_BYTES_PER_LAUNCH if B == 2048 else None      # counters were taken at the default batch
     # what the matrix pipes alone sustain on this machine (register operands, no LDS, no memory): the clock
     # drops under a device-wide MFMA load, further with random operands than with zeros
     zero_tf, zero_mhz = api.probe_mfma_rate(False)
     rand_tf, rand_mhz = api.probe_mfma_rate(True)
     roof["mfma_alone"] = {"zero_operands_tflops": round(zero_tf, 1), "zero_operands_mhz": round(zero_mhz),
-                          "random_operands_tflops": round(rand_tf, 1), "random_operands_mhz": round(rand_mhz),
-                          "frac_of_random_operands_rate": round(roof["achieved"] / rand_tf, 4)}
+                          "random_operands_tflops": round(rand_tf, 1), "random_operands_mhz": round(rand_mhz)}
+    if roof["bound"] == "mfma":
+        roof["mfma_alone"]["frac_of_random_operands_rate"] = round(roof["achieved"] / rand_tf, 4)
 
     out = {
         "metric": "GPT-3 MLP shard latency (us) + % gain vs kernel-boundary sync, B=1..2048",
