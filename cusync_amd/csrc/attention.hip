@@ -68,7 +68,17 @@ struct cusync_attn_layer {
   cusync_stage_desc st[3];         // QKV projection, attention, output projection
   hipStream_t stream[3];
   hipEvent_t eStart, eMid1, eMid2, eEnd;
+  uint32_t timeoutsSeen;           // sum of the stages' give-up counters when the last run returned
 };
+
+extern "C" void cusync_attn_layer_destroy(cusync_attn_layer* L);
+
+// create() failed: gives back what the handle holds so far and keeps the text of the failure
+static void discardLayer(cusync_attn_layer* L) {
+  const std::string why = cusync_rt_last_error();
+  cusync_attn_layer_destroy(L);
+  cusync::rt::setError(why);
+}
 
 extern "C" {
 
@@ -148,7 +158,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
 
   AttnParams p = {};
   p.stage.d = s;
-  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->qkv % 128 == 0 && (a->ldqkv * 2) % 128 == 0 &&
+  p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->qkv % 128 == 0 && (a->ldqkv * 2) % 128 == 0 &&
                         (s.in.kind != CUSYNC_POLICY_TILESYNC || (s.in.tileN * 2) % 128 == 0);
   p.S = a->seq; p.heads = a->heads; p.cached = a->cached_rows;
   p.qkv = (const half_t*)a->qkv; p.ldq = a->ldqkv;
@@ -204,7 +214,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
     setError("attn layer: unknown tile id");
-    delete L;
+    discardLayer(L);
     return nullptr;
   }
   // few rows leave most CUs without a tile: k-slices as in the MLP chain
@@ -238,7 +248,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
       opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
       break;
     case CUSYNC_SYNC_STRIDED:   // ConsecutiveSync into the attention, RowSync out of it, attention.cu:98-110
-      if (L->E % tn1) { setError("attn layer: ConsecutiveSync needs heads*128 % tileN == 0"); delete L; return nullptr; }
+      if (L->E % tn1) { setError("attn layer: ConsecutiveSync needs heads*128 % tileN == 0"); discardLayer(L); return nullptr; }
       sync1.kind = CUSYNC_POLICY_CONSECUTIVESYNC; sync1.order = CUSYNC_ORDER_TRANSPOSE_XY;
       sync1.tileM = tm1; sync1.tileN = tn1; sync1.H = 8 * L->E;
       sync1.waitValue = L->E / tn1; sync1.postValue = 1;
@@ -247,7 +257,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
       break;
     default:
       setError("attn layer: unknown sync mode");
-      delete L;
+      discardLayer(L);
       return nullptr;
   }
   if (cfg->opts >= 0) opts |= cfg->opts;
@@ -258,13 +268,13 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
     memset(&L->st[i], 0, sizeof L->st[i]);
     L->st[i].grid = grids[i]; L->st[i].tileSize = {1, 1, 1}; L->st[i].iter = 1; L->st[i].opts = opts;
     L->st[i].in = ins[i]; L->st[i].out = outs[i];
-    if (cusync_stage_create(&L->st[i], CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) { delete L; return nullptr; }
+    if (cusync_stage_create(&L->st[i], CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) { discardLayer(L); return nullptr; }
   }
   if (cfg->sync != CUSYNC_SYNC_STREAM &&
       (cusync_set_producer_consumer_pair(&L->st[0], &L->st[1]) != CUSYNC_SUCCESS ||
        cusync_set_producer_consumer_pair(&L->st[1], &L->st[2]) != CUSYNC_SUCCESS)) {
     setError("attn layer: pairing the stages failed");
-    delete L;
+    discardLayer(L);
     return nullptr;
   }
   for (int which = 0; which < 2; which++) {
@@ -277,7 +287,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
     const size_t bytes = cusync_gemm_workspace_size(&a);
     if (bytes == 0) continue;
     void* ws = nullptr;
-    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { delete L; return nullptr; }
+    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { discardLayer(L); return nullptr; }
     (which == 0 ? L->ws1 : L->ws3) = ws;
   }
   {
@@ -285,21 +295,23 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
     memset(&a, 0, sizeof a);
     a.seq = cfg->seq; a.heads = cfg->heads; a.cached_rows = cfg->cached_rows; a.kv_split_blocks = L->kvSplit;
     const size_t bytes = cusync_attention_workspace_size(&a);
-    if (bytes && (CUSYNC_HIP(hipMalloc(&L->ws2, bytes)) || CUSYNC_HIP(hipMemset(L->ws2, 0, bytes)))) { delete L; return nullptr; }
+    if (bytes && (CUSYNC_HIP(hipMalloc(&L->ws2, bytes)) || CUSYNC_HIP(hipMemset(L->ws2, 0, bytes)))) { discardLayer(L); return nullptr; }
   }
   for (int i = 0; i < 3; i++)
-    if (CUSYNC_HIP(hipStreamCreateWithFlags(&L->stream[i], hipStreamNonBlocking))) { delete L; return nullptr; }
+    if (CUSYNC_HIP(hipStreamCreateWithFlags(&L->stream[i], hipStreamNonBlocking))) { discardLayer(L); return nullptr; }
   if (CUSYNC_HIP(hipEventCreate(&L->eStart)) || CUSYNC_HIP(hipEventCreate(&L->eMid1)) ||
-      CUSYNC_HIP(hipEventCreate(&L->eMid2)) || CUSYNC_HIP(hipEventCreate(&L->eEnd))) { delete L; return nullptr; }
+      CUSYNC_HIP(hipEventCreate(&L->eMid2)) || CUSYNC_HIP(hipEventCreate(&L->eEnd))) { discardLayer(L); return nullptr; }
   return L;
 }
 
+// Also the clean-up of a create() that failed half way: the handle is value-initialised, so what has not
+// been made yet is null and skipped.
 void cusync_attn_layer_destroy(cusync_attn_layer* L) {
   if (!L) return;
-  for (int i = 0; i < 3; i++) (void)hipStreamSynchronize(L->stream[i]);
+  for (int i = 0; i < 3; i++) if (L->stream[i]) (void)hipStreamSynchronize(L->stream[i]);
   for (int i = 0; i < 3; i++) cusync_stage_free(&L->st[i]);
-  (void)hipEventDestroy(L->eStart); (void)hipEventDestroy(L->eMid1); (void)hipEventDestroy(L->eMid2); (void)hipEventDestroy(L->eEnd);
-  for (int i = 0; i < 3; i++) (void)hipStreamDestroy(L->stream[i]);
+  for (hipEvent_t e : {L->eStart, L->eMid1, L->eMid2, L->eEnd}) if (e) (void)hipEventDestroy(e);
+  for (int i = 0; i < 3; i++) if (L->stream[i]) (void)hipStreamDestroy(L->stream[i]);
   if (L->ws1) (void)hipFree(L->ws1);
   if (L->ws3) (void)hipFree(L->ws3);
   if (L->ws2) (void)hipFree(L->ws2);
@@ -359,7 +371,9 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     }
     for (int i = 0; i < 3; i++) L->st[i].iter += 1;
   }
-  return CUSYNC_SUCCESS;
+  // every run above was synchronised with; a wait that gave up let its kernel go on with unposted data
+  const cusync_stage_desc* stages[3] = {&L->st[0], &L->st[1], &L->st[2]};
+  return cusync::rt::checkSpinTimeouts(stages, 3, &L->timeoutsSeen, "attn layer");
 }
 
 const cusync_stage_desc* cusync_attn_layer_stage(const cusync_attn_layer* L, int which) {

@@ -106,10 +106,15 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
   const uint32_t zWait = consumer && (stage.d.in.kind == CUSYNC_POLICY_ROWSYNC ||
                                       stage.d.in.kind == CUSYNC_POLICY_CONSECUTIVESYNC) ? 1 : 0;
   // Every wave waits for itself: each one fetches part of every block.
+  // `col`: first of the kHD columns of qkv that are about to be read.  They can lie in more than one of the
+  // producer's column tiles (192-wide tiles against 128-wide heads): every one of them is waited for.  The
+  // row policies guard whole rows of a third of qkv with one semaphore, so one wait covers all columns.
   auto waitRows = [&](uint32_t rowBegin, uint32_t rowEnd, uint32_t col) {
-    if (!consumer) return;
-    const uint32_t c = col / tnq * tnq;
-    if (rowBegin < rowEnd) stage.waitWaveRows(rowBegin, rowEnd - 1, tmq, c, zWait);
+    if (!consumer || rowBegin >= rowEnd) return;
+    for (uint32_t c = col / tnq * tnq; c < col + kHD; c += tnq) {
+      stage.waitWaveRows(rowBegin, rowEnd - 1, tmq, c, zWait);
+      if (zWait) break;
+    }
   };
 
   // Thread 0 keeps the ticket state: the start count is issued first and settled after the

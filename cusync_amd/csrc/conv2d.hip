@@ -123,7 +123,7 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
   p.mPad = s.grid.y * ti->bm;
   // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
-  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
+  p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
                         (a->C * 2) % 128 == 0 &&
                         (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
   return p;
@@ -227,9 +227,17 @@ struct cusync_conv_chain {
   std::vector<cusync_stage_desc> st;
   std::vector<hipStream_t> stream;
   std::vector<hipEvent_t> ev;        // layers + 1 events: start, after each layer
+  uint32_t timeoutsSeen = 0;         // sum of the stages' give-up counters when the last run returned
 };
 
 namespace {
+
+// After the runs of a call have been synchronised with: an error if a wait of any layer gave up meanwhile.
+cusync_error chainTimeouts(cusync_conv_chain* c) {
+  std::vector<const cusync_stage_desc*> stages;
+  for (const auto& d : c->st) stages.push_back(&d);
+  return cusync::rt::checkSpinTimeouts(stages.data(), (int)stages.size(), &c->timeoutsSeen, "conv chain");
+}
 
 cusync_policy_desc noSyncDesc() {
   cusync_policy_desc p;
@@ -374,7 +382,7 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
       }
       for (uint32_t i = 0; i < n; i++) c->st[i].iter += 1;
     }
-    return CUSYNC_SUCCESS;
+    return chainTimeouts(c);
   }
   for (int r = 0; r < runs; r++) {
     if (CUSYNC_HIP(hipEventRecord(c->ev[0], c->stream[0]))) return CUSYNC_ERROR_DEVICE;
@@ -405,7 +413,7 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
       }
     for (uint32_t i = 0; i < n; i++) c->st[i].iter += 1;
   }
-  return CUSYNC_SUCCESS;
+  return chainTimeouts(c);
 }
 
 const cusync_stage_desc* cusync_conv_chain_stage(const cusync_conv_chain* c, uint32_t which) {

@@ -205,7 +205,7 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   p.stage.d = s;
   // Producer tiles are whole 128-byte lines of A when the row pitch, the base and
   // the producer's tile width all are multiples of 128 bytes (64 halfs).
-  p.stage.lineAligned = s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 && (a->lda * 2) % 128 == 0 &&
+  p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 && (a->lda * 2) % 128 == 0 &&
                         (s.in.kind == CUSYNC_POLICY_ROWSYNC || s.in.kind == CUSYNC_POLICY_CONSECUTIVESYNC ||
                          (s.in.tileN * 2) % 128 == 0);       // the row policies guard whole rows
   p.M = a->M; p.N = a->N; p.K = a->K;

@@ -130,7 +130,16 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     auto waitColTile = [&](uint32_t ct) {
       if (oneRowBlock && ct == polledTile) {
         cusync_dim3 w = {m0, ct * tnq, 0};
-        if (!stage.needsWait(w) || cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) return;
+        if (!stage.needsWait(w)) return;
+        if (cusync::dev::pollFinish(polledValue) >= stage.waitTarget()) {
+          // The early poll was a relaxed load: it still needs the acquire a wait ends with.  Where a
+          // producer tile is not a whole number of cache lines of A (a pitch or a base that is not a
+          // multiple of 128 bytes) a line can straddle a posted and an unposted tile and sit in this
+          // XCD's caches already; only the agent-scope acquire drops it.
+          if (stage.lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          else cusync::dev::acquireFence();
+          return;
+        }
       }
       waitRows(ct * tnq, 0);
     };

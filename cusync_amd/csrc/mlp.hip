@@ -37,10 +37,7 @@ struct cusync_mlp {
   void* act;                         // [batch][inner] fp16, GEMM2's A operand
   cusync_stage_desc mid;
   hipStream_t sMid;
-  ~cusync_mlp() {
-    if (w1p) (void)hipFree(w1p);
-    if (w2p) (void)hipFree(w2p);
-  }
+  uint32_t timeoutsSeen;             // sum of the stages' give-up counters when the last run returned
 };
 
 namespace {
@@ -122,16 +119,22 @@ __global__ __launch_bounds__(kActThreads) void swigluStageKernel(ActParams p) {
   }
 }
 
-int g_actResident = 0;
-
-cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
-  if (g_actResident == 0) {
+// Workgroups of the activation kernel that stay resident on the device; 0 if the runtime would not say.
+// Worked out once (the initialisation of a function-local static is safe against concurrent first calls).
+int actResident() {
+  static const int resident = [] {
     int dev = 0, perCU = 0;
     hipDeviceProp_t prop;
     if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev)) ||
-        CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, swigluStageKernel, (int)kActThreads, 0))) return CUSYNC_ERROR_DEVICE;
-    g_actResident = std::max(1, std::min(perCU, 4)) * prop.multiProcessorCount;
-  }
+        CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, swigluStageKernel, (int)kActThreads, 0))) return 0;
+    return std::max(1, std::min(perCU, 4)) * prop.multiProcessorCount;
+  }();
+  return resident;
+}
+
+cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
+  const int resident = actResident();
+  if (resident <= 0) return CUSYNC_ERROR_DEVICE;
   const cusync_stage_desc& s = m->mid;
   ActParams p = {};
   p.stage.d = s;
@@ -139,7 +142,7 @@ cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
   p.M = m->cfg.batch; p.d = m->cfg.inner;
   p.G = (const half_t*)h; p.ldg = m->ldh;
   p.A = (half_t*)m->act; p.lda = m->cfg.inner;
-  p.launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)g_actResident);
+  p.launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)resident);
   hipLaunchKernelGGL(swigluStageKernel, dim3(p.launched), dim3(kActThreads), 0, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
@@ -231,6 +234,13 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
   return a;
 }
 
+// create() failed: gives back what the handle holds so far and keeps the text of the failure
+void discard(cusync_mlp* m) {
+  const std::string why = cusync_rt_last_error();
+  cusync_mlp_destroy(m);
+  setError(why);
+}
+
 }  // namespace
 
 extern "C" {
@@ -256,7 +266,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     if (CUSYNC_HIP(hipMalloc(&m->w1p, (size_t)m->k1 * m->ldw1 * sizeof(half_t))) ||
         CUSYNC_HIP(hipMalloc(&m->w2p, (size_t)m->k2 * m->ldw2 * sizeof(half_t))) ||
         cusync_mlp_reload_weights(m) != CUSYNC_SUCCESS) {
-      delete m;
+      discard(m);
       return nullptr;
     }
   }
@@ -275,7 +285,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
     setError("mlp: unknown tile id");
-    delete m;
+    discard(m);
     return nullptr;
   }
 
@@ -304,8 +314,8 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
       break;
     case CUSYNC_SYNC_STRIDED:    // StridedSync<TransposeXY,d,kM,kN,2>, mlp.cu:109; atomic add kept (:9-14)
-      if (!llama) { setError("mlp: StridedSync is for the gate|up layout"); delete m; return nullptr; }
-      if (cfg->inner % tn1 != 0) { setError("mlp: StridedSync needs inner % tileN == 0"); delete m; return nullptr; }
+      if (!llama) { setError("mlp: StridedSync is for the gate|up layout"); discard(m); return nullptr; }
+      if (cfg->inner % tn1 != 0) { setError("mlp: StridedSync needs inner % tileN == 0"); discard(m); return nullptr; }
       pol.kind = CUSYNC_POLICY_STRIDEDSYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
       pol.tileM = tm1; pol.tileN = tn1; pol.waitValue = 2; pol.postValue = 1;
       pol.gridN = cfg->inner; pol.stride = 2;
@@ -313,7 +323,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       break;
     default:
       setError("mlp: unknown sync mode");
-      delete m;
+      discard(m);
       return nullptr;
   }
   if (cfg->opts >= 0) opts |= cfg->opts;
@@ -323,7 +333,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     const bool direct = bk == 32 || m->tile1 >= CUSYNC_TILE_D32x128x64;      // the direct-to-LDS tiles
     if (m->tile1 != m->tile2 || !direct || m->aMode2 != CUSYNC_A_PLAIN || m->actStage) {
       setError("mlp: one launch for both GEMMs needs the same direct-to-LDS tile for both and a plain A operand");
-      delete m;
+      discard(m);
       return nullptr;
     }
   }
@@ -346,7 +356,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->cons.in = m->actStage ? pol2 : pol; m->cons.out = noSync();
   if (cusync_stage_create(&m->prod, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS ||
       cusync_stage_create(&m->cons, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS) {
-    delete m;
+    discard(m);
     return nullptr;
   }
   if (m->actStage) {
@@ -355,7 +365,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     if (cusync_stage_create(&m->mid, CUSYNC_ORDER_TRANSPOSE_XY) != CUSYNC_SUCCESS ||
         CUSYNC_HIP(hipMalloc(&m->act, (size_t)cfg->batch * cfg->inner * sizeof(half_t))) ||
         CUSYNC_HIP(hipStreamCreateWithFlags(&m->sMid, hipStreamNonBlocking))) {
-      delete m;
+      discard(m);
       return nullptr;
     }
   }
@@ -365,7 +375,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
                                 : cusync_set_producer_consumer_pair(&m->prod, &m->cons) == CUSYNC_SUCCESS;
     if (!ok) {
       setError("mlp: pairing the stages failed");
-      delete m;
+      discard(m);
       return nullptr;
     }
   }
@@ -374,14 +384,14 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     const size_t bytes = cusync_gemm_workspace_size(&a);
     if (bytes == 0) continue;
     void* ws = nullptr;
-    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { delete m; return nullptr; }
+    if (CUSYNC_HIP(hipMalloc(&ws, bytes)) || CUSYNC_HIP(hipMemset(ws, 0, bytes))) { discard(m); return nullptr; }
     (which == 0 ? m->ws1 : m->ws2) = ws;
   }
   if (CUSYNC_HIP(hipStreamCreateWithFlags(&m->sProd, hipStreamNonBlocking)) ||
       CUSYNC_HIP(hipStreamCreateWithFlags(&m->sCons, hipStreamNonBlocking)) ||
       CUSYNC_HIP(hipEventCreate(&m->eStart)) || CUSYNC_HIP(hipEventCreate(&m->eMid)) ||
       CUSYNC_HIP(hipEventCreate(&m->eEnd))) {
-    delete m;
+    discard(m);
     return nullptr;
   }
   return m;
@@ -407,21 +417,27 @@ cusync_error cusync_mlp_reload_weights(cusync_mlp* m) {
   return CUSYNC_SUCCESS;
 }
 
+// Also the clean-up of a create() that failed half way: every member is null until it has been made
+// (the handle is value-initialised), and everything here skips what is null.
 void cusync_mlp_destroy(cusync_mlp* m) {
   if (!m) return;
-  (void)hipStreamSynchronize(m->sProd);
-  (void)hipStreamSynchronize(m->sCons);
-  cusync_stage_free(&m->prod);
+  if (m->sProd) (void)hipStreamSynchronize(m->sProd);
+  if (m->sCons) (void)hipStreamSynchronize(m->sCons);
+  if (m->sMid) (void)hipStreamSynchronize(m->sMid);
+  cusync_stage_free(&m->prod);        // null-safe per member
   cusync_stage_free(&m->cons);
-  if (m->actStage) {
-    if (m->sMid) { (void)hipStreamSynchronize(m->sMid); (void)hipStreamDestroy(m->sMid); }
-    cusync_stage_free(&m->mid);
-    if (m->act) (void)hipFree(m->act);
-  }
+  cusync_stage_free(&m->mid);
+  if (m->act) (void)hipFree(m->act);
   if (m->ws1) (void)hipFree(m->ws1);
   if (m->ws2) (void)hipFree(m->ws2);
-  (void)hipEventDestroy(m->eStart); (void)hipEventDestroy(m->eMid); (void)hipEventDestroy(m->eEnd);
-  (void)hipStreamDestroy(m->sProd); (void)hipStreamDestroy(m->sCons);
+  if (m->w1p) (void)hipFree(m->w1p);
+  if (m->w2p) (void)hipFree(m->w2p);
+  if (m->eStart) (void)hipEventDestroy(m->eStart);
+  if (m->eMid) (void)hipEventDestroy(m->eMid);
+  if (m->eEnd) (void)hipEventDestroy(m->eEnd);
+  if (m->sProd) (void)hipStreamDestroy(m->sProd);
+  if (m->sCons) (void)hipStreamDestroy(m->sCons);
+  if (m->sMid) (void)hipStreamDestroy(m->sMid);
   delete m;
 }
 
@@ -482,7 +498,9 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     m->cons.iter += 1;
     m->mid.iter += 1;
   }
-  return CUSYNC_SUCCESS;
+  // every run above was synchronised with; a wait that gave up let its kernel go on with unposted data
+  const cusync_stage_desc* stages[3] = {&m->prod, &m->cons, &m->mid};
+  return cusync::rt::checkSpinTimeouts(stages, 3, &m->timeoutsSeen, "mlp");
 }
 
 cusync_error cusync_mlp_run(cusync_mlp* m, const void* x, void* h, void* y, int runs, double* times_us) {

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <string>
 #include <vector>
@@ -28,6 +29,38 @@ int check(hipError_t e, const char* what, const char* file, int line) {
   return (int)e;
 }
 
+bool forceAcquire() {
+  static const bool on = [] {
+    const char* v = getenv("CUSYNC_FORCE_ACQUIRE");
+    return v && *v && strcmp(v, "0") != 0;
+  }();
+  return on;
+}
+
+bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t* sum) {
+  uint32_t total = 0;
+  for (int i = 0; i < count; i++) {
+    if (!stages[i] || !stages[i]->spinTimeouts) continue;
+    uint32_t v = 0;
+    if (check(hipMemcpy(&v, stages[i]->spinTimeouts, sizeof v, hipMemcpyDeviceToHost), "hipMemcpy(spinTimeouts)", __FILE__, __LINE__)) return false;
+    total += v;
+  }
+  *sum = total;
+  return true;
+}
+
+cusync_error checkSpinTimeouts(const cusync_stage_desc* const* stages, int count, uint32_t* seen, const char* what) {
+  uint32_t now = 0;
+  if (!spinTimeoutsOf(stages, count, &now)) return CUSYNC_ERROR_DEVICE;
+  if (now == *seen) return CUSYNC_SUCCESS;
+  char buf[256];
+  snprintf(buf, sizeof buf, "%s: %u wait(s) gave up after CUSYNC_SPIN_LIMIT polls and went on with data that was not "
+                            "posted; the outputs of this call are not valid", what, now - *seen);
+  *seen = now;
+  setError(buf);
+  return CUSYNC_ERROR_DEVICE;
+}
+
 }  // namespace rt
 }  // namespace cusync
 
@@ -35,8 +68,9 @@ int check(hipError_t e, const char* what, const char* file, int line) {
 
 // One wave; lane 0 polls.  Same contract as waitKernel of the reference
 // (src/cusync.cu:11-19) with a bounded spin.
-__global__ void cusync_wait_kernel_impl(const uint32_t* semaphore, uint32_t value) {
-  if (threadIdx.x == 0) cusync::dev::spinUntilAtLeast(semaphore, value);
+// A wait that gives up is counted in *timeouts (may be null), as the waits inside the kernels are.
+__global__ void cusync_wait_kernel_impl(const uint32_t* semaphore, uint32_t value, uint32_t* timeouts) {
+  if (threadIdx.x == 0 && !cusync::dev::spinUntilAtLeast(semaphore, value) && timeouts) cusync::dev::ticketAdd(timeouts, 1);
 }
 
 extern "C" {
@@ -102,8 +136,15 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   const size_t line = 128;
   char* counters = nullptr;
   if (RT(hipMalloc((void**)&counters, 13 * line))) return CUSYNC_ERROR_DEVICE;
-  if (RT(hipMemset(counters, 0, 13 * line))) return CUSYNC_ERROR_DEVICE;
-  d->tileCounter = (uint32_t*)(counters);
+  d->tileCounter = (uint32_t*)(counters);         // base of the block: what cusync_stage_free releases
+  // a failure from here on gives back what was allocated so far; the text of the failed call is kept
+  auto fail = [&]() {
+    const std::string why = cusync_rt_last_error();
+    cusync_stage_free(d);
+    cusync::rt::setError(why);
+    return CUSYNC_ERROR_DEVICE;
+  };
+  if (RT(hipMemset(counters, 0, 13 * line))) return fail();
   d->startCounter = (uint32_t*)(counters + line);
   d->spinTimeouts = (uint32_t*)(counters + 2 * line);
   d->xcdTickets = (uint32_t*)(counters + 4 * line);
@@ -115,11 +156,11 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
     identity = t.x == i % d->grid.x && t.y == (i / d->grid.x) % d->grid.y && t.z == i / (d->grid.x * d->grid.y);
   }
   d->flags = identity ? CUSYNC_STAGE_IDENTITY_ORDER : 0;
-  if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return CUSYNC_ERROR_DEVICE;
-  if (RT(hipMemcpy(d->tileOrder, host_tile_order, sizeof(cusync_dim3) * n, hipMemcpyHostToDevice))) return CUSYNC_ERROR_DEVICE;
+  if (RT(hipMalloc((void**)&d->tileOrder, sizeof(cusync_dim3) * n))) return fail();
+  if (RT(hipMemcpy(d->tileOrder, host_tile_order, sizeof(cusync_dim3) * n, hipMemcpyHostToDevice))) return fail();
   if (producer) {
-    if (RT(hipMalloc((void**)&d->tileStatusWrite, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return CUSYNC_ERROR_DEVICE;
-    if (RT(hipMemset(d->tileStatusWrite, 0, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return CUSYNC_ERROR_DEVICE;
+    if (RT(hipMalloc((void**)&d->tileStatusWrite, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return fail();
+    if (RT(hipMemset(d->tileStatusWrite, 0, sizeof(uint32_t) * n * CUSYNC_SEM_STRIDE))) return fail();
   }
   return CUSYNC_SUCCESS;
 }
@@ -167,18 +208,22 @@ cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc* prod, cu
   return CUSYNC_SUCCESS;
 }
 
-cusync_error cusync_wait_kernel(uint32_t* semaphore, uint32_t value, void* stream) {
+static cusync_error launchWaitKernel(uint32_t* semaphore, uint32_t value, uint32_t* timeouts, void* stream) {
   if (!semaphore) return CUSYNC_ERROR_NOT_INITIALIZED;
-  hipLaunchKernelGGL(cusync_wait_kernel_impl, dim3(1), dim3(64), 0, (hipStream_t)stream, semaphore, value);
+  hipLaunchKernelGGL(cusync_wait_kernel_impl, dim3(1), dim3(64), 0, (hipStream_t)stream, semaphore, value, timeouts);
   if (RT(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
+}
+
+cusync_error cusync_wait_kernel(uint32_t* semaphore, uint32_t value, void* stream) {
+  return launchWaitKernel(semaphore, value, nullptr, stream);
 }
 
 cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc* prod, void* stream) {
   if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
   if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
   if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
-  return cusync_wait_kernel(prod->kernelExecuted, (uint32_t)prod->iter, stream);
+  return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
 cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void* stream, void* launch_event) {
@@ -186,7 +231,7 @@ cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void
   if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
   if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
   if (launch_event && RT(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)launch_event, 0))) return CUSYNC_ERROR_DEVICE;
-  return cusync_wait_kernel(prod->kernelExecuted, (uint32_t)prod->iter, stream);
+  return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
 cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems, cusync_dim3* tile_order,

@@ -4,12 +4,25 @@
 #include <hip/hip_runtime.h>
 #include <string>
 
+#include "../../include/cusync_amd.h"
+
 namespace cusync {
 namespace rt {
 // Records `msg` as the text cusync_rt_last_error() returns (per host thread).
 void setError(const std::string& msg);
 // Returns 0 on hipSuccess; otherwise records a message and returns the code.
 int check(hipError_t e, const char* what, const char* file, int line);
+// True when the environment variable CUSYNC_FORCE_ACQUIRE is set to something other than 0: every consumer
+// wait then ends with the agent-scope acquire (cache invalidation), also where the launcher found that the
+// producer's tiles are whole cache lines of the consumer's operand and the invalidation can be skipped.
+bool forceAcquire();
+// Adds up the counters of waits that gave up (cusync_stage_desc::spinTimeouts) of the stages given; null
+// entries and stages without a counter are skipped.  Returns false if a copy from the device failed.
+bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t* sum);
+// For the chain handles, after the host has synchronised with a run: CUSYNC_SUCCESS if the sum above still
+// equals *seen, else records a message naming `what`, brings *seen up to date and returns CUSYNC_ERROR_DEVICE
+// (the chain went on with data its producer had not posted: the outputs of that run are not valid).
+cusync_error checkSpinTimeouts(const cusync_stage_desc* const* stages, int count, uint32_t* seen, const char* what);
 }  // namespace rt
 }  // namespace cusync
 

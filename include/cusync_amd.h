@@ -141,6 +141,9 @@ cusync_error cusync_stage_alloc(cusync_stage_desc *desc, const cusync_dim3 *host
 /* The reference never frees (no destructor); this does.  Only call on the
  * descriptor that was passed to cusync_stage_alloc, not on copies. */
 cusync_error cusync_stage_free(cusync_stage_desc *desc);
+/* Environment: CUSYNC_FORCE_ACQUIRE=1 makes every consumer wait of the prebuilt kernels end with the agent-scope
+ * acquire (which drops this XCD's cached lines), also where the launcher would skip it because the producer's
+ * tiles are whole 128-byte lines of the consumer's operand.  A switch for diagnosis; results do not change. */
 /* Same result as cusync_stage_alloc with the tile order generated from
  * desc->grid for one of the two built-in orders. */
 cusync_error cusync_stage_create(cusync_stage_desc *desc, int order);
@@ -442,6 +445,11 @@ cusync_error cusync_mlp_reload_weights(cusync_mlp *mlp);
  * [batch, 2*inner] (LLaMA).  If times_us != NULL it receives one elapsed time
  * per run, measured with events start (producer stream) -> end (consumer stream)
  * exactly as TB/mlp.cu:691-708; each run is then followed by an event wait. */
+/* Returns CUSYNC_ERROR_DEVICE (text in cusync_rt_last_error) when a wait of one of the chain's stages, the wait
+ * kernel's included, gave up after CUSYNC_SPIN_LIMIT polls during the call: the kernel went on with data that
+ * had not been posted, so the outputs of the call are not valid.  The same holds for cusync_conv_chain_run and
+ * cusync_attn_layer_run.  The launchers that do not synchronise (cusync_gemm_run, cusync_conv2d_run,
+ * cusync_attention_run) cannot know: their callers read spin_timeouts with cusync_stage_read_state. */
 cusync_error cusync_mlp_run(cusync_mlp *mlp, const void *x, void *h, void *y, int runs, double *times_us);
 /* Same, but also reports the two kernels' own durations (stream-ordered mode
  * only; TB/mlp.cu:463-488). */

@@ -114,17 +114,23 @@ def layer_weights(hidden, heads):
 
 
 def run_layer(S, hidden, heads, sync, runs=2, **kw):
+    """`runs` passes through one handle; every pass starts from intermediates full of NaN and the passes before
+    the last read another input, so that a stage that read before the post shows in what is returned."""
     import torch
     wqkv, wo, dwqkv, dwo = layer_weights(hidden, heads)
     E = heads * 128
     x = uniform_f16((S, hidden), 1)
-    dx = to_dev(x)
-    dqkv = empty_dev((S, 3 * E), fill=float("nan"))
-    do = empty_dev((S, E), fill=float("nan"))
-    dy = empty_dev((S, hidden), fill=float("nan"))
+    dx, dx_other = to_dev(x), to_dev(uniform_f16((S, hidden), 101))
+    dqkv = empty_dev((S, 3 * E))
+    do = empty_dev((S, E))
+    dy = empty_dev((S, hidden))
     torch.cuda.synchronize()
     layer = api.AttnLayer(S, hidden, heads, sync, dwqkv.data_ptr(), dwo.data_ptr(), **kw)
-    times = layer.run(dx.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=runs)
+    times = []
+    for r in range(runs):
+        dqkv.fill_(float("nan")); do.fill_(float("nan")); dy.fill_(float("nan"))
+        torch.cuda.synchronize()
+        times += layer.run((dx if r == runs - 1 else dx_other).data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=1)
     states = [layer.stage_state(i) for i in range(3)]
     tiles = layer.tiles()
     layer.destroy()
@@ -224,7 +230,11 @@ def test_attention_layer_with_cache(S, cached):
         dy = empty_dev((S, hidden), fill=float("nan"))
         torch.cuda.synchronize()
         layer = api.AttnLayer(S, hidden, heads, sync, dwqkv.data_ptr(), dwo.data_ptr(), cached_rows=cached)
-        layer.run(dx.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=2)
+        dx_other = to_dev(uniform_f16((S, hidden), 101))
+        layer.run(dx_other.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=1)
+        dqkv[cached:] = float("nan"); do.fill_(float("nan")); dy.fill_(float("nan"))       # second pass: fresh NaN, another input
+        torch.cuda.synchronize()
+        layer.run(dx.data_ptr(), dqkv.data_ptr(), do.data_ptr(), dy.data_ptr(), runs=1)
         for i in range(3):
             st = layer.stage_state(i)
             assert st.spin_timeouts == 0 and st.tile_counter == 0

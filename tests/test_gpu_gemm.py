@@ -149,16 +149,18 @@ def test_gemm_can_implement_rejects():
     prod.destroy()
 
 
-def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1), ordered=False):
+def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1), ordered=False, c_offset=0):
     """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`.  `ordered`: the wait kernel
-    goes behind an event recorded on the producer's stream right before the producer's launch."""
+    goes behind an event recorded on the producer's stream right before the producer's launch.  `c_offset`:
+    C starts that many halfs into its allocation (a base that is 16-byte but not 128-byte aligned)."""
     import torch
     L = _lib.load()
     a = uniform_f16((M, K), seed)
     b = uniform_f16((K, N), seed + 1) * np.float16(0.05)
     d = uniform_f16((N, N), seed + 2) * np.float16(0.05)
     da, db, dd = to_dev(a), to_dev(b), to_dev(d)
-    dc = empty_dev((M, N), fill=float("nan"))
+    dc_store = empty_dev((M * N + c_offset,), fill=float("nan"))
+    dc = dc_store[c_offset:].view(M, N)
     de = empty_dev((M, N), fill=float("nan"))
     torch.cuda.synchronize()
     tm, tn, _ = api.tile_shape(tile1)
@@ -181,7 +183,7 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
     ev = C.c_void_p()
     assert L.cusync_rt_event_create(C.byref(ev)) == 0
     for _ in range(iters):
-        dc.fill_(float("nan")); de.fill_(float("nan"))
+        dc_store.fill_(float("nan")); de.fill_(float("nan"))
         torch.cuda.synchronize()
         if ordered:
             assert L.cusync_rt_event_record(ev, s1) == 0
@@ -258,3 +260,55 @@ def test_chained_gemms_with_split_k(policy_kind, opts, tiles):
     assert cs.spin_timeouts == 0
     assert np.array_equal(ps.sems, want_sems)      # entries of the k-slices beyond the first stay 0
     assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.kernel_executed == 2
+
+
+@pytest.mark.parametrize("policy_kind", ["tile", "row"])
+@pytest.mark.parametrize("tiles", [(api.TILE.T128x128x32, api.TILE.T128x128x32), (api.TILE.T128x128x64, api.TILE.T64x128x64)])
+def test_chained_gemms_avoid_wait_kernel(policy_kind, tiles):
+    # AvoidWaitKernel (CS/cusync.h:193-196, 205-206; cusync_device_defs.h:78-83): no flag is allocated, the
+    # producer raises none, invokeWaitKernel launches nothing.  Valid because both launches (16 + 16 or
+    # 16 + 32 workgroups) are resident together, so the producer cannot be kept off the device.
+    print("chained, no wait kernel", policy_kind, tiles, flush=True)
+    opts = api.OPT.AVOID_WAIT_KERNEL | (api.OPT.NO_ATOMIC_ADD if policy_kind == "tile" else 0)
+    a, b, d, c, e, ps, cs, want_sems = chained(256, 1024, 1024, tiles[0], tiles[1], policy_kind, iters=3, opts=opts)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0 and ps.spin_timeouts == 0
+    assert np.array_equal(ps.sems, want_sems)
+    assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
+    assert ps.kernel_executed == 0                       # nobody raised a flag ...
+    st = api.Stage(api.gemm_grid(tiles[0], 256, 1024), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128),
+                   opts=api.OPT.AVOID_WAIT_KERNEL)
+    assert not st.desc.kernelExecuted                    # ... because there is none
+    assert st.invokeWaitKernel(None) == api.ERR.SUCCESS  # and the call is a no-op
+    st.destroy()
+
+
+@pytest.mark.parametrize("policy_kind", ["tile", "row"])
+@pytest.mark.parametrize("tiles,N,c_offset", [((api.TILE.T128x128x64, api.TILE.T128x128x64), 264, 0),     # pitch 528 bytes
+                                              ((api.TILE.T64x128x64, api.TILE.T128x128x64), 1000, 8),    # pitch 2000, base + 16
+                                              ((api.TILE.T128x128x64, api.TILE.T128x128x64), 1024, 8),   # aligned pitch, base + 16
+                                              ((api.TILE.T128x128x32, api.TILE.T128x128x32), 264, 0)])
+def test_chained_gemms_unaligned_intermediate(policy_kind, tiles, N, c_offset):
+    # A producer tile of C is not a whole number of 128-byte lines here, so a line can hold columns of a posted
+    # and of an unposted tile: every successful wait, the early poll included, has to end with the agent-scope
+    # acquire.  C is refilled with NaN before every iteration.
+    print("chained, unaligned C", policy_kind, tiles, N, c_offset, flush=True)
+    a, b, d, c, e, ps, cs, want_sems = chained(300, N, 512, tiles[0], tiles[1], policy_kind, iters=3, c_offset=c_offset)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0
+    assert np.array_equal(ps.sems, want_sems)
+
+
+def test_wait_kernel_that_gives_up_is_counted():
+    # A wait kernel on a stage whose producer never runs: the bounded spin ends by itself (about a second) and
+    # the give-up is counted where the chain handles look for it.
+    import torch
+    L = _lib.load()
+    st = api.Stage((2, 2, 1), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128))
+    assert st.read_state().spin_timeouts == 0
+    assert st.invokeWaitKernel(None) == api.ERR.SUCCESS
+    assert L.cusync_rt_device_sync() == 0, api.last_error()
+    assert st.read_state().spin_timeouts == 1
+    st.destroy()

@@ -28,15 +28,22 @@ def weights(model, hidden, inner):
 
 
 def run_mlp(model, batch, hidden, inner, sync, runs=2, activation=1, **kw):
+    """`runs` passes through one handle.  Every pass starts from intermediates and outputs full of NaN, and the
+    passes before the last one read another input: a consumer that read a tile before its post, or a line of
+    the previous pass left in a cache, would show in the outputs of the last pass, which are the ones returned."""
     import torch
     w1, w2, dw1, dw2 = weights(model, hidden, inner)
     x = uniform_f16((batch, hidden), 1)
-    dx = to_dev(x)
-    dh = empty_dev((batch, w1.shape[1]), fill=float("nan"))
-    dy = empty_dev((batch, hidden), fill=float("nan"))
+    dx, dx_other = to_dev(x), to_dev(uniform_f16((batch, hidden), 101))
+    dh = empty_dev((batch, w1.shape[1]))
+    dy = empty_dev((batch, hidden))
     torch.cuda.synchronize()
     mlp = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr(), activation=activation, **kw)
-    times = mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=runs)
+    times = []
+    for r in range(runs):
+        dh.fill_(float("nan")); dy.fill_(float("nan"))
+        torch.cuda.synchronize()
+        times += mlp.run((dx if r == runs - 1 else dx_other).data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
     prod, cons = mlp.stage_state(0), mlp.stage_state(1)
     tiles = mlp.tiles() + mlp.splits()
     mlp.destroy()
@@ -108,7 +115,7 @@ def test_gpt3_without_activation_matches_reference_check_build():
 
 @pytest.mark.parametrize("in_gemm2", [-1, 1])
 @pytest.mark.parametrize("inner", [2752, 2816])
-@pytest.mark.parametrize("batch", [1, 64, 256, 1024])
+@pytest.mark.parametrize("batch", [1, 16, 64, 256, 512, 1024, 2048])
 def test_llama_mlp(inner, batch, in_gemm2):
     # silu(gate) * up either as a stage of its own between the GEMMs or in GEMM2's A loader
     print("llama", inner, batch, in_gemm2, flush=True)
@@ -216,3 +223,28 @@ def test_mlp_repacked_weights_reload():
     assert mlp.stage_state(1).spin_timeouts == 0
     mlp.destroy()
     check_against_oracle(api.MODEL.GPT3, x, w1, w2, to_host(dh), y_first, inner)
+
+
+def test_mlp_run_reports_waits_that_gave_up():
+    # A consumer wait that runs out of polls lets its kernel go on with unposted data; the run call then
+    # returns an error instead of success.  Forced from the host: the stage's give-up counter is bumped
+    # by hand, exactly what a timed-out wait does, and no kernel is made to spin.
+    import ctypes as C
+    import torch
+    from cusync_amd import _lib
+    L = _lib.load()
+    batch = 64
+    w1, w2, dw1, dw2 = weights(api.MODEL.GPT3, **GPT3)
+    dx = to_dev(uniform_f16((batch, GPT3["hidden"]), 1))
+    dh, dy = empty_dev((batch, GPT3["inner"])), empty_dev((batch, GPT3["hidden"]))
+    torch.cuda.synchronize()
+    mlp = api.Mlp(api.MODEL.GPT3, batch, GPT3["hidden"], GPT3["inner"], api.SYNC.ROW, dw1.data_ptr(), dw2.data_ptr())
+    mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    three = C.c_uint32(3)
+    cons = L.cusync_mlp_stage(mlp.h, 1).contents
+    assert L.cusync_rt_memcpy_h2d(cons.spinTimeouts, C.addressof(three), 4) == 0
+    with pytest.raises(api.CuSyncError) as err:
+        mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
+    assert err.value.code == api.ERR.DEVICE and "3 wait(s) gave up" in str(err.value)
+    mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)       # the count did not move again: fine
+    mlp.destroy()

@@ -39,13 +39,18 @@ def assert_close(got, ref, what="", rel=REL_TOL, abs_=ABS_TOL):
         what, bad, got.size, rel, abs_, mx)
 
 
-def sample_rows(M, k=6, seed=0):
-    """A few rows including the first, the last and tile-boundary neighbours."""
+def sample_rows(M, block=128, seed=0):
+    """Rows the oracle is evaluated on: the first and the last row, one row of every block of `block` rows
+    (so that every row tile of every kernel, whose tiles are 32 to 256 rows tall, is looked at; the position
+    inside the block varies with the block) and both neighbours of every 256-row tile boundary."""
     rows = {0, M - 1, M // 2}
-    for b in (31, 32, 127, 128, 255, 256):
+    rng = np.random.default_rng(seed)
+    for b0 in range(0, M, block):
+        rows.add(int(b0 + rng.integers(0, min(block, M - b0))))
+    for b in (31, 32, 63, 64, 127, 128):
         if b < M:
             rows.add(b)
-    rng = np.random.default_rng(seed)
-    while len(rows) < min(k, M):
-        rows.add(int(rng.integers(0, M)))
-    return sorted(rows)[:max(k, 3)] if M > 3 else sorted(rows)
+    for b in range(256, M, 256):
+        rows.add(b - 1)
+        rows.add(b)
+    return sorted(rows)
