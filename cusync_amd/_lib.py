@@ -113,6 +113,7 @@ SIGNATURES = {
     "cusync_gemm_max_resident": (C.c_int, [C.c_int]),
     "cusync_gemm_chain_run": (C.c_int, [C.POINTER(GemmArgs), C.c_int, vp]),
     "cusync_gemm_run": (C.c_int, [C.POINTER(GemmArgs), vp]),
+    "cusync_gemm_run_static_workspace": (C.c_int, [C.POINTER(GemmArgs), vp]),
     "cusync_conv2d_tile_shape": (C.c_int, [C.c_int, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_conv2d_grid": (Dim3, [C.c_int, u32, u32, u32, u32, u32, u32, u32, u32]),
     "cusync_conv2d_can_implement": (C.c_int, [C.POINTER(Conv2dArgs)]),

@@ -231,6 +231,72 @@ size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {
   return partialBytes(a, ti) + (size_t)g.x * g.y * sizeof(uint32_t);
 }
 
+// ---- split-K workspace held by the library itself ------------------------------------------------------------
+// cusync_gemm_run_static_workspace takes the k-slices' partial sums and arrival counters from this array instead
+// of from memory the caller allocated.  Each device the library runs on holds its own copy until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress: the device address it yields, looked up
+// once per device, is what kernels and fills are given.
+static __device__ __align__(256) unsigned char scratch[CUSYNC_GEMM_STATIC_WORKSPACE_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_scratchPtr[kMaxDevices] = {};      // device address of `scratch` on each device, null until looked up
+std::mutex g_scratchMutex;
+
+// Device address of this device's copy of `scratch`; null (and an error text) if the runtime would not give it.
+void* scratchOfCurrentDevice() {
+  int dev = 0;
+  if (CUSYNC_HIP(hipGetDevice(&dev))) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) { cusync::rt::setError("gemm: device index beyond the table of static workspaces"); return nullptr; }
+  std::lock_guard<std::mutex> lock(g_scratchMutex);
+  if (!g_scratchPtr[dev]) {
+    void* p = nullptr;
+    if (CUSYNC_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)))) return nullptr;
+    g_scratchPtr[dev] = p;
+  }
+  return g_scratchPtr[dev];
+}
+
+// A fill kernel rather than hipMemsetAsync: memset nodes recorded into a captured graph have given wrong
+// results on replays, and this entry point is for callers that may be under capture.
+__global__ void zeroWordsKernel(uint32_t* p, uint32_t n) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+}  // namespace
+
+cusync_error cusync_gemm_run_static_workspace(const cusync_gemm_args* a, void* stream) {
+  if (!a) return CUSYNC_ERROR_NOT_INITIALIZED;
+  cusync_gemm_args mine = *a;
+  mine.workspace = nullptr;
+  if (mine.split_k > 1) {
+    TileInfo* ti = tileInfo(mine.tile);
+    if (!ti) { cusync::rt::setError("gemm: unknown tile id"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    const size_t need = cusync_gemm_workspace_size(&mine);
+    if (need > (size_t)CUSYNC_GEMM_STATIC_WORKSPACE_BYTES) {
+      cusync::rt::setError("gemm: this split-K problem needs " + std::to_string(need) + " bytes of workspace, the library's own holds " +
+                           std::to_string((size_t)CUSYNC_GEMM_STATIC_WORKSPACE_BYTES) + "; use cusync_gemm_run with a workspace of the caller's");
+      return CUSYNC_ERROR_NOT_INITIALIZED;
+    }
+    void* ws = scratchOfCurrentDevice();
+    if (!ws) return CUSYNC_ERROR_DEVICE;
+    mine.workspace = ws;
+    const cusync_error ok = cusync_gemm_can_implement(&mine);
+    if (ok != CUSYNC_SUCCESS) return ok;
+    // The arrival counters sit behind the partial sums, at an offset that depends on the problem: what the last
+    // call left there is another problem's data.  The partial sums need no clearing (every slice writes its own
+    // before anyone adds them up).
+    const cusync_dim3 g = cusync_gemm_grid(mine.tile, mine.M, mine.N, mine.split_k);
+    const uint32_t counters = g.x * g.y;
+    uint32_t* arrivals = (uint32_t*)((char*)ws + partialBytes(&mine, ti));
+    hipLaunchKernelGGL(zeroWordsKernel, dim3((counters + 255) / 256), dim3(256), 0, (hipStream_t)stream, arrivals, counters);
+    if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  }
+  return cusync_gemm_run(&mine, stream);
+}
+
 cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   cusync_error e = cusync_gemm_can_implement(a);
   if (e != CUSYNC_SUCCESS) return e;

@@ -249,6 +249,18 @@ size_t cusync_gemm_workspace_size(const cusync_gemm_args *args);
 int cusync_gemm_max_resident(int tile);
 /* run(stream) (cusyncgemm.h:525-563).  args->stage.iter selects the run. */
 cusync_error cusync_gemm_run(const cusync_gemm_args *args, void *stream);
+/* cusync_gemm_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose split-K workspace always comes
+ * from the caller (cusyncgemm.h:388-404, 407-456).  args->workspace is ignored: with split_k > 1 the k-slices'
+ * partial sums and arrival counters live in an array the library holds in device memory
+ * (CUSYNC_GEMM_STATIC_WORKSPACE_BYTES on every device it runs on, until the process ends); problems whose
+ * cusync_gemm_workspace_size exceeds that are refused with CUSYNC_ERROR_NOT_INITIALIZED and a text in
+ * cusync_rt_last_error().  The call allocates and frees nothing; it clears the arrival counters it is going to use
+ * with a small fill kernel on `stream` (no memset) and launches the same kernel as cusync_gemm_run, so results are
+ * bit-identical.  All calls on one device share the one array: two calls with split_k > 1 that overlap in time on
+ * a device (different streams, or a graph replayed while another runs) race and give wrong results. */
+#define CUSYNC_GEMM_STATIC_WORKSPACE_BYTES (32u << 20)
+cusync_error cusync_gemm_run_static_workspace(const cusync_gemm_args *args, void *stream);
 /* `count` (1..4) dependent GEMMs of one direct-to-LDS tile shape in ONE launch: every workgroup works through the
  * tiles of args[0] it can draw, then those of args[1], ...; a tile of args[i] waits on the semaphores args[i-1]
  * posts, exactly as in separate launches (the stages are created and paired the same way), but no kernel boundary,
