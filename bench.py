@@ -12,6 +12,11 @@ better); `per_batch` holds the metric proper: latency per B in {1..2048} for the
 three modes, % gain over stream-ordered, TFLOP/s and roofline fraction, measured
 with the reference's protocol (10 warm-up runs, 20 timed, slowest 10 % dropped;
 src/ml-bench/transformer/mlp.cu:954-955, eval_mlp.py:40-50).
+
+Every comparison is timed INTERLEAVED: the handles of all modes of one shape are
+alive together and take turns step by step (stream, row, tile, stream, row, ...),
+after a fixed number of untimed steps that lets the device's clock settle, so that
+clock drift, the memory-side cache and the order of the legs cannot favour a mode.
 """
 import argparse
 import json
@@ -28,9 +33,25 @@ HIDDEN, INNER = 12288, 6144
 BATCHES = [1, 16, 64, 256, 512, 1024, 2048]
 PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
-# HBM bytes one GEMM launch of the B = 2048 step moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by
-# a plain copy of known size (profiles/gemm_dma_gpt3_mlp_b2048.md).
-TRAFFIC_BYTES_PER_LAUNCH = 582e6
+SETTLE_STEPS = 40              # untimed steps of the timed shape before anything is measured: after a light load
+                               # the device needs about 30 steps of this size until its clock settles
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_by_tile.md")
+
+
+def traffic_bytes(tiles, batch):
+    """HBM bytes per GEMM launch from the committed counter runs (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
+    plain copy of known size), looked up by the tile ids of the two launches and the batch; None if that
+    combination was never profiled."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 4 and cells[0].isdigit() and cells[1].isdigit() and cells[2].isdigit():
+                    if (int(cells[0]), int(cells[1]), int(cells[2])) == (tiles[0], tiles[1], batch):
+                        return float(cells[3]) * 1e6
+    except OSError:
+        pass
+    return None
 
 
 def trimmed(times):
@@ -80,17 +101,17 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=50,
-                    help="untimed steps before the timed ones; after a light load the device needs about 30 steps of\n"
-                         "this size before its clock settles")
+    ap.add_argument("--warmup", type=int, default=10,
+                    help="untimed rounds before the timed ones, on top of a fixed settling preamble")
     ap.add_argument("--batch", type=int, default=2048, help="B of the timed step")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-batch table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the leg that times the dominant kernel (stream-ordered GEMM1/GEMM2 at --batch) "
                          "plus a plain copy of known size; used under rocprofv3 so its per-kernel averages match")
-    ap.add_argument("--profile-chain", choices=["attention", "conv"], default=None,
-                    help="run only the stream-ordered attention chain (S = 2048) or convolution pairs, for rocprofv3")
+    ap.add_argument("--profile-chain", choices=["attention", "conv", "mlp"], default=None,
+                    help="run only the stream-ordered attention chain (S = 2048) or convolution pairs, or (mlp) --steps rounds of "
+                         "the GPT-3 MLP at --batch stream-ordered / RowSync / TileSync in turn, for rocprofv3")
     ap.add_argument("--tile1", type=int, default=-1)
     ap.add_argument("--tile2", type=int, default=-1)
     args = ap.parse_args()
@@ -115,29 +136,52 @@ def main():
     w1, w2, x_all = (torch.from_numpy(a).cuda() for a in (w1_host, w2_host, x_host))
     torch.cuda.synchronize()
 
-    def make(batch, sync, one_launch=False, repack=False):
-        h = torch.empty((batch, INNER), dtype=torch.float16, device="cuda")
-        y = torch.empty((batch, HIDDEN), dtype=torch.float16, device="cuda")
-        torch.cuda.synchronize()
-        m = api.Mlp(api.MODEL.GPT3, batch, HIDDEN, INNER, sync, w1.data_ptr(), w2.data_ptr(),
-                    tile1=args.tile1, tile2=args.tile2, one_launch=one_launch, repack_weights=repack)
-        return m, h, y
+    class Chain:
+        """One MLP handle with its intermediate and output buffers."""
 
-    def protocol(batch, sync, warm=10, timed=20, split=False, one_launch=False, repack=False):
-        m, h, y = make(batch, sync, one_launch, repack)
-        x = x_all[:batch]
-        m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=warm)
-        out = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=timed, split=split)
-        timeouts = m.stage_state(1).spin_timeouts
-        tiles = m.tiles()
-        m.destroy()
-        if timeouts:
-            sys.exit("bench.py: %d consumer waits timed out — results invalid" % timeouts)
-        return out, tiles
+        def __init__(self, batch, sync, one_launch=False, repack=False):
+            self.h = torch.empty((batch, INNER), dtype=torch.float16, device="cuda")
+            self.y = torch.empty((batch, HIDDEN), dtype=torch.float16, device="cuda")
+            self.x = x_all[:batch]
+            torch.cuda.synchronize()
+            self.m = api.Mlp(api.MODEL.GPT3, batch, HIDDEN, INNER, sync, w1.data_ptr(), w2.data_ptr(),
+                             tile1=args.tile1, tile2=args.tile2, one_launch=one_launch, repack_weights=repack)
+            self.tiles = self.m.tiles()
+
+        def step(self, split=False):
+            """One pass; elapsed microseconds by HIP events on the chain's own streams (a wait that gave up raises)."""
+            out = self.m.run(self.x.data_ptr(), self.h.data_ptr(), self.y.data_ptr(), runs=1, split=split)
+            return (out[0][0], out[1][0], out[2][0]) if split else out[0]
+
+        def close(self):
+            self.m.destroy()
+
+    def interleaved(chains, warm, timed, split_first=False):
+        """Runs the chains in turn, one step each per round: `warm` untimed rounds, then `timed` rounds.  Returns
+        one list of step times per chain (for the first chain, with split_first, triples: step, GEMM1, GEMM2)."""
+        for _ in range(warm):
+            for c in chains:
+                c.step()
+        times = [[] for _ in chains]
+        for _ in range(timed):
+            for i, c in enumerate(chains):
+                times[i].append(c.step(split=split_first and i == 0))
+        return times
+
+    def settle(batch, steps=SETTLE_STEPS):
+        """Untimed steps of the timed shape: brings the clock to where it stays under this load."""
+        c = Chain(batch, api.SYNC.STREAM)
+        for _ in range(steps):
+            c.step()
+        c.close()
 
     def roofline_leg(B, warm, timed):
         """Durations of the two GEMM launches, HIP events on the stream they run on."""
-        (t_s, g1, g2), tiles = protocol(B, api.SYNC.STREAM, warm=warm, timed=timed, split=True)
+        c = Chain(B, api.SYNC.STREAM)
+        (t3,) = interleaved([c], warm, timed, split_first=True)
+        tiles = c.tiles
+        c.close()
+        t_s, g1, g2 = [v[0] for v in t3], [v[1] for v in t3], [v[2] for v in t3]
         k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
         flops_per_launch = 2.0 * B * HIDDEN * INNER
         achieved = flops_per_launch / (k_us * 1e-6) / 1e12
@@ -156,12 +200,24 @@ def main():
                 if hbm_bound else
                 {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                  "frac": round(achieved / PEAK_FP16_TFLOPS, 4)})
-        return {**head, "traffic": None,
+        return {**head, "traffic": traffic_bytes(tiles, B),
                 "kernel": "gemmDmaKernel, mean of the two launches of the step: GEMM1 tile %s %.1f us, GEMM2 tile %s %.1f us "
                           "(stream-ordered, %.1f GFLOP per launch)" % (shapes[0], statistics.fmean(g1), shapes[1], statistics.fmean(g2),
                                                                        flops_per_launch / 1e9),
                 }, statistics.fmean(t_s), tiles
 
+    if args.profile_chain == "mlp":
+        # every round enqueues six GEMM launches in this order: stream-ordered GEMM1, GEMM2; RowSync producer, consumer;
+        # TileSync producer, consumer.  A kernel trace of this run shows when each started and ended.
+        settle(args.batch)
+        chains = [Chain(args.batch, api.SYNC.STREAM), Chain(args.batch, api.SYNC.ROW), Chain(args.batch, api.SYNC.TILE)]
+        times = interleaved(chains, args.warmup, args.steps)
+        for c in chains:
+            c.close()
+        print(json.dumps({"metric": "GPT-3 MLP rounds of stream / rowsync / tilesync", "batch": args.batch, "warmup_rounds": args.warmup,
+                          "rounds": args.steps, "settle_steps": SETTLE_STEPS,
+                          "event_us": {n: round(statistics.fmean(t), 2) for n, t in zip(("stream", "rowsync", "tilesync"), times)}}))
+        return
     if args.profile_chain == "attention":
         heads, e, seq = 12, 12 * 128, 2048
         g = torch.Generator(device="cuda").manual_seed(4)
@@ -206,31 +262,47 @@ def main():
 
     per_batch = []
     if not args.no_sweep:
+        settle(max(BATCHES))
         for b in BATCHES:
-            (t_s, g1, g2), tiles = protocol(b, api.SYNC.STREAM, split=True)
-            t_r, _ = protocol(b, api.SYNC.ROW)
-            t_t, _ = protocol(b, api.SYNC.TILE)
-            # RowSync with both GEMMs in one launch (same stages and semaphores, no wait kernel, no second launch)
-            one = trimmed(protocol(b, api.SYNC.ROW, one_launch=True)[0])[0] if tiles[0] == tiles[1] else None
-            # the same chain reading copies of the weights whose rows are 256 bytes longer (cusync_mlp_config.
-            # repack_weights): a column tile's k rows then spread over all memory channels instead of one class
-            s_rp = trimmed(protocol(b, api.SYNC.STREAM, repack=True)[0])[0]
-            r_rp = trimmed(protocol(b, api.SYNC.ROW, repack=True)[0])[0]
-            one_rp = trimmed(protocol(b, api.SYNC.ROW, one_launch=True, repack=True)[0])[0] if tiles[0] == tiles[1] else None
-            s, s_sd = trimmed(t_s)
-            r, r_sd = trimmed(t_r)
-            t, t_sd = trimmed(t_t)
-            best = min(r, t) if one is None else min(r, t, one)
+            # all modes of this batch size alive together, one step each per round (10 untimed rounds, 20 timed):
+            # stream-ordered, RowSync, TileSync, RowSync with both GEMMs in one launch (same stages and semaphores,
+            # no wait, no second launch), and the same with copies of the weights whose rows are 256 bytes longer
+            # (cusync_mlp_config.repack_weights: a column tile's k rows then spread over all memory channels)
+            names = ["stream", "rowsync", "tilesync"]
+            chains = [Chain(b, api.SYNC.STREAM), Chain(b, api.SYNC.ROW), Chain(b, api.SYNC.TILE)]
+            tiles = chains[0].tiles
+            if tiles[0] == tiles[1]:
+                names.append("rowsync_one_launch")
+                chains.append(Chain(b, api.SYNC.ROW, one_launch=True))
+            names += ["stream_rp", "rowsync_rp"]
+            chains += [Chain(b, api.SYNC.STREAM, repack=True), Chain(b, api.SYNC.ROW, repack=True)]
+            if tiles[0] == tiles[1]:
+                names.append("rowsync_one_launch_rp")
+                chains.append(Chain(b, api.SYNC.ROW, one_launch=True, repack=True))
+            times = interleaved(chains, 10, 20, split_first=True)
+            for c in chains:
+                c.close()
+            t = dict(zip(names, times))
+            g1, g2 = [v[1] for v in t["stream"]], [v[2] for v in t["stream"]]
+            t["stream"] = [v[0] for v in t["stream"]]
+            m = {k: trimmed(v) for k, v in t.items()}
+            s_us = m["stream"][0]
+            in_place = [k for k in ("rowsync", "tilesync", "rowsync_one_launch") if k in m]
+            best = min(m[k][0] for k in in_place)
+            rp = [m[k][0] for k in ("stream_rp", "rowsync_rp", "rowsync_one_launch_rp") if k in m]
             per_batch.append({
                 "B": b, "tiles": list(tiles),
-                "stream_us": round(s, 2), "stream_std": round(s_sd, 2),
+                "stream_us": round(s_us, 2), "stream_std": round(m["stream"][1], 2),
                 "gemm1_us": round(trimmed(g1)[0], 2), "gemm2_us": round(trimmed(g2)[0], 2),
-                "rowsync_us": round(r, 2), "rowsync_std": round(r_sd, 2), "rowsync_gain_pct": round(100 - r / s * 100, 2),
-                "tilesync_us": round(t, 2), "tilesync_std": round(t_sd, 2), "tilesync_gain_pct": round(100 - t / s * 100, 2),
-                "rowsync_one_launch_us": None if one is None else round(one, 2),
-                "repacked_weights": {"stream_us": round(s_rp, 2), "rowsync_us": round(r_rp, 2),
-                                     "rowsync_one_launch_us": None if one_rp is None else round(one_rp, 2),
-                                     "roofline_frac": round(ideal_us(b) / min(v for v in (s_rp, r_rp, one_rp) if v), 4)},
+                "rowsync_us": round(m["rowsync"][0], 2), "rowsync_std": round(m["rowsync"][1], 2),
+                "rowsync_gain_pct": round(100 - m["rowsync"][0] / s_us * 100, 2),
+                "tilesync_us": round(m["tilesync"][0], 2), "tilesync_std": round(m["tilesync"][1], 2),
+                "tilesync_gain_pct": round(100 - m["tilesync"][0] / s_us * 100, 2),
+                "rowsync_one_launch_us": round(m["rowsync_one_launch"][0], 2) if "rowsync_one_launch" in m else None,
+                "best_gain_pct": round(100 - best / s_us * 100, 2),
+                "repacked_weights": {"stream_us": round(m["stream_rp"][0], 2), "rowsync_us": round(m["rowsync_rp"][0], 2),
+                                     "rowsync_one_launch_us": round(m["rowsync_one_launch_rp"][0], 2) if "rowsync_one_launch_rp" in m else None,
+                                     "roofline_frac": round(ideal_us(b) / min(rp), 4)},
                 "best_tflops": round(mlp_flops(b) / best / 1e6, 1),
                 "bound": "mfma" if mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12) > mlp_bytes(b) / (PEAK_HBM_GBS * 1e9) else "hbm",
                 "roofline_frac": round(ideal_us(b) / best, 4),
@@ -326,31 +398,39 @@ def main():
             "handover_ns_other_xcd": round(api.sync_overhead_pingpong(1) / 2, 1),
         }
 
-    # ---- the timed step: B = args.batch under the better CuSync policy ----------
-    syncs = {"rowsync": api.SYNC.ROW, "tilesync": api.SYNC.TILE}
-    measured = [r for r in per_batch if r["B"] == B]
-    if measured:        # the sweep above already timed both policies at this batch with the full protocol
-        policy = min(syncs, key=lambda k: measured[0][k + "_us"])
-    else:
-        cand = {name: trimmed(protocol(B, sync, warm=10, timed=30)[0])[0] for name, sync in syncs.items()}
-        policy = min(cand, key=cand.get)
-    m, h, y = make(B, syncs[policy])
-    x = x_all[:B]
-    m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=args.warmup)
+    # ---- the timed step: B = args.batch, CuSync against stream-ordered, interleaved ----------
+    # Both policies and the stream-ordered pair are alive together and take turns, one step each per round: the
+    # settling preamble (fixed, whatever --warmup says), then --warmup untimed rounds, then --steps timed rounds.
+    # `value` is the better policy's mean; the gain is computed from steps that ran next to each other.
+    settle(B)
+    names = ["stream", "rowsync", "tilesync"]
+    chains = [Chain(B, api.SYNC.STREAM), Chain(B, api.SYNC.ROW), Chain(B, api.SYNC.TILE)]
+    tiles = chains[1].tiles
+    for _ in range(args.warmup):
+        for c in chains:
+            c.step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    step_times = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=args.steps)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    if m.stage_state(1).spin_timeouts:
-        sys.exit("bench.py: consumer waits timed out — results invalid")
-    tiles = m.tiles()
-    m.destroy()
-    ms_per_step = wall / args.steps * 1e3
+    step_times = {n: [] for n in names}
+    wall = {n: 0.0 for n in names}
+    for _ in range(args.steps):
+        for n, c in zip(names, chains):
+            t0 = time.perf_counter()
+            step_times[n].append(c.step())        # returns after the step's last kernel has finished
+            wall[n] += time.perf_counter() - t0
+    for c in chains:
+        c.close()
+    policy = min(("rowsync", "tilesync"), key=lambda k: statistics.fmean(step_times[k]))
+    ms_per_step = wall[policy] / args.steps * 1e3
 
-    # stream-ordered on the same shape: baseline latency and the kernels' own durations
-    roof, stream_us, _ = roofline_leg(B, args.warmup, max(10, args.steps))
-    roof["traffic"] = TRAFFIC_BYTES_PER_LAUNCH if B == 2048 else None      # counters were taken at the default batch
+    def spread(v):
+        return {"mean": round(statistics.fmean(v), 2), "median": round(statistics.median(v), 2),
+                "min": round(min(v), 2), "max": round(max(v), 2)}
+
+    stream_mean = statistics.fmean(step_times["stream"])
+    value = statistics.fmean(step_times[policy])
+
+    # the kernels' own durations (stream-ordered, HIP events on the launching stream) for the roofline
+    roof, _, _ = roofline_leg(B, 5, max(10, args.steps))
     # what the matrix pipes alone sustain on this machine (register operands, no LDS, no memory): the clock
     # drops under a device-wide MFMA load, further with random operands than with zeros
     zero_tf, zero_mhz = api.probe_mfma_rate(False)
@@ -362,7 +442,7 @@ def main():
 
     out = {
         "metric": "GPT-3 MLP shard latency (us) + % gain vs kernel-boundary sync, B=1..2048",
-        "value": round(statistics.fmean(step_times), 2),
+        "value": round(value, 2),
         "unit": "us",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
@@ -370,12 +450,14 @@ def main():
         "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "GPT-3 175B MLP 1/8 shard, B=%d: X[B,12288] x W1[12288,6144] +GeLU -> x W2[6144,12288]" % B,
                    "policy": policy, "tiles": list(tiles), "device": dev["arch"], "cus": dev["cus"]},
-        # the same two GEMMs stream-ordered, same warm-up and step count, plain mean like `value`
-        "stream_ordered_us": round(stream_us, 2),
-        "gain_pct": round(100 - statistics.fmean(step_times) / stream_us * 100, 2),
-        "step_us": {"median": round(statistics.median(step_times), 2), "min": round(min(step_times), 2),
-                    "max": round(max(step_times), 2)},
-        "tflops": round(mlp_flops(B) / statistics.fmean(step_times) / 1e6, 1),
+        # the same two GEMMs stream-ordered, timed in the same rounds as `value` (one step of each per round)
+        "stream_ordered_us": round(stream_mean, 2),
+        "gain_pct": round(100 - value / stream_mean * 100, 2),
+        "gain_pct_median": round(100 - statistics.median(step_times[policy]) / statistics.median(step_times["stream"]) * 100, 2),
+        "step_us": spread(step_times[policy]),
+        "stream_step_us": spread(step_times["stream"]),
+        "other_policy_step_us": {k: spread(v) for k, v in step_times.items() if k not in ("stream", policy)},
+        "tflops": round(mlp_flops(B) / value / 1e6, 1),
         "roofline": roof,
         "per_batch": per_batch,
         "other_chains": other,

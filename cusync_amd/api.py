@@ -16,7 +16,7 @@ ERR = SimpleNamespace(NOT_PRODUCER=0, NOT_CONSUMER=1, NOT_INITIALIZED=2,
 OPT = SimpleNamespace(NONE=0, NO_ATOMIC_ADD=1, AVOID_WAIT_KERNEL=2, AVOID_CUSTOM_ORDER=4, REORDER_TILE_LOADS=8)
 ORDER = SimpleNamespace(IDENTITY=0, TRANSPOSE_XY=1)
 POLICY = SimpleNamespace(NOSYNC=0, ROWSYNC=1, TILESYNC=2, STRIDEDSYNC=3, CONV2DTILESYNC=4, CONSECUTIVESYNC=5)
-EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2)
+EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2, SWIGLU=3)
 TILE = SimpleNamespace(T256x256x32=0, T256x128x64=1, T128x128x64=2, T64x128x64=3, T32x128x64=4,
                        T128x256x64=5, T256x64x64=6, T128x64x64=7, T256x128x32=8, T128x256x32=9, T128x128x32=10,
                        T128x192x32=11, T256x192x32=12, D32x128x64=13, D64x128x64=14, D64x192x64=15, T128x192x32_ALONE=16, COUNT=17)

@@ -39,11 +39,29 @@ struct GemmParams {
   float* partials;         // [splitK][m-tiles][n-tiles][BM*BN] fp32 partial sums in register order
   uint32_t* arrivals;      // [m-tiles * n-tiles] slices finished per output tile; 0 between launches
   uint32_t mPad;           // m-tiles * BM
+  // Consumer whose producer's tiles are not whole 128-byte lines of A (a tile policy with a tile width that is
+  // not a multiple of 64 halfs): 64, and every wait of a K chunk then covers all producer column tiles that
+  // reach into the lines the chunk touches, not only the columns it reads.  A line is then never fetched
+  // before everything in it has been posted, so no stale line can sit in this XCD's caches and the waits can
+  // do without the cache invalidation (DynStage::lineAligned).  1 otherwise.
+  uint32_t waitRound;
   // implicit-GEMM convolution (A is gathered from an NHWC tensor): M = n*P*Q, K = R*S*C, k = (r*S + s)*C + c
   uint32_t cvN, cvH, cvW, cvC, cvP, cvQ, cvR, cvS, cvPad, cvStride;
 };
 
 enum { kAPlain = 0, kAConv = 1 };
+
+// First output column of the tile whose first column of the product is n0: the SwiGLU epilogue folds pairs of
+// column groups, so its tiles are half as wide in the output, and that is what a consumer's policy sees.
+__device__ __forceinline__ uint32_t outputColumn(const GemmParams& p, uint32_t n0) {
+  return p.epilogue == CUSYNC_EPILOGUE_SWIGLU ? n0 / 2 : n0;
+}
+// Posts of the output policy one finished tile stands for.  StridedSync folds the tile of the gate columns and
+// the tile of the up columns of one column range onto one semaphore that counts to two
+// (src/ml-bench/transformer/mlp.cu:76-101); a tile of the SwiGLU epilogue holds both and posts for both.
+__device__ __forceinline__ uint32_t postsPerTile(const GemmParams& p) {
+  return p.epilogue == CUSYNC_EPILOGUE_SWIGLU && p.stage.d.out.kind == CUSYNC_POLICY_STRIDEDSYNC ? p.stage.d.out.stride : 1;
+}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
@@ -136,13 +154,50 @@ template<class C>
 __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
                                            const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
   const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
+  const bool through = p.stage.isProducer();
+  const __amdgpu_buffer_rsrc_t rD = makeRsrc(p.D, p.M * p.ldd * 2);
   // Final values go through LDS so that global memory sees whole rows: a lane holds 4 consecutive columns of
   // 32 different rows, which stored directly would be 8-byte pieces scattered over 32 cache lines per
   // instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
   // applied) into a [WM*32][BN] buffer (rows padded by 16 bytes against bank conflicts), then all threads
   // copy the buffer out, 16 bytes per lane, consecutive lanes along a row.
   // storePass(i, value): MFMA row tile i of every wave, value(j, g) its four floats of tile j, group g.
+  // CUSYNC_EPILOGUE_SWIGLU: the tile's columns are gate and up columns in alternating groups of eight, and in the
+  // MFMA result layout group g of a lane is columns 8g + 4*(lane/32) + 0..3 of its 32-column tile: groups 0 and 2
+  // are gate values, groups 1 and 3 the up values of the same output columns.  The tile's output is BN/2 wide.
+  auto storePassPairs = [&](int i, auto&& value) {
+    constexpr int PITCH = C::BN + 16;                 // BN/2 halfs and the pad
+    constexpr int ROWS = C::WM * 32;
+    constexpr int CPR = C::BN / 16;
+    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
+    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
+    constexpr int STEPS = ROWS * CPR / C::THREADS;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int gp = 0; gp < 2; gp++) {
+        const floatx4 vg = value(j, 2 * gp), vu = value(j, 2 * gp + 1);
+        half4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (half_t)(siluf(vg[e]) * vu[e]);
+        *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * (C::WTN / 2) + j * 16 + 8 * gp + 4 * (lane >> 5)) * 2) = o;
+      }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+      const uint32_t idx = s * C::THREADS + threadIdx.x;
+      const uint32_t lr = idx / CPR, c = idx % CPR;
+      const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 / 2 + c * 8;
+      if (m < p.M && n < p.N / 2) {
+        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
+        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
+      }
+    }
+  };
   auto storePass = [&](int i, auto&& value) {
+    if (p.epilogue == CUSYNC_EPILOGUE_SWIGLU) { storePassPairs(i, value); return; }
     constexpr int PITCH = C::BN * 2 + 16;
     constexpr int ROWS = C::WM * 32;
     constexpr int CPR = C::BN / 8;
@@ -167,8 +222,15 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
         const uint32_t idx = s * C::THREADS + threadIdx.x;
         const uint32_t lr = idx / CPR, c = idx % CPR;
         const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
-        if (m < p.M && n < p.N)
-          *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+        if (m < p.M && n < p.N) {
+          const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+          // A producer's output is written through to memory (device scope) as it is stored: the release of the
+          // post then finds no dirty lines of it in this XCD's L2.  Left to the post, every one of the workgroups
+          // of an XCD that finish together starts a write-back of the whole L2 (measured: the producer of the
+          // 2048-row MLP runs 5 us longer than the same kernel without a post).
+          if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
+          else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
+        }
       }
     }
   };

@@ -31,8 +31,7 @@
 #include "rt_internal.h"
 #include "stage_device.h"
 
-#include "gemm_kernel_staged.h"
-#include "gemm_kernel_dma.h"
+#include "gemm_tiles.h"
 
 namespace {
 
@@ -42,51 +41,22 @@ using namespace cusync::gemm;
 // Host side
 // ---------------------------------------------------------------------------
 
-struct TileInfo {
-  uint32_t bm, bn, bk;
-  uint32_t threads;
-  size_t lds;
-  void (*kernel[2])(GemmParams);   // [plain A, SwiGLU A]
-  int residentPerCU;     // filled lazily
-  void (*chainKernel)(GemmChainParams);   // several dependent GEMMs in one launch; direct-to-LDS tiles only
-};
-
-#define CUSYNC_TILE(BM, BN, BK, WM, WN) \
-  { BM, BN, BK, kThreads, (size_t)TileCfg<BM, BN, BK, WM, WN>::LDS_BYTES, \
-    { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1, nullptr }
-
-// Direct-to-LDS tiles have no SwiGLU variant (that operand needs arithmetic on its way into LDS).
-#define CUSYNC_TILE_DMA(...) \
-  { DmaCfg<__VA_ARGS__>::BM, DmaCfg<__VA_ARGS__>::BN, DmaCfg<__VA_ARGS__>::BK, DmaCfg<__VA_ARGS__>::THREADS, \
-    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1, gemmDmaChainKernel<DmaCfg<__VA_ARGS__>> }
-
-TileInfo g_tiles[CUSYNC_TILE_COUNT] = {
-  // eight wavefronts of 128x64: an A fragment costs one LDS read, a B fragment two transposing ones, so the tall
-  // wavefront tile is the cheaper one (measured against 64x128: 641 -> 630 us per B=2048 step)
-  CUSYNC_TILE_DMA(256, 256, 32, 2, 4, 4, 2, false, true),   // CUSYNC_TILE_256x256x32: direct-to-LDS, 4 stages, one workgroup per CU
-  CUSYNC_TILE(256, 128, 64, 2, 2),   // CUSYNC_TILE_256x128x64
-  CUSYNC_TILE(128, 128, 64, 2, 2),   // CUSYNC_TILE_128x128x64
-  CUSYNC_TILE(64, 128, 64, 1, 4),    // CUSYNC_TILE_64x128x64
-  CUSYNC_TILE(32, 128, 64, 1, 4),    // CUSYNC_TILE_32x128x64
-  CUSYNC_TILE(128, 256, 64, 2, 2),   // CUSYNC_TILE_128x256x64
-  CUSYNC_TILE(256, 64, 64, 4, 1),    // CUSYNC_TILE_256x64x64
-  CUSYNC_TILE(128, 64, 64, 2, 2),    // CUSYNC_TILE_128x64x64
-  CUSYNC_TILE_DMA(256, 128, 32, 2, 2, 3, 2),   // CUSYNC_TILE_256x128x32: direct-to-LDS, 3 stages, two workgroups per CU
-  CUSYNC_TILE_DMA(128, 256, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x256x32
-  CUSYNC_TILE_DMA(128, 128, 32, 2, 2, 3, 3),   // CUSYNC_TILE_128x128x32: three workgroups per CU
-  CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 3, 2),   // CUSYNC_TILE_128x192x32: 6144 and 12288 columns are 32 and 64 tiles
-  CUSYNC_TILE_DMA(256, 192, 32, 4, 2, 4, 2, false, true),   // CUSYNC_TILE_256x192x32: eight wavefronts of 64x96
-  CUSYNC_TILE_DMA(32, 128, 64, 1, 4, 4, 2),     // CUSYNC_TILE_D32x128x64: 60 KB of loads in flight per workgroup
-  CUSYNC_TILE_DMA(64, 128, 64, 1, 4, 3, 2),     // CUSYNC_TILE_D64x128x64
-  CUSYNC_TILE_DMA(64, 192, 64, 2, 2, 4, 1),     // CUSYNC_TILE_D64x192x64: 96 KB of loads in flight per CU
-  CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 4, 2, false, true),   // CUSYNC_TILE_128x192x32_ALONE: 80 KB of LDS, so one workgroup per CU
-};
+TileInfo g_tiles[CUSYNC_TILE_COUNT];
+std::once_flag g_tilesOnce;
 
 std::mutex g_mutex;
 int g_numCUs = 0;
 
+// The kernels are instantiated in several translation units (they take minutes to compile); each fills in
+// the entries of the tiles it holds.
 TileInfo* tileInfo(int tile) {
   if (tile < 0 || tile >= CUSYNC_TILE_COUNT) return nullptr;
+  std::call_once(g_tilesOnce, [] {
+    fillStagedTiles(g_tiles);
+    fillDmaTilesWide(g_tiles);
+    fillDmaTilesMid(g_tiles);
+    fillDmaTilesFew(g_tiles);
+  });
   return &g_tiles[tile];
 }
 
@@ -156,8 +126,10 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   if (a->K % 8 || a->N % 8) { setError("gemm: K and N must be multiples of 8 (16-byte loads)"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->lda % 8 || a->ldb % 8 || a->ldd % 8) { setError("gemm: leading dimensions must keep 16-byte alignment"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const uint32_t aCols = a->a_mode == CUSYNC_A_SWIGLU ? 2 * a->K : a->K;
-  if (a->lda < aCols || a->ldb < a->N || a->ldd < a->N) { setError("gemm: leading dimension smaller than the row"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if ((uint64_t)a->M * a->lda * 2 >= 0x80000000ull || (uint64_t)a->K * a->ldb * 2 >= 0x80000000ull) {
+  const uint32_t dCols = a->epilogue == CUSYNC_EPILOGUE_SWIGLU ? a->N / 2 : a->N;
+  if (a->lda < aCols || a->ldb < a->N || a->ldd < dCols) { setError("gemm: leading dimension smaller than the row"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if ((uint64_t)a->M * a->lda * 2 >= 0x80000000ull || (uint64_t)a->K * a->ldb * 2 >= 0x80000000ull ||
+      (uint64_t)a->M * a->ldd * 2 >= 0x80000000ull) {
     setError("gemm: operand larger than 2 GiB is not addressable by one buffer descriptor");
     return CUSYNC_ERROR_NOT_INITIALIZED;
   }
@@ -170,7 +142,8 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
     if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   }
   if (a->a_mode != CUSYNC_A_PLAIN && a->a_mode != CUSYNC_A_SWIGLU) { setError("gemm: unknown a_mode"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_RELU) { setError("gemm: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_SWIGLU) { setError("gemm: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (a->epilogue == CUSYNC_EPILOGUE_SWIGLU && a->N % 16) { setError("gemm: the SwiGLU epilogue pairs groups of eight columns: N must be a multiple of 16"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
   const cusync_stage_desc& s = a->stage;
   if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) {
@@ -203,11 +176,16 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   const cusync_stage_desc& s = a->stage;
   GemmParams p;
   p.stage.d = s;
-  // Producer tiles are whole 128-byte lines of A when the row pitch, the base and
-  // the producer's tile width all are multiples of 128 bytes (64 halfs).
-  p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 && (a->lda * 2) % 128 == 0 &&
-                        (s.in.kind == CUSYNC_POLICY_ROWSYNC || s.in.kind == CUSYNC_POLICY_CONSECUTIVESYNC ||
-                         (s.in.tileN * 2) % 128 == 0);       // the row policies guard whole rows
+  // Producer tiles are whole 128-byte lines of A when the row pitch, the base and the producer's tile width all
+  // are multiples of 128 bytes (64 halfs); the row policies guard whole rows.  With a tile width that is not,
+  // the direct-to-LDS kernels make every wait cover whole lines instead (GemmParams::waitRound), which serves
+  // the same end: no line of A is fetched before everything in it has been posted.
+  const bool rowPolicy = s.in.kind == CUSYNC_POLICY_ROWSYNC || s.in.kind == CUSYNC_POLICY_CONSECUTIVESYNC;
+  const bool wholeLineTiles = rowPolicy || (s.in.tileN * 2) % 128 == 0;
+  const bool canRound = ti->chainKernel != nullptr && a->a_mode == CUSYNC_A_PLAIN;      // a direct-to-LDS tile
+  p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 &&
+                        (a->lda * 2) % 128 == 0 && (wholeLineTiles || canRound);
+  p.waitRound = p.stage.lineAligned && !wholeLineTiles ? 64 : 1;
   p.M = a->M; p.N = a->N; p.K = a->K;
   p.A = (const half_t*)a->A; p.lda = a->lda;
   p.B = (const half_t*)a->B; p.ldb = a->ldb;

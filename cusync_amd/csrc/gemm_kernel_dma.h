@@ -32,7 +32,7 @@
 // (kt, k-step 1); the loads of chunk kt+STAGES-1 go into the stage of chunk kt-1.
 #pragma once
 
-#include "gemm_common.h"
+#include "gemm_tiles.h"
 
 namespace cusync {
 namespace gemm {
@@ -217,7 +217,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     }
 
     // ---- consumer side (same protocol as the staged kernel) ------------------
-    uint32_t nextColTile = kBegin / tnq;
+    uint32_t nextColTile = (kBegin & ~(p.waitRound - 1)) / tnq;     // the first chunk's line may begin in the tile before
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
     uint32_t readyEnd = 0;        // column tiles of the producer below this one are known to be posted (one row block)
     auto waitRows = [&](uint32_t col, uint32_t z) { stage.waitWaveRows(m0, mEnd - 1, tmq, col, z); };
@@ -251,10 +251,12 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
         cvWaitRows(stage.d.in.kind == CUSYNC_POLICY_CONV2DTILESYNC ? ct * p.cvR * p.cvS * tnq : ct * tnq, 0);
         return;
       }
-      const uint32_t kLast = min(k0 + (uint32_t)C::BK, kEnd) - 1;
+      // last column whose producer tile must be there: the chunk's last column, or (waitRound) the last column
+      // of the 128-byte line it lies in
+      const uint32_t kLast = min((min(k0 + (uint32_t)C::BK, kEnd) - 1) | (p.waitRound - 1), p.K - 1);
       for (; nextColTile <= kLast / tnq; nextColTile++) {
         if (nextColTile < readyEnd) continue;            // seen posted by an earlier look-ahead
-        if (oneRowBlock) readyEnd = nextColTile + stage.waitWaveAhead(m0, nextColTile * tnq, tnq, (kEnd - 1) / tnq - nextColTile + 1);
+        if (oneRowBlock) readyEnd = nextColTile + stage.waitWaveAhead(m0, nextColTile * tnq, tnq, max(kEnd - 1, kLast) / tnq - nextColTile + 1);
         else waitRows(nextColTile * tnq, 0);
       }
     };
@@ -464,8 +466,8 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
 
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
-    cusync_dim3 done = {m0, n0, t.z};
-    if (completed && stage.isProducer()) stage.post(done);
+    cusync_dim3 done = {m0, outputColumn(p, n0), t.z};
+    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p));
     else __syncthreads();
   }
 }
@@ -482,12 +484,6 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
 // (few rows: 30 us in the kernel, 10 us around it) pays most for.  Forward progress: the launch has
 // no more workgroups than stay resident, and a workgroup only moves on when the GEMM it is on has no
 // tile left to hand out, so every tile a consumer tile waits for is in the hands of a running workgroup.
-constexpr int kMaxChainedGemms = 4;
-struct GemmChainParams {
-  GemmParams gemm[kMaxChainedGemms];
-  uint32_t count;
-};
-
 template<class C>
 __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaChainKernel(GemmChainParams cp) {
   for (uint32_t g = 0; g < cp.count; g++) {

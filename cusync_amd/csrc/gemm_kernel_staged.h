@@ -268,9 +268,9 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
 
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
-    cusync_dim3 done = {m0, n0, t.z};
+    cusync_dim3 done = {m0, outputColumn(p, n0), t.z};
     // the post's barrier (or this one) keeps the next tile's LDS writes behind the epilogue's LDS reads
-    if (completed && stage.isProducer()) stage.post(done);
+    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p));
     else __syncthreads();
   }
 }

@@ -32,6 +32,9 @@ struct cusync_mlp {
   cusync_stage_desc prod, cons;
   hipStream_t sProd, sCons;
   hipEvent_t eStart, eMid, eEnd;
+  // LLaMA with silu(gate) * up as GEMM1's epilogue: w1p holds W1 with the gate and up columns interleaved in
+  // groups of eight, the intermediate is [batch][inner]
+  bool fused;
   // LLaMA with the activation as a stage of its own between the GEMMs: silu(gate) * up, once per element
   bool actStage;
   void* act;                         // [batch][inner] fp16, GEMM2's A operand
@@ -59,6 +62,15 @@ constexpr uint32_t kActM = 128, kActN = 128, kActThreads = 256;
 __global__ __launch_bounds__(256) void repackRowsKernel(const uint4v* src, uint4v* dst, uint32_t vecs, uint32_t dstPitch) {
   const uint32_t c = blockIdx.x * 256 + threadIdx.x;
   if (c < vecs) dst[(size_t)blockIdx.y * dstPitch + c] = src[(size_t)blockIdx.y * vecs + c];
+}
+
+// dst[row] = the gate and up halves of src[row] ([2d] halfs, gate | up) interleaved in 16-byte pieces: piece 2q of
+// dst is piece q of the gate half, piece 2q + 1 is piece q of the up half (d / 8 pieces per half); dst rows are
+// dstPitch pieces apart.  The layout CUSYNC_EPILOGUE_SWIGLU reads.
+__global__ __launch_bounds__(256) void interleaveGateUpKernel(const uint4v* src, uint4v* dst, uint32_t piecesPerHalf, uint32_t dstPitch) {
+  const uint32_t j = blockIdx.x * 256 + threadIdx.x;
+  if (j < 2 * piecesPerHalf)
+    dst[(size_t)blockIdx.y * dstPitch + j] = src[(size_t)blockIdx.y * 2 * piecesPerHalf + (j & 1) * piecesPerHalf + (j >> 1)];
 }
 
 struct ActParams {
@@ -152,7 +164,22 @@ cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
 // direct-to-LDS tiles are used; below that the M extent follows the batch.  A SwiGLU consumer has
 // to use a register-staged tile, and StridedSync needs the gate|up split on a
 // tile boundary (2752 = 43 * 64).
-void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, int* t1, int* t2) {
+void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, int* t1, int* t2) {
+  if (fused) {
+    // silu(gate) * up in GEMM1's epilogue: both GEMMs have plain operands and run the direct-to-LDS tiles at every
+    // batch size; the kernels mask the ragged last column tile of the shard's widths (2 * 2752 and 8192).  The
+    // policies count columns of the intermediate, half a GEMM1 tile wide, and no width constrains StridedSync.
+    int a, b;
+    if (c.batch <= 32) a = b = CUSYNC_TILE_D32x128x64;
+    else if (c.batch <= 64) a = b = CUSYNC_TILE_D64x128x64;
+    else if (c.batch <= 256) a = b = CUSYNC_TILE_D64x192x64;
+    else if (c.batch <= 1024) a = b = CUSYNC_TILE_128x192x32_ALONE;
+    else { a = CUSYNC_TILE_256x192x32; b = CUSYNC_TILE_256x256x32; }
+    *t1 = c.tile1 >= 0 ? c.tile1 : a;
+    *t2 = c.tile2 >= 0 ? c.tile2 : b;
+    if (c.one_launch && sync != CUSYNC_SYNC_STREAM && c.tile2 < 0) *t2 = *t1;
+    return;
+  }
   int small;
   if (c.batch <= 32) small = CUSYNC_TILE_32x128x64;
   else if (c.batch <= 64) small = CUSYNC_TILE_64x128x64;
@@ -259,6 +286,14 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->ldh = m->n1;
   m->w1p = m->w2p = nullptr;
   m->ldw1 = m->n1; m->ldw2 = m->n2;
+  const bool swiglu = llama && cfg->activation;
+  // where silu(gate) * up is computed: 2 = GEMM1's epilogue (the built-in choice), -1 = a stage of its own, 1 = GEMM2's A loader
+  const int where = !swiglu ? 0 : cfg->swiglu_in_gemm2 == 0 ? 2 : cfg->swiglu_in_gemm2;
+  if (swiglu && where != 2 && where != -1 && where != 1) { setError("mlp: swiglu_in_gemm2 must be -1, 0, 1 or 2"); discard(m); return nullptr; }
+  m->fused = swiglu && where == 2;
+  m->actStage = swiglu && where == -1;
+  m->aMode2 = (swiglu && where == 1) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : m->fused ? CUSYNC_EPILOGUE_SWIGLU : CUSYNC_EPILOGUE_NONE;
   if (cfg->repack_weights) {
     // rows 256 bytes longer than the data: consecutive k rows of a column tile then fall into consecutive
     // channel classes (address bits 8..11) instead of all into one
@@ -270,18 +305,24 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       return nullptr;
     }
   }
-  m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : CUSYNC_EPILOGUE_NONE;
-  const bool swiglu = llama && cfg->activation;
-  // up to 128 rows the third launch costs more than the repeated arithmetic (64 rows: 87 against 82 us)
-  m->actStage = swiglu && (cfg->swiglu_in_gemm2 < 0 || (cfg->swiglu_in_gemm2 == 0 && cfg->batch > 128));
-  m->aMode2 = (swiglu && !m->actStage) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  if (m->fused) {
+    if (cfg->inner % 8 != 0) { setError("mlp: the SwiGLU epilogue needs inner % 8 == 0"); discard(m); return nullptr; }
+    m->ldh = cfg->inner;              // the intermediate is silu(gate) * up itself
+    if (!m->w1p) {                    // not yet there from repack_weights: the handle's interleaved copy of W1
+      m->ldw1 = m->n1;
+      if (CUSYNC_HIP(hipMalloc(&m->w1p, (size_t)m->k1 * m->ldw1 * sizeof(half_t))) || cusync_mlp_reload_weights(m) != CUSYNC_SUCCESS) {
+        discard(m);
+        return nullptr;
+      }
+    }
+  }
   m->act = nullptr;
   m->sMid = nullptr;
   memset(&m->mid, 0, sizeof m->mid);
 
   int sync = cfg->sync;
-  if (swiglu && sync == CUSYNC_SYNC_TILE && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
-  pickTiles(*cfg, sync, m->aMode2 == CUSYNC_A_SWIGLU, &m->tile1, &m->tile2);
+  if (swiglu && !m->fused && sync == CUSYNC_SYNC_TILE && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
+  pickTiles(*cfg, sync, m->aMode2 == CUSYNC_A_SWIGLU, m->fused, &m->tile1, &m->tile2);
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
     setError("mlp: unknown tile id");
@@ -291,6 +332,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
 
   cusync_policy_desc pol = noSync();
   int opts = 0;
+  const uint32_t tnOut = m->fused ? tn1 / 2 : tn1;      // width of a GEMM1 tile in columns of the intermediate
   uint32_t bk1 = 0, bk2 = 0;
   cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk1);
   cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, &bk2);
@@ -310,15 +352,18 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       break;
     case CUSYNC_SYNC_TILE:       // TileSync<TransposeXY,kM,kN> + NoAtomicAdd + ReorderTileLoads, mlp.cu:9-16,111
       pol.kind = CUSYNC_POLICY_TILESYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
-      pol.tileM = tm1; pol.tileN = tn1; pol.waitValue = 1; pol.postValue = 1;
+      pol.tileM = tm1; pol.tileN = tnOut; pol.waitValue = 1; pol.postValue = 1;
       opts = CUSYNC_OPT_NO_ATOMIC_ADD | CUSYNC_OPT_REORDER_TILE_LOADS;
       break;
     case CUSYNC_SYNC_STRIDED:    // StridedSync<TransposeXY,d,kM,kN,2>, mlp.cu:109; atomic add kept (:9-14)
       if (!llama) { setError("mlp: StridedSync is for the gate|up layout"); discard(m); return nullptr; }
-      if (cfg->inner % tn1 != 0) { setError("mlp: StridedSync needs inner % tileN == 0"); discard(m); return nullptr; }
+      if (!m->fused && cfg->inner % tn1 != 0) { setError("mlp: StridedSync needs inner % tileN == 0"); discard(m); return nullptr; }
       pol.kind = CUSYNC_POLICY_STRIDEDSYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
-      pol.tileM = tm1; pol.tileN = tn1; pol.waitValue = 2; pol.postValue = 1;
-      pol.gridN = cfg->inner; pol.stride = 2;
+      pol.tileM = tm1; pol.tileN = tnOut; pol.waitValue = 2; pol.postValue = 1;
+      // GridN: the width of one group (gate, or up) in whole tiles.  With the epilogue computing silu(gate) * up a
+      // workgroup holds the gate tile and the up tile of its column range and posts for both at once; the width
+      // is rounded up to whole tiles (the reference rounds its 2731 columns up to 2816, mlp.cu:247-250).
+      pol.gridN = m->fused ? (cfg->inner + tnOut - 1) / tnOut * tnOut : cfg->inner; pol.stride = 2;
       opts = CUSYNC_OPT_REORDER_TILE_LOADS;
       break;
     default:
@@ -399,18 +444,20 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
 
 cusync_error cusync_mlp_reload_weights(cusync_mlp* m) {
   if (!m) return CUSYNC_ERROR_NOT_INITIALIZED;
-  if (!m->w1p) return CUSYNC_SUCCESS;
-  // a kernel, not a copy-engine transfer: the GEMMs of the last run may have left lines of the padded buffers
+  if (!m->w1p && !m->w2p) return CUSYNC_SUCCESS;
+  // a kernel, not a copy-engine transfer: the GEMMs of the last run may have left lines of the handle's buffers
   // in the L2s, and only a kernel boundary on the device is sure to drop them
   hipStream_t s = nullptr;
   if (CUSYNC_HIP(hipDeviceSynchronize())) return CUSYNC_ERROR_DEVICE;
-  const struct { const void* src; void* dst; uint32_t rows, cols, pitch; } job[2] = {
-      {m->w1, m->w1p, m->k1, m->n1, m->ldw1}, {m->w2, m->w2p, m->k2, m->n2, m->ldw2}};
+  const struct { const void* src; void* dst; uint32_t rows, cols, pitch; bool interleave; } job[2] = {
+      {m->w1, m->w1p, m->k1, m->n1, m->ldw1, m->fused}, {m->w2, m->w2p, m->k2, m->n2, m->ldw2, false}};
   for (const auto& j : job) {
-    if (j.cols % 8 != 0) { setError("mlp: repack_weights needs rows of whole 16-byte pieces"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (!j.dst) continue;
+    if (j.cols % 8 != 0 || (j.interleave && j.cols % 16 != 0)) { setError("mlp: the handle's copies of the weights need rows of whole 16-byte pieces"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     const uint32_t vecs = j.cols / 8;
     const dim3 grid((vecs + 255) / 256, j.rows, 1);
-    hipLaunchKernelGGL(repackRowsKernel, grid, dim3(256), 0, s, (const uint4v*)j.src, (uint4v*)j.dst, vecs, j.pitch / 8);
+    if (j.interleave) hipLaunchKernelGGL(interleaveGateUpKernel, grid, dim3(256), 0, s, (const uint4v*)j.src, (uint4v*)j.dst, vecs / 2, j.pitch / 8);
+    else hipLaunchKernelGGL(repackRowsKernel, grid, dim3(256), 0, s, (const uint4v*)j.src, (uint4v*)j.dst, vecs, j.pitch / 8);
     if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   }
   if (CUSYNC_HIP(hipDeviceSynchronize())) return CUSYNC_ERROR_DEVICE;

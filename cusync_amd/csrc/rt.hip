@@ -226,10 +226,34 @@ cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc* prod, void* stre
   return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
+// True when the stream can be held back by the command processor itself (hipStreamWaitValue32) and the
+// environment does not ask for the wait kernel (CUSYNC_WAIT_KERNEL set to something other than 0).
+static bool queueWaitAvailable() {
+  static const bool ok = [] {
+    const char* v = getenv("CUSYNC_WAIT_KERNEL");
+    if (v && *v && strcmp(v, "0") != 0) return false;
+    int dev = 0, can = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    if (hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, dev) != hipSuccess) return false;
+    return can != 0;
+  }();
+  return ok;
+}
+
 cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void* stream, void* launch_event) {
   if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
   if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
   if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
+  if (!prod->kernelExecuted) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (queueWaitAvailable()) {
+    // The command processor polls the flag: no wave sits on a CU, so the wait cannot take a slot from the
+    // producer's workgroups wherever it lands relative to their dispatch, and no launch event is needed.
+    // The producer's flag store is an agent-scope release, which writes through to memory where the
+    // command processor reads.
+    if (RT(hipStreamWaitValue32((hipStream_t)stream, prod->kernelExecuted, (uint32_t)prod->iter, hipStreamWaitValueGte, 0xffffffffu)))
+      return CUSYNC_ERROR_DEVICE;
+    return CUSYNC_SUCCESS;
+  }
   if (launch_event && RT(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)launch_event, 0))) return CUSYNC_ERROR_DEVICE;
   return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }

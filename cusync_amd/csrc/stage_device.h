@@ -256,13 +256,14 @@ struct DynStage {
     return ready;
   }
 
-  // Workgroup-wide post; contains a barrier, call from all threads.
-  __device__ __forceinline__ void post(const cusync_dim3& tile) const {
+  // Workgroup-wide post; contains a barrier, call from all threads.  `times`: how many posts of the policy this
+  // one stands for (a workgroup that finished several logical tiles guarded by one semaphore adds them at once).
+  __device__ __forceinline__ void post(const cusync_dim3& tile, uint32_t times = 1) const {
     if (!isProducer()) return;
     __syncthreads();
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
       const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid) * CUSYNC_SEM_STRIDE;
-      const uint32_t v = dyn::postValue(d.out);
+      const uint32_t v = dyn::postValue(d.out) * times;
       if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::releaseStore(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
       else dev::releaseAdd(&d.tileStatusWrite[idx], v);
     }

@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <string>
+#include <vector>
 #include <stdint.h>
 
 #include "../../include/cusync_amd.h"
@@ -101,6 +103,27 @@ cusync_error cusync_sync_overhead_pair(uint32_t blocks, uint32_t threads, int wa
       if (i >= warmup) total[mode] += nowUs() - t0;
       if (mode == 0) { prod.incrementIter(); cons.incrementIter(); }
     }
+    // The pair's result (sync-overhead.cu checks nothing; tests/simple-test.cu checks a synced pair this way):
+    // every element is what the producer of the LAST run wrote, plus one.  A consumer block that read before
+    // its producer block had posted would have found the value of the run before.
+    if (result == CUSYNC_SUCCESS) {
+      std::vector<float> host(n);
+      if (CUSYNC_HIP(hipMemcpy(host.data(), out, n * 4, hipMemcpyDeviceToHost))) { result = CUSYNC_ERROR_DEVICE; break; }
+      const float want = (float)(warmup + iters - 1) + 1.0f;
+      size_t bad = 0;
+      for (size_t k = 0; k < n; k++) bad += host[k] != want;
+      if (bad) {
+        cusync::rt::setError(std::string("sync overhead pair: ") + std::to_string(bad) + " of " + std::to_string(n) +
+                             " elements are not the producer's value plus one (" + (mode == 0 ? "post/wait on two streams" : "stream order") + ")");
+        result = CUSYNC_ERROR_DEVICE;
+      }
+    }
+  }
+  if (result == CUSYNC_SUCCESS) {
+    const cusync_stage_desc cd = cons.desc();
+    uint32_t gaveUp = 0;
+    if (cusync_stage_read_state(&cd, nullptr, nullptr, nullptr, nullptr, nullptr, &gaveUp) != CUSYNC_SUCCESS) result = CUSYNC_ERROR_DEVICE;
+    else if (gaveUp) { cusync::rt::setError("sync overhead pair: a wait gave up"); result = CUSYNC_ERROR_DEVICE; }
   }
   *with_sync_us = total[0] / iters;
   *without_sync_us = total[1] / iters;

@@ -153,16 +153,18 @@ cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc *prod, cu
  * enqueues a one-wave kernel on `stream` that returns once the producer's flag
  * has reached desc->iter.  No-op with AVOID_WAIT_KERNEL. */
 cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc *prod, void *stream);
-/* Same, but `stream` first waits for `launch_event` (a hipEvent_t the caller
- * recorded on the producer's stream immediately before launching the producer's
- * kernel; NULL = no ordering).  The two streams are separate hardware queues and
- * the wait kernel's wave can reach the GPU before the producer's workgroups do.
- * It then holds registers on one CU until every producer workgroup has started;
- * a producer whose workgroups need whole CUs and fill the machine cannot place
- * its last workgroup there, the flag is not raised until another workgroup
- * retires, and that run of the chain is one producer tile longer.  Behind the
- * event the wait kernel is dispatched after the producer's launch has begun.
- * No counterpart in the reference, which launches the wait kernel unordered
+/* What the chains of this library call in place of invokeWaitKernel.  Where the device can hold a stream back
+ * on a memory value by itself (hipStreamWaitValue32; every MI355X) no kernel is launched at all: the command
+ * processor polls the producer's flag and releases `stream` when it has reached desc->iter.  A wait kernel is a
+ * wave that holds registers on one CU until the flag rises; it runs in another hardware queue than the producer
+ * and can reach the GPU first, and a producer whose workgroups need whole CUs and fill the machine then cannot
+ * place its last workgroup, the flag is not raised until another workgroup retires, and that run of the chain is
+ * one producer tile longer (seen as a second mode in the step times, 700-790 us against 610).  The queue-side
+ * wait holds no CU.  It has no give-up: only call it for a producer that has been, or is about to be, launched.
+ * With CUSYNC_WAIT_KERNEL=1 in the environment, or on a device without the queue-side wait, the wait kernel is
+ * launched instead, behind `launch_event` (a hipEvent_t the caller recorded on the producer's stream immediately
+ * before launching the producer's kernel; NULL = no ordering), which keeps its wave behind the producer's
+ * dispatch in all but rare cases.  No counterpart in the reference, which launches the wait kernel unordered
  * (src/ml-bench/transformer/mlp.cu:683-699). */
 cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc *prod, void *stream, void *launch_event);
 /* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
@@ -188,7 +190,16 @@ cusync_dim3 cusync_order_tile_to_block(int order, cusync_dim3 tile);
 /* cusyncgemm.h:208-399)                                                      */
 /* ------------------------------------------------------------------------- */
 
-enum { CUSYNC_EPILOGUE_NONE = 0, CUSYNC_EPILOGUE_GELU = 1, CUSYNC_EPILOGUE_RELU = 2 };
+enum {
+  CUSYNC_EPILOGUE_NONE = 0, CUSYNC_EPILOGUE_GELU = 1, CUSYNC_EPILOGUE_RELU = 2,
+  /* D[m, 8q + t] = silu(P[m, 16q + t]) * P[m, 16q + 8 + t], P = A*B, t = 0..7: B holds the gate and the up
+   * projection of a SwiGLU feed-forward with their columns interleaved in groups of eight (gate columns 8q..8q+7,
+   * then up columns 8q..8q+7), so that a workgroup has both factors of an output element in its own registers and
+   * the activation costs no pass of its own (LinearCombinationSilu + LinearCombinationSwiGLU of the reference's
+   * library build, TB/mlp-lib.cu:122-133, in one epilogue).  D has N/2 columns; N % 16 == 0.  The tile is posted
+   * under the output's coordinates {row, n0 / 2}: a consumer's policy counts columns of D. */
+  CUSYNC_EPILOGUE_SWIGLU = 3
+};
 /* How the A operand is formed while it is staged into LDS. */
 enum {
   CUSYNC_A_PLAIN = 0,
@@ -226,7 +237,7 @@ typedef struct cusync_gemm_args {
   uint32_t M, N, K;            /* problem_size */
   const void *A; uint32_t lda; /* fp16 row-major [M,K] (or [M,2K] gate|up for CUSYNC_A_SWIGLU) */
   const void *B; uint32_t ldb; /* fp16 row-major [K,N] */
-  void *D; uint32_t ldd;       /* fp16 row-major [M,N]; D = epilogue(A*B), alpha = 1, beta = 0 */
+  void *D; uint32_t ldd;       /* fp16 row-major [M,N] ([M,N/2] with CUSYNC_EPILOGUE_SWIGLU); D = epilogue(A*B), alpha = 1, beta = 0 */
   int32_t epilogue;            /* CUSYNC_EPILOGUE_* */
   int32_t a_mode;              /* CUSYNC_A_* */
   int32_t tile;                /* CUSYNC_TILE_* */
@@ -430,11 +441,18 @@ typedef struct cusync_mlp_config {
   int32_t max_wg1, max_wg2;    /* workgroups per launch of each GEMM; 0 = built-in choice, -1 = as many as stay resident */
   int32_t one_launch;          /* 1 (with a CuSync mode): both GEMMs in one launch, cusync_gemm_chain_run; needs the same
                                   direct-to-LDS tile for both and a plain A operand in GEMM2 */
-  int32_t swiglu_in_gemm2;     /* LLaMA with activation: where silu(gate)*up is computed.  -1: in a stage of its own between
-                                  the GEMMs (a third kernel and stream, every element once; GEMM2 then runs the
-                                  direct-to-LDS tiles).  1: in GEMM2's A loader as the data passes (one kernel fewer,
-                                  but repeated for every column tile of GEMM2: 357 against 128 us at 2048 rows).
-                                  0: built-in choice, the stage of its own above 128 rows */
+  int32_t swiglu_in_gemm2;     /* LLaMA with activation: where silu(gate)*up is computed.
+                                  2: in GEMM1's epilogue (CUSYNC_EPILOGUE_SWIGLU).  create() copies w1 into a buffer of its
+                                  own with the gate and up columns interleaved in groups of eight (call
+                                  cusync_mlp_reload_weights after changing the caller's copy); the intermediate h is then
+                                  silu(gate)*up itself, [batch][inner] packed at the front of the caller's buffer, GEMM2
+                                  reads it with the direct-to-LDS tiles, and the policies count its columns (a GEMM1 tile
+                                  is half as wide there; under StridedSync it posts for its gate half and its up half at
+                                  once).  Two kernels, every element once, half the intermediate traffic.
+                                  -1: in a stage of its own between the GEMMs (a third kernel and stream; h is gate|up).
+                                  1: in GEMM2's A loader as the data passes (repeated for every column tile of GEMM2:
+                                  357 against 128 us at 2048 rows; h is gate|up).
+                                  0: built-in choice, which is 2 */
   int32_t repack_weights;      /* 1: create() copies w1 and w2 into buffers of its own whose row pitch is 256 bytes longer
                                   than the row, and the GEMMs read those (call cusync_mlp_reload_weights after changing
                                   the caller's copies).  The shards' rows are multiples of 4 KiB, so a column tile of the
@@ -453,8 +471,9 @@ void cusync_mlp_destroy(cusync_mlp *mlp);
 /* With repack_weights: copies the caller's w1 / w2 (the pointers given to create) into the padded buffers again. */
 cusync_error cusync_mlp_reload_weights(cusync_mlp *mlp);
 /* runLLAMA / runCuSyncLLAMA (TB/mlp-lib.cu:569-576, 611-618): `runs` back-to-back
- * passes x -> h -> y.  h is the intermediate [batch, inner] (GPT-3) or
- * [batch, 2*inner] (LLaMA).  If times_us != NULL it receives one elapsed time
+ * passes x -> h -> y.  h is the intermediate [batch, inner] (GPT-3) or a buffer of
+ * [batch, 2*inner] (LLaMA: gate|up, or silu(gate)*up in its first batch*inner elements
+ * when the activation is GEMM1's epilogue, see cusync_mlp_config::swiglu_in_gemm2).  If times_us != NULL it receives one elapsed time
  * per run, measured with events start (producer stream) -> end (consumer stream)
  * exactly as TB/mlp.cu:691-708; each run is then followed by an event wait. */
 /* Returns CUSYNC_ERROR_DEVICE (text in cusync_rt_last_error) when a wait of one of the chain's stages, the wait
@@ -479,7 +498,9 @@ int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 /* The example's experiment (sync-overhead.cu:40-105): a producer kernel that writes one value per thread and a
  * consumer kernel that adds one to it, `blocks` x `threads`, timed from the host over `iters` runs after `warmup`:
  * once with CuStage tile/post/wait per block on two streams, once stream-ordered without any of it.
- * Overhead in percent = (with - without) / without * 100 (:104). */
+ * Overhead in percent = (with - without) / without * 100 (:104).  After each of the two legs the consumer's output
+ * is checked: every element must be the value the producer wrote in the last run plus one, and no wait may have
+ * given up; otherwise CUSYNC_ERROR_DEVICE with the count in cusync_rt_last_error(). */
 cusync_error cusync_sync_overhead_pair(uint32_t blocks, uint32_t threads, int warmup, int iters,
                                        double *with_sync_us, double *without_sync_us);
 /* Latency of a post -> wait hand-over: workgroup 0 and workgroup `partner` (1..63) of one launch pass a

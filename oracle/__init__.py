@@ -89,6 +89,8 @@ def lib():
     L.orc_gemm_f16.argtypes = [u32, u32, u32, vp, u32, vp, u32, vp, u32, i32]
     L.orc_swiglu_f16.restype = None
     L.orc_swiglu_f16.argtypes = [u32, u32, vp, u32, vp, u32]
+    L.orc_gemm_swiglu_f16.restype = None
+    L.orc_gemm_swiglu_f16.argtypes = [u32, u32, u32, vp, u32, vp, u32, vp, u32]
     L.orc_attention_f16.restype = None
     L.orc_attention_f16.argtypes = [u32, u32, u32, vp, u32, vp, u32, i32]
     L.orc_attention_kv_f16.restype = None
@@ -222,6 +224,16 @@ def swiglu(gu, d):
     M, ld = gu.shape
     h = np.empty((M, d), dtype=np.uint16)
     lib().orc_swiglu_f16(M, d, _ptr(gu), ld, _ptr(h), d)
+    return h.view(np.float16)
+
+
+def gemm_swiglu(a, w, d):
+    """H[M,d] = silu(A @ W[:, :d]) * (A @ W[:, d:]) with the activation applied to the fp32 accumulators."""
+    a, w = _h(a), _h(w)
+    M, K = a.shape
+    assert w.shape == (K, 2 * d)
+    h = np.empty((M, d), dtype=np.uint16)
+    lib().orc_gemm_swiglu_f16(M, d, K, _ptr(a), K, _ptr(w), 2 * d, _ptr(h), d)
     return h.view(np.float16)
 
 

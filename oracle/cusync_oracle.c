@@ -349,6 +349,29 @@ void orc_swiglu_f16(uint32_t M, uint32_t d, const uint16_t *gu, uint32_t ld_gu,
     }
 }
 
+/* The LLaMA feed-forward's first stage with the activation applied to the accumulators, as an epilogue of the
+ * GEMM: H[i][j] = silu(sum_k X[i][k] W[k][j]) * (sum_k X[i][k] W[k][d + j]), W = gate | up side by side
+ * ([K][2d]).  Both sums are ref_cpumatmul's (TB/common.h:89-102: fp32, k ascending), the product is formed in
+ * fp32 and rounded to fp16 once.  This is where the reference puts the activation in its library build
+ * (TB/mlp-lib.cu:122-133: LinearCombinationSilu on X W1, then LinearCombinationSwiGLU scaling the accumulator
+ * of X V by it); its arithmetic lives in CUTLASS, which is absent, so the closed form x*sigmoid(x)*u stands in. */
+void orc_gemm_swiglu_f16(uint32_t M, uint32_t d, uint32_t K,
+                         const uint16_t *A, uint32_t lda, const uint16_t *W, uint32_t ldw,
+                         uint16_t *H, uint32_t ldh) {
+  for (uint32_t i = 0; i < M; i++) {
+    #pragma omp parallel for
+    for (uint32_t j = 0; j < d; j++) {
+      float gate = 0, up = 0;
+      for (uint32_t k = 0; k < K; k++) {
+        const float a = orc_h2f(A[(size_t)i * lda + k]);
+        gate += a * orc_h2f(W[(size_t)k * ldw + j]);
+        up += a * orc_h2f(W[(size_t)k * ldw + d + j]);
+      }
+      H[(size_t)i * ldh + j] = orc_f2h(orc_silu(gate) * up);
+    }
+  }
+}
+
 /* Textbook softmax(mask(Q K^T / sqrt(hd))) V per head, all in fp32.  The S query rows are rows
  * cached .. cached+S-1 of qkv; keys and values are rows 0 .. cached+S-1 (rows below `cached` are the
  * key/value cache of TB/attention.cu:272-276, 289: the projection writes its rows behind `seqlen` cached

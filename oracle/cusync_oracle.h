@@ -131,6 +131,10 @@ void orc_gemm_f16(uint32_t M, uint32_t N, uint32_t K,
 /* h[r,i] = fp16( silu(gu[r,i]) * gu[r,i+d] ), gu has row pitch ld_gu. */
 void orc_swiglu_f16(uint32_t M, uint32_t d, const uint16_t *gu, uint32_t ld_gu,
                     uint16_t *h, uint32_t ld_h);
+/* H = silu(A W[:, 0:d]) * (A W[:, d:2d]) with the activation on the fp32 accumulators (one rounding). */
+void orc_gemm_swiglu_f16(uint32_t M, uint32_t d, uint32_t K,
+                         const uint16_t *A, uint32_t lda, const uint16_t *W, uint32_t ldw,
+                         uint16_t *H, uint32_t ldh);
 /* Causal multi-head attention over one sequence.  qkv is [S, 3*heads*hd] laid
  * out as [Q | K | V] blocks of heads*hd columns; out is [S, heads*hd]. */
 void orc_attention_f16(uint32_t S, uint32_t heads, uint32_t hd,

@@ -50,13 +50,18 @@ def run_mlp(model, batch, hidden, inner, sync, runs=2, activation=1, **kw):
     return x, w1, w2, to_host(dh), to_host(dy), prod, cons, tiles, times
 
 
-def check_against_oracle(model, x, w1, w2, h, y, inner, activation=1):
+def check_against_oracle(model, x, w1, w2, h, y, inner, activation=1, fused=False):
     rows = sample_rows(x.shape[0])
     xs = np.ascontiguousarray(x[rows])
     if model == api.MODEL.GPT3:
         h_ref = orc.gemm(xs, w1, orc.EPI_GELU if activation else orc.EPI_NONE)
         assert_close(h[rows], h_ref, "H rows")
         a2 = np.ascontiguousarray(h[rows])
+    elif fused:
+        # silu(gate) * up is GEMM1's epilogue: the intermediate is [batch][inner], packed at the front of the buffer
+        hh = h.reshape(-1)[:x.shape[0] * inner].reshape(x.shape[0], inner)
+        assert_close(hh[rows], orc.gemm_swiglu(xs, w1, inner), "silu(gate)*up rows")
+        a2 = np.ascontiguousarray(hh[rows])
     else:
         h_ref = orc.gemm(xs, w1)
         assert_close(h[rows], h_ref, "gate|up rows")
@@ -65,12 +70,18 @@ def check_against_oracle(model, x, w1, w2, h, y, inner, activation=1):
     assert_close(y[rows], orc.gemm(a2, w2), "Y rows")
 
 
-def expected_sems(prod, tiles, iters):
+def expected_sems(prod, tiles, iters, fused=False):
     d = prod.desc
     p = orc.Policy(d.out.kind, d.out.order, d.out.tileM, d.out.tileN, d.out.waitValue, d.out.postValue,
                    d.out.gridN, d.out.stride, d.out.R, d.out.S, d.out.H)
     tm, tn, _ = api.tile_shape(tiles[0])
-    return orc.expected_sems_gemm(p, prod.grid, tm, tn, iters, d.opts)
+    if fused and d.out.kind == api.POLICY.STRIDEDSYNC:
+        # the reference's grid has a gate tile and an up tile per column range, folded onto one semaphore that
+        # counts to 2 per run (TB/mlp.cu:90-96); a tile of the SwiGLU epilogue is both
+        want = np.zeros(prod.grid[0] * prod.grid[1] * prod.grid[2], np.uint32)
+        want[:prod.grid[0] * prod.grid[1]] = 2 * iters
+        return want
+    return orc.expected_sems_gemm(p, prod.grid, tm, tn // 2 if fused else tn, iters, d.opts)
 
 
 @pytest.mark.parametrize("batch", [1, 16, 64, 256, 512])
@@ -113,26 +124,40 @@ def test_gpt3_without_activation_matches_reference_check_build():
     check_against_oracle(api.MODEL.GPT3, x, w1, w2, h, y, inner=6144, activation=0)
 
 
-@pytest.mark.parametrize("in_gemm2", [-1, 1])
+@pytest.mark.parametrize("in_gemm2", [2, -1, 1])
 @pytest.mark.parametrize("inner", [2752, 2816])
 @pytest.mark.parametrize("batch", [1, 16, 64, 256, 512, 1024, 2048])
 def test_llama_mlp(inner, batch, in_gemm2):
-    # silu(gate) * up either as a stage of its own between the GEMMs or in GEMM2's A loader
+    # silu(gate) * up as GEMM1's epilogue (2, the built-in choice), as a stage of its own between the GEMMs (-1) or in
+    # GEMM2's A loader (1)
     print("llama", inner, batch, in_gemm2, flush=True)
+    fused = in_gemm2 == 2
     outs = {}
-    # StridedSync constrains the tile width (gate|up split on a tile boundary); the other modes are run with
-    # the same tiles and k-slices so that all three execute the same kernels and must agree bit for bit
+    # StridedSync constrains the tile width when gate|up is the intermediate (the split on a tile boundary); the other
+    # modes are run with the same tiles and k-slices so that all execute the same kernels and must agree bit for bit
     same = {}
-    for sync in (api.SYNC.STRIDED, api.SYNC.STREAM, api.SYNC.ROW):
+    modes = (api.SYNC.STRIDED, api.SYNC.STREAM, api.SYNC.ROW) + ((api.SYNC.TILE,) if fused else ())
+    for sync in modes:
         x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, inner, sync, runs=2, swiglu_in_gemm2=in_gemm2, **same)
         same = dict(tile1=tiles[0], tile2=tiles[1], split_k1=tiles[2], split_k2=tiles[3])
         outs[sync] = (h, y)
         assert cons.spin_timeouts == 0
         if sync != api.SYNC.STREAM:
-            assert np.array_equal(prod.sems, expected_sems(prod, tiles, 2))
-    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, *outs[api.SYNC.STREAM], inner=inner)
-    for sync in (api.SYNC.ROW, api.SYNC.STRIDED):
+            assert np.array_equal(prod.sems, expected_sems(prod, tiles, 2, fused))
+    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, *outs[api.SYNC.STREAM], inner=inner, fused=fused)
+    for sync in modes:
         assert np.array_equal(outs[sync][1].view(np.uint16), outs[api.SYNC.STREAM][1].view(np.uint16))
+
+
+def test_llama_built_in_choice_is_the_fused_epilogue():
+    # swiglu_in_gemm2 = 0: two kernels, the intermediate is silu(gate) * up
+    x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, 300, 8192, 2752, api.SYNC.STRIDED, runs=2)
+    assert api.tile_shape(tiles[0])[2] in (32, 64) and cons.spin_timeouts == 0
+    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, h, y, inner=2752, fused=True)
+    # against the unfused arithmetic on the caller's weights: round gate|up to fp16, then the activation
+    rows = sample_rows(300)
+    hh = h.reshape(-1)[:300 * 2752].reshape(300, 2752)
+    assert_close(hh[rows], orc.swiglu(orc.gemm(np.ascontiguousarray(x[rows]), w1), 2752), "against swiglu(gemm)")
 
 
 def test_llama_reference_wiring_no_activation():
@@ -147,7 +172,7 @@ def test_strided_sync_rejects_unaligned_split():
     w = torch.zeros(16, device="cuda", dtype=torch.float16)
     with pytest.raises(RuntimeError, match="inner % tileN"):
         api.Mlp(api.MODEL.LLAMA, 256, 8192, 2752, api.SYNC.STRIDED, w.data_ptr(), w.data_ptr(),
-                tile1=api.TILE.T256x128x64)
+                tile1=api.TILE.T256x128x64, swiglu_in_gemm2=-1)
 
 
 @pytest.mark.parametrize("batch", [1, 16, 64, 256, 512, 1024, 2048])
@@ -188,9 +213,10 @@ def test_mlp_with_repacked_weights(model, inner, batch, sync):
     x, w1, w2, h0, y0, _, _, tiles0, _ = run_mlp(model, batch, hidden, inner, sync)
     _, _, _, h1, y1, prod, cons, tiles1, _ = run_mlp(model, batch, hidden, inner, sync, repack_weights=True)
     assert tiles0 == tiles1
-    assert np.array_equal(h0, h1) and np.array_equal(y0, y1)
+    # bit for bit (the LLaMA intermediate fills only the front of its buffer, the rest stays NaN)
+    assert np.array_equal(h0.view(np.uint16), h1.view(np.uint16)) and np.array_equal(y0.view(np.uint16), y1.view(np.uint16))
     assert cons.spin_timeouts == 0
-    check_against_oracle(model, x, w1, w2, h1, y1, inner)
+    check_against_oracle(model, x, w1, w2, h1, y1, inner, fused=model == api.MODEL.LLAMA)
 
 
 def test_mlp_repacked_weights_reload():

@@ -8,7 +8,9 @@ pytestmark = pytest.mark.gpu
 
 
 def test_sync_overhead_pair_runs():
-    # the example's grid: 80 * 2 * (1024 / 128) blocks of 128 threads (sync-overhead.cu:69-71)
+    # the example's grid: 80 * 2 * (1024 / 128) blocks of 128 threads (sync-overhead.cu:69-71).  The call itself
+    # checks the consumer's output after each leg (out[i] == producer's last value + 1, as tests/simple-test.cu
+    # checks a synced pair) and raises if an element differs or a wait gave up.
     with_sync, without = api.sync_overhead_pair(1280, 128, warmup=5, iters=30)
     print("pair: with sync %.1f us, without %.1f us, overhead %.1f %%" % (with_sync, without, (with_sync - without) / without * 100))
     assert 0 < without < 1e4 and 0 < with_sync < 1e4
@@ -19,6 +21,13 @@ def test_pingpong_terminates_with_sane_latency(partner):
     ns = api.sync_overhead_pingpong(partner, rounds=500)
     print("partner %d: %.0f ns per round trip" % (partner, ns))
     assert 100 < ns < 100000      # a round trip is two hand-overs through the coherent level of the memory system
+
+
+@pytest.mark.parametrize("blocks,threads", [(1, 64), (7, 1024), (4096, 256)])
+def test_sync_overhead_pair_checks_its_output(blocks, threads):
+    # other grids than the example's: one block, blocks of the largest size, more blocks than stay resident
+    with_sync, without = api.sync_overhead_pair(blocks, threads, warmup=2, iters=5)
+    assert with_sync > 0 and without > 0
 
 
 def test_pingpong_rejects_bad_arguments():

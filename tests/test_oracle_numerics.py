@@ -111,6 +111,30 @@ def test_swiglu():
     assert np.max(np.abs(got.astype(np.float32) - wrong.astype(np.float32))) > 0.05
 
 
+def test_gemm_swiglu_fused_on_the_accumulators():
+    # silu(X Wg) * (X Wu) with one rounding at the end: against numpy in float64, against the two-step form
+    # (round gate|up to fp16, then orc.swiglu) within fp16 rounding, and not symmetric in gate and up
+    rng = np.random.default_rng(14)
+    M, K, d = 7, 96, 24
+    x = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, 2 * d)) * 0.3).astype(np.float16)
+    got = orc.gemm_swiglu(x, w, d).astype(np.float64)
+    acc = x.astype(np.float64) @ w.astype(np.float64)
+    g, u = acc[:, :d], acc[:, d:]
+    want = g / (1 + np.exp(-g)) * u
+    assert np.max(np.abs(got - want)) <= 2e-3 + 1e-3 * np.max(np.abs(want))
+    two_step = orc.swiglu(orc.gemm(x, w), d).astype(np.float64)
+    assert np.max(np.abs(got - two_step)) <= 1e-2 * np.max(np.abs(want)) + 1e-3
+    wrong = u / (1 + np.exp(-u)) * g
+    assert np.max(np.abs(got - wrong)) > 0.05
+    # integer data with gate = 0 columns: silu(0) * u == 0 exactly; with up = 1: silu(gate) alone
+    xi = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    wi = rng.integers(-1, 2, (K, 2 * d)).astype(np.float16)
+    wi[:, :d // 2] = 0
+    hi = orc.gemm_swiglu(xi, wi, d)
+    assert np.all(hi[:, :d // 2] == 0)
+
+
 def test_attention_invariants_and_numpy():
     rng = np.random.default_rng(5)
     S, heads, hd = 37, 3, 16
