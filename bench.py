@@ -272,8 +272,8 @@ def main():
             chains = [Chain(b, api.SYNC.STREAM), Chain(b, api.SYNC.ROW), Chain(b, api.SYNC.TILE)]
             tiles = chains[0].tiles
             if tiles[0] == tiles[1]:
-                names.append("rowsync_one_launch")
-                chains.append(Chain(b, api.SYNC.ROW, one_launch=True))
+                names += ["rowsync_one_launch", "tilesync_one_launch"]
+                chains += [Chain(b, api.SYNC.ROW, one_launch=True), Chain(b, api.SYNC.TILE, one_launch=True)]
             names += ["stream_rp", "rowsync_rp"]
             chains += [Chain(b, api.SYNC.STREAM, repack=True), Chain(b, api.SYNC.ROW, repack=True)]
             if tiles[0] == tiles[1]:
@@ -287,7 +287,7 @@ def main():
             t["stream"] = [v[0] for v in t["stream"]]
             m = {k: trimmed(v) for k, v in t.items()}
             s_us = m["stream"][0]
-            in_place = [k for k in ("rowsync", "tilesync", "rowsync_one_launch") if k in m]
+            in_place = [k for k in ("rowsync", "tilesync", "rowsync_one_launch", "tilesync_one_launch") if k in m]
             best = min(m[k][0] for k in in_place)
             rp = [m[k][0] for k in ("stream_rp", "rowsync_rp", "rowsync_one_launch_rp") if k in m]
             per_batch.append({
@@ -299,6 +299,8 @@ def main():
                 "tilesync_us": round(m["tilesync"][0], 2), "tilesync_std": round(m["tilesync"][1], 2),
                 "tilesync_gain_pct": round(100 - m["tilesync"][0] / s_us * 100, 2),
                 "rowsync_one_launch_us": round(m["rowsync_one_launch"][0], 2) if "rowsync_one_launch" in m else None,
+                "tilesync_one_launch_us": round(m["tilesync_one_launch"][0], 2) if "tilesync_one_launch" in m else None,
+                "best_policy": min(in_place, key=lambda k: m[k][0]),
                 "best_gain_pct": round(100 - best / s_us * 100, 2),
                 "repacked_weights": {"stream_us": round(m["stream_rp"][0], 2), "rowsync_us": round(m["rowsync_rp"][0], 2),
                                      "rowsync_one_launch_us": round(m["rowsync_one_launch_rp"][0], 2) if "rowsync_one_launch_rp" in m else None,
@@ -406,6 +408,11 @@ def main():
     names = ["stream", "rowsync", "tilesync"]
     chains = [Chain(B, api.SYNC.STREAM), Chain(B, api.SYNC.ROW), Chain(B, api.SYNC.TILE)]
     tiles = chains[1].tiles
+    if tiles[0] == tiles[1]:
+        # the same stages and semaphores with both GEMMs in ONE launch: every workgroup works through the producer's
+        # tiles it draws, then the consumer's, waiting on the tiles' semaphores in between (no second stream)
+        names += ["rowsync_one_launch", "tilesync_one_launch"]
+        chains += [Chain(B, api.SYNC.ROW, one_launch=True), Chain(B, api.SYNC.TILE, one_launch=True)]
     for _ in range(args.warmup):
         for c in chains:
             c.step()
@@ -419,7 +426,7 @@ def main():
             wall[n] += time.perf_counter() - t0
     for c in chains:
         c.close()
-    policy = min(("rowsync", "tilesync"), key=lambda k: statistics.fmean(step_times[k]))
+    policy = min((n for n in names if n != "stream"), key=lambda k: statistics.fmean(step_times[k]))
     ms_per_step = wall[policy] / args.steps * 1e3
 
     def spread(v):

@@ -74,6 +74,7 @@ class MlpConfig(C.Structure):
 # every symbol include/cusync_amd.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "cusync_rt_last_error": (C.c_char_p, []),
+    "cusync_rt_set_timeline": (C.c_int, [vp, sz]),
     "cusync_rt_device_count": (C.c_int, []),
     "cusync_rt_device_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz), C.c_char_p, sz]),
     "cusync_rt_malloc": (C.c_int, [C.POINTER(vp), sz]),
@@ -98,6 +99,7 @@ SIGNATURES = {
     "cusync_set_producer_consumer_pair": (C.c_int, [C.POINTER(StageDesc), C.POINTER(StageDesc)]),
     "cusync_invoke_wait_kernel": (C.c_int, [C.POINTER(StageDesc), vp]),
     "cusync_invoke_wait_kernel_after": (C.c_int, [C.POINTER(StageDesc), vp, vp]),
+    "cusync_wait_producer_started": (C.c_int, [C.POINTER(StageDesc), u32]),
     "cusync_wait_kernel": (C.c_int, [vp, u32, vp]),
     "cusync_stage_read_state": (C.c_int, [C.POINTER(StageDesc), vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_policy_tile_index": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),
@@ -111,6 +113,7 @@ SIGNATURES = {
     "cusync_gemm_can_implement": (C.c_int, [C.POINTER(GemmArgs)]),
     "cusync_gemm_workspace_size": (sz, [C.POINTER(GemmArgs)]),
     "cusync_gemm_max_resident": (C.c_int, [C.c_int]),
+    "cusync_gemm_fills_device": (C.c_int, [C.POINTER(GemmArgs)]),
     "cusync_gemm_chain_run": (C.c_int, [C.POINTER(GemmArgs), C.c_int, vp]),
     "cusync_gemm_run": (C.c_int, [C.POINTER(GemmArgs), vp]),
     "cusync_gemm_run_static_workspace": (C.c_int, [C.POINTER(GemmArgs), vp]),

@@ -344,14 +344,15 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     cusync_error e;
     if (CUSYNC_HIP(hipEventRecord(L->eStart, s0))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_gemm_run(&a1, s0)) != CUSYNC_SUCCESS) return e;
-    // overlapped: each wait kernel goes behind the event recorded right before its producer's launch (ahead of
-    // it, its wave would hold a CU that one of the producer's workgroups needs); eMid1 marks the attention launch
+    // overlapped: each consumer's stream is held back until every workgroup of its producer has started: from the
+    // host when the producer's launch takes every workgroup slot of the device (a wait kernel's wave would keep its
+    // last workgroup off the device), by the wait kernel otherwise.  eMid1 / eMid2 only serve the stage timing.
     if (overlapped) {
-      if ((e = cusync_invoke_wait_kernel_after(&L->st[0], s1, L->eStart)) != CUSYNC_SUCCESS) return e;
+      if ((e = cusync_gemm_fills_device(&a1) ? cusync_wait_producer_started(&L->st[0], 0) : cusync_invoke_wait_kernel(&L->st[0], s1)) != CUSYNC_SUCCESS) return e;
     }
     if (CUSYNC_HIP(hipEventRecord(L->eMid1, s1))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_attention_run(&a2, s1)) != CUSYNC_SUCCESS) return e;
-    if (overlapped) { if ((e = cusync_invoke_wait_kernel_after(&L->st[1], s2, L->eMid1)) != CUSYNC_SUCCESS) return e; }
+    if (overlapped) { if ((e = cusync_invoke_wait_kernel(&L->st[1], s2)) != CUSYNC_SUCCESS) return e; }
     else if (CUSYNC_HIP(hipEventRecord(L->eMid2, s0))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_gemm_run(&a3, s2)) != CUSYNC_SUCCESS) return e;
     if (CUSYNC_HIP(hipEventRecord(L->eEnd, s2))) return CUSYNC_ERROR_DEVICE;

@@ -123,6 +123,7 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
   p.mPad = s.grid.y * ti->bm;
   p.waitRound = 1;
+  p.timeline = nullptr; p.timelineCap = 0;
   // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
                         (a->C * 2) % 128 == 0 &&
@@ -391,10 +392,10 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
       hipStream_t s = c->stream[overlapped ? i : 0];
       const cusync_conv2d_args a = layerArgs(i);
       cusync_error e;
-      // overlapped: ev[i] marks the launch of layer i on its stream, and the wait kernel for layer i - 1 goes
-      // behind ev[i - 1] (ahead of that launch its wave would hold a CU one of the producer's workgroups needs)
-      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel_after(&c->st[i - 1], s, c->ev[i - 1])) != CUSYNC_SUCCESS) return e;
-      if (overlapped && i > 0 && i + 1 < n && CUSYNC_HIP(hipEventRecord(c->ev[i], s))) return CUSYNC_ERROR_DEVICE;
+      // overlapped: the reference's wait kernel holds layer i's stream back until layer i - 1 is on the device.  A
+      // layer's launch leaves workgroup slots free (392 tiles on 512 slots for the benchmark shapes; any launch of
+      // fewer workgroups than stay resident), so the wait kernel's wave takes nothing from the producer.
+      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
       if ((e = cusync_conv2d_run(&a, s)) != CUSYNC_SUCCESS) return e;
       if ((!overlapped || i + 1 == n) && CUSYNC_HIP(hipEventRecord(c->ev[i + 1], s))) return CUSYNC_ERROR_DEVICE;
     }

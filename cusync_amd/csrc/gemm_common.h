@@ -45,11 +45,34 @@ struct GemmParams {
   // before everything in it has been posted, so no stale line can sit in this XCD's caches and the waits can
   // do without the cache invalidation (DynStage::lineAligned).  1 otherwise.
   uint32_t waitRound;
+  // Diagnosis (cusync_rt_set_timeline): null, or a buffer of 64-bit words, word 0 the number of records written
+  // so far, then records of eight words per finished tile (see recordTile).
+  unsigned long long* timeline;
+  uint32_t timelineCap;    // records the buffer holds
   // implicit-GEMM convolution (A is gathered from an NHWC tensor): M = n*P*Q, K = R*S*C, k = (r*S + s)*C + c
   uint32_t cvN, cvH, cvW, cvC, cvP, cvQ, cvR, cvS, cvPad, cvStride;
 };
 
 enum { kAPlain = 0, kAConv = 1 };
+
+// One record of the diagnosis timeline, written by the first thread of a workgroup when a tile is done:
+// [0] role (1 producer, 2 consumer, 3 both, 0 neither) | workgroup index << 8 | XCD id << 40
+// [1] tile x | y << 16 | z << 32 | tiles this workgroup did before << 48
+// [2..6] constant-rate 100 MHz clock: tile drawn, first loads issued (the waits of the first chunks are over),
+//        main loop done, epilogue and post done, and the clock at kernel entry of this workgroup;  [7] launched
+__device__ __forceinline__ void recordTile(const GemmParams& p, const cusync_dim3& t, uint32_t round,
+                                           unsigned long long tEntry, unsigned long long t0, unsigned long long t1,
+                                           unsigned long long t2, unsigned long long t3) {
+  if (!p.timeline) return;
+  const unsigned long long slot = __hip_atomic_fetch_add(p.timeline, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (slot >= p.timelineCap) return;
+  unsigned long long* r = p.timeline + 1 + slot * 8;
+  const uint32_t role = (p.stage.isProducer() ? 1u : 0u) | (p.stage.isConsumer() ? 2u : 0u);
+  const uint32_t xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20);       // HW_REG_XCC_ID, bits 0..3
+  r[0] = role | ((unsigned long long)cusync::DynStage::workgroupIndex() << 8) | ((unsigned long long)xcc << 40);
+  r[1] = t.x | ((unsigned long long)t.y << 16) | ((unsigned long long)t.z << 32) | ((unsigned long long)round << 48);
+  r[2] = t0; r[3] = t1; r[4] = t2; r[5] = t3; r[6] = tEntry; r[7] = p.launched;
+}
 
 // First output column of the tile whose first column of the product is n0: the SwiGLU epilogue folds pairs of
 // column groups, so its tiles are half as wide in the output, and that is what a consumer's policy sees.

@@ -197,6 +197,7 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   const uint32_t chunks = (a->K + ti->bk - 1) / ti->bk;
   p.kPerSlice = (chunks + p.splitK - 1) / p.splitK * ti->bk;
   p.mPad = s.grid.y * ti->bm;
+  cusync::rt::timeline(&p.timeline, &p.timelineCap);
   p.partials = (float*)a->workspace;
   p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
   return p;
@@ -294,6 +295,16 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
+}
+
+int cusync_gemm_fills_device(const cusync_gemm_args* a) {
+  if (!a || !tileInfo(a->tile)) return 0;
+  const int resident = residentWorkgroups(a->tile);
+  if (resident <= 0) return 0;
+  const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
+  uint32_t launched = std::min<uint32_t>(g.x * g.y * g.z, (uint32_t)resident);
+  if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
+  return launched >= (uint32_t)resident ? 1 : 0;
 }
 
 cusync_error cusync_gemm_chain_run(const cusync_gemm_args* args, int count, void* stream) {

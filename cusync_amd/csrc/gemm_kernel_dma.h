@@ -167,6 +167,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   // first tile's loads are under way; the draw of the next ticket is issued while a tile is
   // being computed and settled when the tile is done.
   uint32_t dryXcds = 0, nextRaw = 0;
+  const unsigned long long tlEntry = p.timeline ? wall_clock64() : 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
   const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
@@ -178,6 +179,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       break;
     }
     const cusync_dim3 t = stage.ticketToTile(ticket);
+    const unsigned long long tl0 = p.timeline ? wall_clock64() : 0;
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
     const uint32_t kBegin = t.z * p.kPerSlice, kEnd = min(p.K, kBegin + p.kPerSlice);
@@ -435,6 +437,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     if constexpr (C::STAGES > 4) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); issueAll(Parity<3>{}, 3); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 5, "prologue written for 2..5 stages");
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+    const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
     if constexpr (C::PIPE) {
       waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
@@ -461,6 +464,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // The loads issued for chunks past the end of K (zeros) may still be on their way into LDS, which the
     // epilogue is about to reuse.
     waitVmcnt<0>();
+    const unsigned long long tl2 = p.timeline ? wall_clock64() : 0;
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
 
@@ -469,6 +473,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     cusync_dim3 done = {m0, outputColumn(p, n0), t.z};
     if (completed && stage.isProducer()) stage.post(done, postsPerTile(p));
     else __syncthreads();
+    if (tid == 0) recordTile(p, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }
 }
 

@@ -505,14 +505,19 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
     } else if ((e = cusync_gemm_run(&a1, m->sProd)) != CUSYNC_SUCCESS) {
       return e;
     } else if (overlapped) {
-      // each wait kernel goes behind the event recorded right before its producer's launch: ahead of it, its wave
-      // would hold a CU that one of the producer's workgroups needs (see cusync_invoke_wait_kernel_after)
-      if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a wait kernel per edge
-        if ((e = cusync_invoke_wait_kernel_after(&m->prod, m->sMid, m->eStart)) != CUSYNC_SUCCESS) return e;
-        if (CUSYNC_HIP(hipEventRecord(m->eMid, m->sMid))) return CUSYNC_ERROR_DEVICE;
+      // The consumer's stream is held back until every workgroup of the producer has started.  A producer launch
+      // that takes every workgroup slot of the device is waited for here on the host (a wait kernel's wave on one
+      // of the CUs would keep the last producer workgroup off the device until another retires); for any other
+      // the reference's wait kernel goes into the consumer's stream, unordered like the reference's.
+      auto holdBack = [&](const cusync_stage_desc* prod, bool fills, hipStream_t s) {
+        return fills ? cusync_wait_producer_started(prod, 0) : cusync_invoke_wait_kernel(prod, s);
+      };
+      const bool fills1 = cusync_gemm_fills_device(&a1) != 0;
+      if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a hold-back per edge
+        if ((e = holdBack(&m->prod, fills1, m->sMid)) != CUSYNC_SUCCESS) return e;
         if ((e = runActStage(m, h, m->sMid)) != CUSYNC_SUCCESS) return e;
-        if ((e = cusync_invoke_wait_kernel_after(&m->mid, m->sCons, m->eMid)) != CUSYNC_SUCCESS) return e;
-      } else if ((e = cusync_invoke_wait_kernel_after(&m->prod, m->sCons, m->eStart)) != CUSYNC_SUCCESS) {
+        if ((e = cusync_invoke_wait_kernel(&m->mid, m->sCons)) != CUSYNC_SUCCESS) return e;
+      } else if ((e = holdBack(&m->prod, fills1, m->sCons)) != CUSYNC_SUCCESS) {
         return e;
       }
       if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;

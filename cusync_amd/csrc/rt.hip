@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <algorithm>
+#include <chrono>
 #include <string>
 #include <vector>
 
@@ -29,6 +31,11 @@ int check(hipError_t e, const char* what, const char* file, int line) {
   return (int)e;
 }
 
+static unsigned long long* g_timeline = nullptr;
+static uint32_t g_timelineCap = 0;
+void timeline(unsigned long long** buffer, uint32_t* capacity) { *buffer = g_timeline; *capacity = g_timelineCap; }
+void setTimeline(unsigned long long* buffer, uint32_t capacity) { g_timeline = buffer; g_timelineCap = capacity; }
+
 bool forceAcquire() {
   static const bool on = [] {
     const char* v = getenv("CUSYNC_FORCE_ACQUIRE");
@@ -41,9 +48,7 @@ bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t*
   uint32_t total = 0;
   for (int i = 0; i < count; i++) {
     if (!stages[i] || !stages[i]->spinTimeouts) continue;
-    uint32_t v = 0;
-    if (check(hipMemcpy(&v, stages[i]->spinTimeouts, sizeof v, hipMemcpyDeviceToHost), "hipMemcpy(spinTimeouts)", __FILE__, __LINE__)) return false;
-    total += v;
+    total += __atomic_load_n(stages[i]->spinTimeouts, __ATOMIC_ACQUIRE);     // host memory: no copy
   }
   *sum = total;
   return true;
@@ -70,12 +75,19 @@ cusync_error checkSpinTimeouts(const cusync_stage_desc* const* stages, int count
 // (src/cusync.cu:11-19) with a bounded spin.
 // A wait that gives up is counted in *timeouts (may be null), as the waits inside the kernels are.
 __global__ void cusync_wait_kernel_impl(const uint32_t* semaphore, uint32_t value, uint32_t* timeouts) {
-  if (threadIdx.x == 0 && !cusync::dev::spinUntilAtLeast(semaphore, value) && timeouts) cusync::dev::ticketAdd(timeouts, 1);
+  if (threadIdx.x == 0 && !cusync::dev::spinUntilAtLeast(semaphore, value) && timeouts) cusync::dev::countGiveUp(timeouts);
 }
 
 extern "C" {
 
 const char* cusync_rt_last_error(void) { return cusync::rt::g_last_error.c_str(); }
+
+cusync_error cusync_rt_set_timeline(void* device_buffer, size_t bytes) {
+  if (!device_buffer || bytes < 72) { cusync::rt::setTimeline(nullptr, 0); return CUSYNC_SUCCESS; }
+  if ((uintptr_t)device_buffer % 8) { cusync::rt::setError("timeline: the buffer must be 8-byte aligned"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  cusync::rt::setTimeline((unsigned long long*)device_buffer, (uint32_t)std::min<size_t>((bytes - 8) / 64, 0xffffffffu));
+  return CUSYNC_SUCCESS;
+}
 
 int cusync_rt_device_count(void) {
   int n = 0;
@@ -131,8 +143,8 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   if (n == 0) { cusync::rt::setError("cusync_stage_alloc: empty grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr; d->xcdTickets = nullptr;
   d->kernelExecuted = nullptr; d->spinTimeouts = nullptr; d->tileStatusWrite = nullptr;
-  // The small counters share one allocation: [tileCounter, startCounter, spinTimeouts, kernelExecuted,
-  // xcdTickets[9]], each on its own 128-byte line so that polling one does not disturb the others.
+  // The small device counters share one allocation: [tileCounter, startCounter, -, kernelExecuted, xcdTickets[9]], each on its
+  // own 128-byte line so that polling one does not disturb the others.
   const size_t line = 128;
   char* counters = nullptr;
   if (RT(hipMalloc((void**)&counters, 13 * line))) return CUSYNC_ERROR_DEVICE;
@@ -146,8 +158,15 @@ cusync_error cusync_stage_alloc(cusync_stage_desc* d, const cusync_dim3* host_ti
   };
   if (RT(hipMemset(counters, 0, 13 * line))) return fail();
   d->startCounter = (uint32_t*)(counters + line);
-  d->spinTimeouts = (uint32_t*)(counters + 2 * line);
   d->xcdTickets = (uint32_t*)(counters + 4 * line);
+  // The two words the host wants to look at while kernels run, or without a copy after them, live in pinned host
+  // memory the device reaches over the bus: the count of waits that gave up (first line: the base of the block)
+  // and a mirror of the wait-kernel flag (second line, CUSYNC_HOST_FLAG_OFFSET words on).  Each is written at most
+  // once per kernel; the flag the wait kernel polls stays in device memory.
+  char* shared = nullptr;
+  if (RT(hipHostMalloc((void**)&shared, 2 * line, hipHostMallocDefault))) return fail();
+  memset(shared, 0, 2 * line);
+  d->spinTimeouts = (uint32_t*)shared;
   const bool producer = d->out.kind != CUSYNC_POLICY_NOSYNC;
   if (producer && !(d->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) d->kernelExecuted = (uint32_t*)(counters + 3 * line);
   bool identity = true;
@@ -169,6 +188,7 @@ cusync_error cusync_stage_free(cusync_stage_desc* d) {
   if (!d) return CUSYNC_ERROR_NOT_INITIALIZED;
   int bad = 0;
   if (d->tileCounter) bad |= RT(hipFree(d->tileCounter));       // base of the counters block
+  if (d->spinTimeouts) bad |= RT(hipHostFree(d->spinTimeouts));  // base of the block in host memory
   if (d->tileOrder) bad |= RT(hipFree(d->tileOrder));
   if (d->tileStatusWrite) bad |= RT(hipFree(d->tileStatusWrite));
   d->tileOrder = nullptr; d->tileCounter = nullptr; d->startCounter = nullptr; d->xcdTickets = nullptr;
@@ -226,36 +246,29 @@ cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc* prod, void* stre
   return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
-// True when the stream can be held back by the command processor itself (hipStreamWaitValue32) and the
-// environment does not ask for the wait kernel (CUSYNC_WAIT_KERNEL set to something other than 0).
-static bool queueWaitAvailable() {
-  static const bool ok = [] {
-    const char* v = getenv("CUSYNC_WAIT_KERNEL");
-    if (v && *v && strcmp(v, "0") != 0) return false;
-    int dev = 0, can = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return false;
-    if (hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, dev) != hipSuccess) return false;
-    return can != 0;
-  }();
-  return ok;
-}
-
 cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void* stream, void* launch_event) {
   if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
   if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
   if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
-  if (!prod->kernelExecuted) return CUSYNC_ERROR_NOT_INITIALIZED;
-  if (queueWaitAvailable()) {
-    // The command processor polls the flag: no wave sits on a CU, so the wait cannot take a slot from the
-    // producer's workgroups wherever it lands relative to their dispatch, and no launch event is needed.
-    // The producer's flag store is an agent-scope release, which writes through to memory where the
-    // command processor reads.
-    if (RT(hipStreamWaitValue32((hipStream_t)stream, prod->kernelExecuted, (uint32_t)prod->iter, hipStreamWaitValueGte, 0xffffffffu)))
-      return CUSYNC_ERROR_DEVICE;
-    return CUSYNC_SUCCESS;
-  }
   if (launch_event && RT(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)launch_event, 0))) return CUSYNC_ERROR_DEVICE;
   return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
+}
+
+cusync_error cusync_wait_producer_started(const cusync_stage_desc* prod, uint32_t timeout_ms) {
+  if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
+  if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
+  if (!prod->kernelExecuted) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const auto t0 = std::chrono::steady_clock::now();
+  const uint32_t want = (uint32_t)prod->iter;
+  for (uint32_t spins = 0;; spins++) {
+    if (__atomic_load_n(prod->spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, __ATOMIC_ACQUIRE) >= want) return CUSYNC_SUCCESS;
+    if ((spins & 1023u) == 1023u &&
+        std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(timeout_ms ? timeout_ms : 2000)) {
+      cusync::rt::setError("cusync_wait_producer_started: the producer's workgroups did not all start in time");
+      return CUSYNC_ERROR_DEVICE;
+    }
+  }
 }
 
 cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems, cusync_dim3* tile_order,
@@ -279,10 +292,15 @@ cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems,
     *tile_counter = sum;
   }
   if (start_counter) bad |= RT(hipMemcpy(start_counter, d->startCounter, 4, hipMemcpyDeviceToHost));
-  if (spin_timeouts) bad |= RT(hipMemcpy(spin_timeouts, d->spinTimeouts, 4, hipMemcpyDeviceToHost));
-  if (kernel_executed) {
+  if (spin_timeouts) *spin_timeouts = d->spinTimeouts ? __atomic_load_n(d->spinTimeouts, __ATOMIC_ACQUIRE) : 0;
+  if (kernel_executed) {       // the flag's mirror in host memory, which the producer writes right after the flag
     *kernel_executed = 0;
-    if (d->kernelExecuted) bad |= RT(hipMemcpy(kernel_executed, d->kernelExecuted, 4, hipMemcpyDeviceToHost));
+    if (d->kernelExecuted) {
+      uint32_t dev = 0;
+      bad |= RT(hipMemcpy(&dev, d->kernelExecuted, 4, hipMemcpyDeviceToHost));
+      const uint32_t host = __atomic_load_n(d->spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, __ATOMIC_ACQUIRE);
+      *kernel_executed = dev == host ? dev : 0xffffffffu;     // the two must agree once the device is idle
+    }
   }
   return bad ? CUSYNC_ERROR_DEVICE : CUSYNC_SUCCESS;
 }

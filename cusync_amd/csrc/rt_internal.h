@@ -22,6 +22,9 @@ bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t*
 // For the chain handles, after the host has synchronised with a run: CUSYNC_SUCCESS if the sum above still
 // equals *seen, else records a message naming `what`, brings *seen up to date and returns CUSYNC_ERROR_DEVICE
 // (the chain went on with data its producer had not posted: the outputs of that run are not valid).
+// The diagnosis buffer set with cusync_rt_set_timeline (null when off) and the records it holds.
+void timeline(unsigned long long** buffer, uint32_t* capacity);
+void setTimeline(unsigned long long* buffer, uint32_t capacity);
 cusync_error checkSpinTimeouts(const cusync_stage_desc* const* stages, int count, uint32_t* seen, const char* what);
 }  // namespace rt
 }  // namespace cusync

@@ -116,6 +116,7 @@ struct DynStage {
     if (token == launched - 1) {
       dev::storeRelaxed(d.startCounter, 0);
       dev::releaseStore(d.kernelExecuted, (uint32_t)d.iter);
+      dev::releaseStoreSystem(d.spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, (uint32_t)d.iter);     // mirror for a host that holds the consumer back itself
     }
   }
 
@@ -197,7 +198,7 @@ struct DynStage {
     const bool ok = lineAligned ? dev::spinUntilAtLeastNoInvalidate(&d.tileStatusRead[idx], waitTarget())
                                 : dev::spinUntilAtLeast(&d.tileStatusRead[idx], waitTarget());
     if (!ok && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0)
-      dev::ticketAdd(d.spinTimeouts, 1);
+      dev::countGiveUp(d.spinTimeouts);
   }
 
   // Wave-uniform wait for every tile {r, col, z} whose rows meet rowLo..rowHi (row blocks of tileM rows):
@@ -225,7 +226,7 @@ struct DynStage {
     }
     if (lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     else dev::acquireFence();
-    if (timedOut && lane == 0) dev::ticketAdd(d.spinTimeouts, 1);
+    if (timedOut && lane == 0) dev::countGiveUp(d.spinTimeouts);
   }
 
   // Wave-uniform wait for tile {row, col, 0} that looks ahead: the first poll reads, one per lane, the

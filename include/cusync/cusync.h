@@ -233,6 +233,11 @@ public:
   // Declares `tile` complete.  Contains a workgroup barrier, so every thread of
   // the workgroup must call it after its last store to the tile.
   CUSYNC_DEVICE CuSyncError post(const dim3& tile, uint32_t postThread = 0);
+  // The wait-kernel flag and, for a host that holds the consumer back itself, its mirror in host memory.
+  CUSYNC_DEVICE void raiseFlag() {
+    dev::releaseStore(kernelExecuted_, (uint32_t)iter);
+    dev::releaseStoreSystem(spinTimeouts_ + CUSYNC_HOST_FLAG_OFFSET, (uint32_t)iter);
+  }
 
   // First statement of a sync-aware kernel: returns the tile this workgroup
   // processes (a ticket through the tile order, or blockIdx with
@@ -268,7 +273,7 @@ CUSTAGE_METHOD(CuSyncError) wait(dim3& tile, uint32_t waitingThread, bool callSy
   if (flat == waitingThread) {
     const uint32_t need = (uint32_t)iter * inputPolicy_.waitValue(tile, prodGrid_);
     const uint32_t idx = inputPolicy_.tileIndex(tile, prodGrid_);
-    if (!dev::spinUntilAtLeast(&tileStatusRead_[idx * CUSYNC_SEM_STRIDE], need)) dev::ticketAdd(spinTimeouts_, 1);
+    if (!dev::spinUntilAtLeast(&tileStatusRead_[idx * CUSYNC_SEM_STRIDE], need)) dev::countGiveUp(spinTimeouts_);
   }
   if (callSync) __syncthreads();
   return CuSyncSuccess;
@@ -296,7 +301,7 @@ CUSTAGE_METHOD(dim3) tile(dim3* shared_storage) {
     // Hardware order.  Only the first block can speak for the kernel being on
     // the device; the caller vouches that the rest fits beside its consumer.
     if (raisesFlag && leader && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)
-      dev::releaseStore(kernelExecuted_, (uint32_t)iter);
+      raiseFlag();
     return dim3(blockIdx.x, blockIdx.y, blockIdx.z);
   }
   if (leader) {
@@ -306,7 +311,7 @@ CUSTAGE_METHOD(dim3) tile(dim3* shared_storage) {
       // can be kept off the device by a spinning consumer.  Re-arm the
       // dispenser and let the consumer's stream go.
       dev::storeRelaxed(tileCounter, 0);
-      if (raisesFlag) dev::releaseStore(kernelExecuted_, (uint32_t)iter);
+      if (raisesFlag) raiseFlag();
     }
     *shared_storage = tileOrder[ticket];
   }

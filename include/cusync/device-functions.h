@@ -103,6 +103,15 @@ CUSYNC_DEVICE void releaseStore(volatile uint32_t* addr, uint32_t value) {
   __hip_atomic_store((uint32_t*)addr, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The wait-kernel flag and the count of waits that gave up live in host memory that the device can reach, so that
+// the host reads them without a copy: they are written at system scope.
+CUSYNC_DEVICE void releaseStoreSystem(volatile uint32_t* addr, uint32_t value) {
+  __hip_atomic_store((uint32_t*)addr, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+CUSYNC_DEVICE void countGiveUp(uint32_t* addr) {
+  __hip_atomic_fetch_add(addr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 CUSYNC_DEVICE uint32_t ticketAdd(uint32_t* addr, uint32_t value) {
   return __hip_atomic_fetch_add(addr, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

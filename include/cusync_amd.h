@@ -80,6 +80,7 @@ enum { CUSYNC_STAGE_IDENTITY_ORDER = 1 };
  * waves polling one semaphore do not queue up behind those polling its neighbours (the reference packs them,
  * CS/cusync.h:186-190).  cusync_stage_read_state returns them packed. */
 #define CUSYNC_SEM_STRIDE 32
+#define CUSYNC_HOST_FLAG_OFFSET 32
 
 typedef struct cusync_stage_desc {
   cusync_dim3 grid;           /* grid_     : logical tile grid of this stage */
@@ -97,7 +98,10 @@ typedef struct cusync_stage_desc {
   uint32_t *xcdTickets;       /* 9 counters, 128 bytes apart: one ticket dispenser per XCD for the prebuilt
                                  kernels plus a count of workgroups that ran dry; all 0 between runs */
   uint32_t *kernelExecuted;   /* wait-kernel flag: == iter once every workgroup of the run has begun */
-  uint32_t *spinTimeouts;     /* number of waits of this stage that gave up (0 in a healthy chain) */
+  uint32_t *spinTimeouts;     /* number of waits of this stage that gave up, 0 in a healthy chain.  Pinned host memory
+                                 that the device writes to, so that the host reads it without a copy; the word
+                                 CUSYNC_HOST_FLAG_OFFSET words behind it mirrors the wait-kernel flag for
+                                 cusync_wait_producer_started (written right after the flag itself) */
   uint32_t *tileStatusWrite;  /* semaphores this stage posts, CUSYNC_SEM_STRIDE apart */
   uint32_t *tileStatusRead;   /* semaphores this stage waits on (its producer's) */
 } cusync_stage_desc;
@@ -108,6 +112,12 @@ typedef struct cusync_stage_desc {
 /* ------------------------------------------------------------------------- */
 
 const char *cusync_rt_last_error(void);            /* text of the last failed HIP call, "" if none */
+/* Diagnosis, off by default.  With a device buffer set (8-byte aligned, zeroed by the caller) the direct-to-LDS GEMM
+ * kernels append one record of eight 64-bit words per finished tile behind a record count in word 0: role and
+ * workgroup and XCD, tile, and the 100 MHz clock at five points of the tile (drawn, first loads issued, main loop
+ * done, posted, kernel entry).  This is how the per-workgroup timelines in profiles/ were taken.  NULL switches it
+ * off again; when off the kernels pay one test per tile.  No counterpart in the reference. */
+cusync_error cusync_rt_set_timeline(void *device_buffer, size_t bytes);
 int cusync_rt_device_count(void);
 int cusync_rt_device_info(int *num_cus, int *clock_khz, size_t *lds_per_cu, size_t *hbm_bytes,
                           char *name, size_t name_len);
@@ -153,20 +163,23 @@ cusync_error cusync_set_producer_consumer_pair(const cusync_stage_desc *prod, cu
  * enqueues a one-wave kernel on `stream` that returns once the producer's flag
  * has reached desc->iter.  No-op with AVOID_WAIT_KERNEL. */
 cusync_error cusync_invoke_wait_kernel(const cusync_stage_desc *prod, void *stream);
-/* What the chains of this library call in place of invokeWaitKernel.  Where the device can hold a stream back
- * on a memory value by itself (hipStreamWaitValue32; every MI355X) no kernel is launched at all: the command
- * processor polls the producer's flag and releases `stream` when it has reached desc->iter.  A wait kernel is a
- * wave that holds registers on one CU until the flag rises; it runs in another hardware queue than the producer
- * and can reach the GPU first, and a producer whose workgroups need whole CUs and fill the machine then cannot
- * place its last workgroup, the flag is not raised until another workgroup retires, and that run of the chain is
- * one producer tile longer (seen as a second mode in the step times, 700-790 us against 610).  The queue-side
- * wait holds no CU.  It has no give-up: only call it for a producer that has been, or is about to be, launched.
- * With CUSYNC_WAIT_KERNEL=1 in the environment, or on a device without the queue-side wait, the wait kernel is
- * launched instead, behind `launch_event` (a hipEvent_t the caller recorded on the producer's stream immediately
- * before launching the producer's kernel; NULL = no ordering), which keeps its wave behind the producer's
- * dispatch in all but rare cases.  No counterpart in the reference, which launches the wait kernel unordered
- * (src/ml-bench/transformer/mlp.cu:683-699). */
+/* Same, but `stream` first waits for `launch_event` (a hipEvent_t the caller recorded on the producer's stream
+ * immediately before launching the producer's kernel; NULL = no ordering, i.e. cusync_invoke_wait_kernel).  The two
+ * streams are separate hardware queues and the wait kernel's wave can reach the GPU before the producer's
+ * workgroups do; behind the event it is dispatched after the producer's launch has begun.  No counterpart in the
+ * reference, which launches the wait kernel unordered (src/ml-bench/transformer/mlp.cu:683-699). */
 cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc *prod, void *stream, void *launch_event);
+/* The same hold-back done by the calling host thread instead of a kernel: returns once every workgroup of the
+ * producer's run prod->iter has started (the mirror of its flag in host memory, which the device writes to, has
+ * reached prod->iter), or CUSYNC_ERROR_DEVICE after timeout_ms (0 = two seconds).  The caller then launches the consumer.
+ * Why: a wait kernel is a wave that holds registers on one CU until the flag rises (hipStreamWaitValue32 is such a
+ * kernel too on this runtime).  A producer whose workgroups need whole CUs and whose launch fills every CU cannot
+ * place its last workgroup on that CU; the flag is then not raised until another workgroup retires and the chain
+ * is one producer tile longer (measured on the 2048-row GPT-3 MLP: 720-790 us against 610 in one run out of ten;
+ * per-workgroup timestamps show workgroup 249 of 256 entering at 313 us).  The host holds no CU.  The chain
+ * handles of this library use it for exactly those producers and the wait kernel for all others.  No counterpart
+ * in the reference. */
+cusync_error cusync_wait_producer_started(const cusync_stage_desc *prod, uint32_t timeout_ms);
 /* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
 cusync_error cusync_wait_kernel(uint32_t *semaphore, uint32_t value, void *stream);
 /* Reads back device state for tests (the reference reaches it through the
@@ -258,6 +271,11 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args *args);
 size_t cusync_gemm_workspace_size(const cusync_gemm_args *args);
 /* Workgroups of this tile shape that stay resident on the device at once. */
 int cusync_gemm_max_resident(int tile);
+/* 1 when the launch of these arguments takes every workgroup slot the device has for its kernel (as many
+ * workgroups as stay resident).  A single wave of another kernel that gets onto a CU first, a wait kernel for
+ * instance, then keeps one of the workgroups off the device until another retires; the chains hold such a
+ * producer's consumer back from the host instead (cusync_wait_producer_started).  No counterpart in the reference. */
+int cusync_gemm_fills_device(const cusync_gemm_args *args);
 /* run(stream) (cusyncgemm.h:525-563).  args->stage.iter selects the run. */
 cusync_error cusync_gemm_run(const cusync_gemm_args *args, void *stream);
 /* cusync_gemm_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving

@@ -149,7 +149,7 @@ def test_gemm_can_implement_rejects():
     prod.destroy()
 
 
-def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1), ordered=False, c_offset=0):
+def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=10, split=(1, 1), ordered=False, c_offset=0, host_hold=False):
     """C = A*B on one stream, E = C*D on another, synchronised per `policy_kind`.  `ordered`: the wait kernel
     goes behind an event recorded on the producer's stream right before the producer's launch.  `c_offset`:
     C starts that many halfs into its allocation (a base that is 16-byte but not 128-byte aligned)."""
@@ -189,7 +189,10 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
             assert L.cusync_rt_event_record(ev, s1) == 0
         assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1, stream=s1,
                         max_workgroups=max_wg, split_k=split[0], workspace=ws[0].data_ptr()) == api.ERR.SUCCESS, api.last_error()
-        assert prod.invokeWaitKernel(s2, after=ev if ordered else None) == api.ERR.SUCCESS
+        if host_hold:      # the host waits until every producer workgroup has started, then launches the consumer
+            assert L.cusync_wait_producer_started(C.byref(prod.desc), 0) == api.ERR.SUCCESS, api.last_error()
+        else:
+            assert prod.invokeWaitKernel(s2, after=ev if ordered else None) == api.ERR.SUCCESS
         assert api.gemm(cons, M, N, N, dc.data_ptr(), N, dd.data_ptr(), N, de.data_ptr(), N, tile2, stream=s2,
                         max_workgroups=max_wg, split_k=split[1], workspace=ws[1].data_ptr()) == api.ERR.SUCCESS, api.last_error()
         assert L.cusync_rt_device_sync() == 0, api.last_error()
@@ -299,6 +302,25 @@ def test_chained_gemms_unaligned_intermediate(policy_kind, tiles, N, c_offset):
     assert_close(e, orc.gemm(c, d), "E")
     assert cs.spin_timeouts == 0
     assert np.array_equal(ps.sems, want_sems)
+
+
+@pytest.mark.parametrize("policy_kind", ["tile", "row"])
+def test_chained_gemms_consumer_held_back_by_the_host(policy_kind):
+    # cusync_wait_producer_started instead of a wait kernel: what the chain handles do when the producer's launch
+    # takes every workgroup slot of the device (2 x 128 tiles of 256x192 here: one per CU)
+    print("chained, host-side hold", policy_kind, flush=True)
+    M, N, K = 2048, 6144, 256
+    tile = api.TILE.T256x192x32
+    L = _lib.load()
+    a, b, d, c, e, ps, cs, want_sems = chained(M, N, K, tile, tile, policy_kind, iters=3, host_hold=True)
+    rows = [0, 255, 256, 1000, 2047]
+    assert_close(c[rows], orc.gemm(np.ascontiguousarray(a[rows]), b), "C rows")
+    assert_close(e[rows], orc.gemm(np.ascontiguousarray(c[rows]), d), "E rows")
+    assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3
+    # a stage whose producer never ran: the host-side wait gives up after its time-out, nothing hangs
+    st = api.Stage((2, 2, 1), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128))
+    assert L.cusync_wait_producer_started(C.byref(st.desc), 50) == api.ERR.DEVICE and "did not all start" in api.last_error()
+    st.destroy()
 
 
 def test_wait_kernel_that_gives_up_is_counted():

@@ -266,9 +266,8 @@ def test_mlp_run_reports_waits_that_gave_up():
     torch.cuda.synchronize()
     mlp = api.Mlp(api.MODEL.GPT3, batch, GPT3["hidden"], GPT3["inner"], api.SYNC.ROW, dw1.data_ptr(), dw2.data_ptr())
     mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
-    three = C.c_uint32(3)
     cons = L.cusync_mlp_stage(mlp.h, 1).contents
-    assert L.cusync_rt_memcpy_h2d(cons.spinTimeouts, C.addressof(three), 4) == 0
+    C.c_uint32.from_address(cons.spinTimeouts).value = 3          # the counter lives in pinned host memory
     with pytest.raises(api.CuSyncError) as err:
         mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)
     assert err.value.code == api.ERR.DEVICE and "3 wait(s) gave up" in str(err.value)
