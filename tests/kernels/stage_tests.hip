@@ -13,6 +13,8 @@
 #include <vector>
 
 #include <cusync/cusync.h>
+#include <cusync/gemm.h>
+#include <type_traits>
 
 #define HIP_OK(cmd) do { hipError_t e_ = (cmd); if (e_ != hipSuccess) { \
   printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); return -1; } } while (0)
@@ -207,6 +209,168 @@ int run_error_paths(int* out) {
   P empty;
   out[4] = CuSync::setProducerConsumerPair(empty, cons);
   prod.destroy(); cons.destroy();
+  return 0;
+}
+
+// ---- the GPT-3 MLP loop of the reference's driver, on the launcher objects ------------------------------------
+// Written after runCuSyncGPT3 (src/ml-bench/transformer/mlp.cu:645-716): Arguments{stage, size, refs, {alpha, beta},
+// split_k}, get_workspace_size, can_implement, initialize, and per run  gemm_op1.run(true, NULL, producer_stream),
+// prod.invokeWaitKernel(consumer_stream), gemm_op2.run(true, NULL, consumer_stream), then incrementIter on the
+// stages and on the launchers' params_.custage.  policy 0: TileSync + NoAtomicAdd (mlp.cu:9-16, 111), 1: RowSync.
+// x [M][K1], w1 [K1][N1], h [M][N1], w2 [N1][N2], y [M][N2]: fp16 device pointers.
+// out[0] sum of every Status / CuSyncError that was not success (0 = all good)  out[1] spin time-outs
+// out[2] producer's wait-kernel flag after the last run  out[3] semaphore mismatches against iters (TileSync) or iters * gN (RowSync)
+}  // extern "C"
+
+constexpr int kLauncherTile = CUSYNC_TILE_128x128x32;
+using LTileSync = TileSync<TransposeXYOrder, 128, 128>;
+using LRowSync = RowSync<128>;
+
+template<typename Sync, int Opts>
+static int launcherChainImpl(Sync sync, uint32_t M, uint32_t K1, uint32_t N1, uint32_t N2, const void* x, const void* w1, void* h,
+                             const void* w2, void* y, int splitK1, int iters, int* out) {
+  using ProdCuStage = CuStage<TransposeXYOrder, NoSync, Sync, Opts>;
+  using ConsCuStage = CuStage<TransposeXYOrder, Sync, NoSync, Opts>;
+  using Gemm1 = CuSyncGemm<ProdCuStage, kLauncherTile, CUSYNC_EPILOGUE_GELU>;
+  using Gemm2 = CuSyncGemm<ConsCuStage, kLauncherTile, CUSYNC_EPILOGUE_NONE>;
+  int bad = 0;
+  const GemmCoord size1((int)M, (int)N1, (int)K1), size2((int)M, (int)N2, (int)N1);
+  const dim3 gridDim1 = Gemm1::get_grid_shape(size1, splitK1), gridDim2 = Gemm2::get_grid_shape(size2, 1);
+  ProdCuStage prod(gridDim1, dim3(1, 1, 1), NoSync(), sync);
+  ConsCuStage cons(gridDim2, dim3(1, 1, 1), sync, NoSync());
+  bad += CuSync::setProducerConsumerPair(prod, cons) != CuSyncSuccess;
+
+  hipStream_t producer_stream, consumer_stream;
+  HIP_OK(hipStreamCreateWithFlags(&producer_stream, hipStreamNonBlocking));
+  HIP_OK(hipStreamCreateWithFlags(&consumer_stream, hipStreamNonBlocking));
+
+  typename Gemm1::Arguments args1{prod, size1, {(const half_bits*)x, (int)K1}, {(const half_bits*)w1, (int)N1},
+                                  {(const half_bits*)h, (int)N1}, {(half_bits*)h, (int)N1}, {1.0f, 0.0f}, splitK1};
+  Gemm1 gemm_op1;
+  size_t workspace_size = Gemm1::get_workspace_size(args1);
+  void* workspace1 = nullptr;
+  if (workspace_size) HIP_OK(hipMalloc(&workspace1, workspace_size));
+  bad += gemm_op1.can_implement(args1) != Status::kSuccess;
+  bad += gemm_op1.initialize(args1, workspace1) != Status::kSuccess;
+
+  typename Gemm2::Arguments args2{cons, size2, {(const half_bits*)h, (int)N1}, {(const half_bits*)w2, (int)N2},
+                                  {(const half_bits*)y, (int)N2}, {(half_bits*)y, (int)N2}, {1.0f, 0.0f}, 1};
+  Gemm2 gemm_op2;
+  bad += Gemm2::get_workspace_size(args2) != 0;
+  bad += gemm_op2.can_implement(args2) != Status::kSuccess;
+  bad += gemm_op2.initialize(args2, nullptr) != Status::kSuccess;
+  // what the launcher refuses: a beta term, and k-slices without a workspace
+  typename Gemm2::Arguments withBeta = args2;
+  withBeta.epilogue = {1.0f, 1.0f};
+  bad += Gemm2::can_implement(withBeta) != Status::kErrorNotSupported;
+  typename Gemm1::Arguments sliced = args1;
+  sliced.split_k_slices = 2;
+  { Gemm1 tmp; bad += tmp.initialize(sliced, nullptr) != Status::kErrorWorkspaceNull; }
+
+  hipEvent_t start, end;
+  HIP_OK(hipEventCreate(&start)); HIP_OK(hipEventCreate(&end));
+  for (int r = 0; r < iters; r++) {
+    HIP_OK(hipEventRecord(start, producer_stream));
+    bad += gemm_op1.run(true, NULL, producer_stream) != Status::kSuccess;
+    bad += prod.invokeWaitKernel(consumer_stream) != CuSyncSuccess;
+    bad += gemm_op2.run(true, NULL, consumer_stream) != Status::kSuccess;
+    HIP_OK(hipEventRecord(end, consumer_stream));
+    HIP_OK(hipEventSynchronize(end));
+    HIP_OK(hipStreamSynchronize(producer_stream));
+    prod.incrementIter();
+    cons.incrementIter();
+    gemm_op2.params_.custage.incrementIter();
+    gemm_op1.params_.custage.incrementIter();
+  }
+  out[0] = bad;
+  const cusync_stage_desc pd = prod.desc(), cd = cons.desc();
+  const uint32_t tiles = gridDim1.x * gridDim1.y * gridDim1.z;
+  std::vector<uint32_t> sems(tiles);
+  uint32_t flag = 0, timeouts = 0;
+  if (cusync_stage_read_state(&pd, sems.data(), nullptr, nullptr, nullptr, &flag, nullptr) != CUSYNC_SUCCESS) return -1;
+  if (cusync_stage_read_state(&cd, nullptr, nullptr, nullptr, nullptr, nullptr, &timeouts) != CUSYNC_SUCCESS) return -1;
+  out[1] = (int)timeouts;
+  out[2] = (int)flag;
+  int mismatches = 0;
+  const bool rows = std::is_same<Sync, LRowSync>::value;
+  for (uint32_t i = 0; i < tiles; i++) {
+    const uint32_t want = rows ? (i < gridDim1.y ? (uint32_t)iters * gridDim1.x : 0u) : (i < gridDim1.x * gridDim1.y ? (uint32_t)iters : 0u);
+    mismatches += sems[i] != want;
+  }
+  out[3] = mismatches;
+  prod.destroy(); cons.destroy();
+  if (workspace1) HIP_OK(hipFree(workspace1));
+  HIP_OK(hipEventDestroy(start)); HIP_OK(hipEventDestroy(end));
+  HIP_OK(hipStreamDestroy(producer_stream)); HIP_OK(hipStreamDestroy(consumer_stream));
+  return 0;
+}
+
+extern "C" {
+
+int run_launcher_mlp(int policy, uint32_t M, uint32_t K1, uint32_t N1, uint32_t N2, const void* x, const void* w1, void* h,
+                     const void* w2, void* y, int splitK1, int iters, int* out) {
+  if (policy == 0) {
+    LTileSync sync;
+    return launcherChainImpl<LTileSync, NoAtomicAdd | ReorderTileLoads>(sync, M, K1, N1, N2, x, w1, h, w2, y, splitK1, iters, out);
+  }
+  const dim3 g1 = CuSyncGemm<CuStage<TransposeXYOrder, NoSync, LRowSync>, kLauncherTile>::get_grid_shape(GemmCoord((int)M, (int)N1, (int)K1), splitK1);
+  LRowSync sync(g1.x);
+  return launcherChainImpl<LRowSync, NoOptimization>(sync, M, K1, N1, N2, x, w1, h, w2, y, splitK1, iters, out);
+}
+
+// ---- the ResNet pair on the convolution launcher (src/ml-bench/volta_conv2d/resnet.cu:107-116, 704-744) -------------
+// x [N][H][W][C], w1 and w2 [C][3][3][C], y1 and y2 [N][H][W][C].  out as above (semaphores: TileSync, all == iters).
+int run_launcher_conv_pair(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const void* x, const void* w1, void* y1, const void* w2, void* y2,
+                           int iters, int* out) {
+  constexpr int kTile = CUSYNC_CONV_TILE_128x64x32;
+  using Sync1 = TileSync<TransposeXYOrder, 128, 64>;
+  using Sync2 = Conv2DTileSync<TransposeXYOrder, 3, 3, 128, 64>;
+  using ProdCuStage = CuStage<TransposeXYOrder, NoSync, Sync1>;
+  using ConsCuStage = CuStage<TransposeXYOrder, Sync2, NoSync>;
+  using Conv1 = CuSyncImplicitGemmConvolution<ProdCuStage, kTile, CUSYNC_EPILOGUE_RELU>;
+  using Conv2 = CuSyncImplicitGemmConvolution<ConsCuStage, kTile, CUSYNC_EPILOGUE_NONE>;
+  int bad = 0;
+  const Conv2dProblemSize problem((int)N, (int)H, (int)W, (int)C, (int)C, 3, 3, 1, 1);
+  const dim3 grid = Conv1::get_grid_shape(problem);
+  Sync1 sync1;
+  Sync2 sync2;
+  ProdCuStage prod(grid, dim3(1, 1, 1), NoSync(), sync1);
+  ConsCuStage cons(grid, dim3(1, 1, 1), sync2, NoSync());
+  bad += CuSync::setProducerConsumerPair(prod, cons) != CuSyncSuccess;
+  hipStream_t s1, s2;
+  HIP_OK(hipStreamCreateWithFlags(&s1, hipStreamNonBlocking));
+  HIP_OK(hipStreamCreateWithFlags(&s2, hipStreamNonBlocking));
+  typename Conv1::Arguments args1(prod, problem, {(const half_bits*)x, (int)C}, {(const half_bits*)w1, (int)C}, {(const half_bits*)y1, (int)C}, {(half_bits*)y1, (int)C});
+  typename Conv2::Arguments args2(cons, problem, {(const half_bits*)y1, (int)C}, {(const half_bits*)w2, (int)C}, {(const half_bits*)y2, (int)C}, {(half_bits*)y2, (int)C});
+  Conv1 conv1;
+  Conv2 conv2;
+  bad += Conv1::can_implement(args1) != Status::kSuccess;
+  bad += conv1.initialize(args1) != Status::kSuccess;
+  bad += conv2.initialize(args2) != Status::kSuccess;
+  for (int r = 0; r < iters; r++) {
+    bad += conv1.run(true, NULL, s1) != Status::kSuccess;
+    bad += prod.invokeWaitKernel(s2) != CuSyncSuccess;
+    bad += conv2.run(true, NULL, s2) != Status::kSuccess;
+    HIP_OK(hipDeviceSynchronize());
+    prod.incrementIter();
+    cons.incrementIter();
+    conv1.params_.custage.incrementIter();
+    conv2.params_.custage.incrementIter();
+  }
+  out[0] = bad;
+  const cusync_stage_desc pd = prod.desc(), cd = cons.desc();
+  const uint32_t tiles = grid.x * grid.y * grid.z;
+  std::vector<uint32_t> sems(tiles);
+  uint32_t flag = 0, timeouts = 0;
+  if (cusync_stage_read_state(&pd, sems.data(), nullptr, nullptr, nullptr, &flag, nullptr) != CUSYNC_SUCCESS) return -1;
+  if (cusync_stage_read_state(&cd, nullptr, nullptr, nullptr, nullptr, nullptr, &timeouts) != CUSYNC_SUCCESS) return -1;
+  out[1] = (int)timeouts;
+  out[2] = (int)flag;
+  int mismatches = 0;
+  for (uint32_t i = 0; i < tiles; i++) mismatches += sems[i] != (uint32_t)iters;
+  out[3] = mismatches;
+  prod.destroy(); cons.destroy();
+  HIP_OK(hipStreamDestroy(s1)); HIP_OK(hipStreamDestroy(s2));
   return 0;
 }
 

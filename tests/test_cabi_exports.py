@@ -93,6 +93,7 @@ def test_host_headers_compile_without_hipcc(tmp_path):
     src.write_text(r'''
 #include <cusync/cusync.h>
 #include <cusync/wait-kernel.h>
+#include <cusync/gemm.h>
 using namespace cusync;
 using Sync = TileSync<TransposeXYOrder, 256, 128>;
 using Prod = CuStage<TransposeXYOrder, NoSync, Sync, NoAtomicAdd | ReorderTileLoads>;
@@ -107,6 +108,17 @@ int main() {
   if (st.tileIndex(dim3(256, 30 * 128, 0), dim3(44, 4, 1)) != 8 + 44) return 3;
   if (CuSyncSuccess != 5 || CuSyncErrorNotProducer != 0) return 4;
   Cons* c = nullptr; (void)c;
+  // the launcher objects are host code over the C ABI: they compile without hipcc, and the parts that need no GPU work
+  typedef CuSyncGemm<Prod, CUSYNC_TILE_256x128x32, CUSYNC_EPILOGUE_GELU> Gemm1;
+  const dim3 g = Gemm1::get_grid_shape(GemmCoord(2048, 6144, 12288), 2);
+  if (g.x != 48 || g.y != 8 || g.z != 2) return 5;
+  Gemm1::Arguments args;
+  args.problem_size = GemmCoord(2048, 6144, 12288);
+  args.split_k_slices = 2;
+  if (Gemm1::get_workspace_size(args) != (size_t)2 * 8 * 48 * 256 * 128 * 4 + 8 * 48 * 4) return 6;
+  typedef CuSyncImplicitGemmConvolution<Cons, CUSYNC_CONV_TILE_128x64x32> Conv;
+  const dim3 cg = Conv::get_grid_shape(Conv2dProblemSize(32, 56, 56, 64, 64));
+  if (cg.x != 1 || cg.y != 32 * 56 * 56 / 128 || cg.z != 1) return 7;
   return 0;
 }
 ''')

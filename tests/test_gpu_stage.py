@@ -122,3 +122,55 @@ def test_stage_state_after_create():
     assert api.set_producer_consumer_pair(c, s) == api.ERR.NOT_PRODUCER
     assert c.invokeWaitKernel(None) == api.ERR.NOT_PRODUCER     # rejected on the host, nothing is enqueued
     s.destroy(); c.destroy()
+
+
+@pytest.mark.parametrize("policy,split_k1", [(0, 1), (1, 1), (0, 2), (1, 4)])
+def test_mlp_loop_on_the_launcher_objects(policy, split_k1):
+    """The reference's runCuSyncGPT3 loop (TB/mlp.cu:645-716), written on cusync::CuSyncGemm (include/cusync/gemm.h):
+    Arguments -> get_workspace_size -> can_implement -> initialize, then run(true, NULL, stream) per iteration with
+    incrementIter on the stages and on params_.custage.  H is refilled with NaN before the call; the outputs are
+    compared with the oracle, the semaphores with iters (TileSync) / iters * gN (RowSync)."""
+    import torch
+    from util import assert_close, normal_f16, to_dev, to_host, uniform_f16
+    print("launcher mlp", policy, split_k1, flush=True)
+    T = _lib.load_stage_tests()
+    M, K1, N1, N2 = 300, 1024, 512, 768
+    x, w1, w2 = uniform_f16((M, K1), 1), normal_f16((K1, N1), 2, std=0.05), normal_f16((N1, N2), 3, std=0.05)
+    dx, dw1, dw2 = to_dev(x), to_dev(w1), to_dev(w2)
+    dh = torch.full((M, N1), float("nan"), dtype=torch.float16, device="cuda")
+    dy = torch.full((M, N2), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    out = (C.c_int * 4)(-1, -1, -1, -1)
+    iters = 3
+    rc = T.run_launcher_mlp(policy, C.c_uint32(M), C.c_uint32(K1), C.c_uint32(N1), C.c_uint32(N2), C.c_void_p(dx.data_ptr()),
+                            C.c_void_p(dw1.data_ptr()), C.c_void_p(dh.data_ptr()), C.c_void_p(dw2.data_ptr()), C.c_void_p(dy.data_ptr()),
+                            split_k1, iters, out)
+    assert rc == 0
+    assert list(out) == [0, 0, iters, 0], list(out)       # every status success, no time-out, flag == iters, semaphores as expected
+    h, y = to_host(dh), to_host(dy)
+    assert_close(h, orc.gemm(x, w1, orc.EPI_GELU), "H")
+    assert_close(y, orc.gemm(h, w2), "Y")
+
+
+def test_resnet_pair_on_the_convolution_launcher():
+    """The ResNet pair (CV/resnet.cu:107-116, 704-744) on cusync::CuSyncImplicitGemmConvolution: TileSync producer,
+    Conv2DTileSync consumer, run(true, NULL, stream) per iteration."""
+    import torch
+    from util import assert_close, to_dev, to_host, uniform_f16
+    T = _lib.load_stage_tests()
+    N, H, W, Cc = 4, 20, 20, 64
+    rng = np.random.default_rng(5)
+    x = uniform_f16((N, H, W, Cc), 4)
+    w1, w2 = ((rng.standard_normal((Cc, 3, 3, Cc)) * np.sqrt(2.0 / (9 * Cc))).astype(np.float16) for _ in range(2))
+    dx, dw1, dw2 = to_dev(x), to_dev(w1), to_dev(w2)
+    dy1 = torch.full((N, H, W, Cc), float("nan"), dtype=torch.float16, device="cuda")
+    dy2 = torch.full((N, H, W, Cc), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    out = (C.c_int * 4)(-1, -1, -1, -1)
+    rc = T.run_launcher_conv_pair(C.c_uint32(N), C.c_uint32(H), C.c_uint32(W), C.c_uint32(Cc), C.c_void_p(dx.data_ptr()), C.c_void_p(dw1.data_ptr()),
+                                  C.c_void_p(dy1.data_ptr()), C.c_void_p(dw2.data_ptr()), C.c_void_p(dy2.data_ptr()), 2, out)
+    assert rc == 0
+    assert list(out) == [0, 0, 2, 0], list(out)
+    y1, y2 = to_host(dy1), to_host(dy2)
+    assert_close(y1, orc.conv2d_nhwc(x, w1, epilogue=orc.EPI_RELU), "y1")
+    assert_close(y2, orc.conv2d_nhwc(y1, w2), "y2")
