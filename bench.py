@@ -214,9 +214,20 @@ def main():
         times = interleaved(chains, args.warmup, args.steps)
         for c in chains:
             c.close()
+        def dist(v):
+            med = statistics.median(v)
+            lo = int(min(v) // 10 * 10)
+            bins = {}
+            for t in v:
+                b = int((t - lo) // 10)
+                bins[b] = bins.get(b, 0) + 1
+            return {"mean": round(statistics.fmean(v), 2), "median": round(med, 2), "min": round(min(v), 2), "max": round(max(v), 2),
+                    "p99": round(sorted(v)[min(len(v) - 1, int(len(v) * 0.99))], 2), "steps_over_1.05_median": sum(1 for t in v if t > 1.05 * med),
+                    "histogram_10us_bins_from_%d" % lo: [bins.get(i, 0) for i in range(max(bins) + 1)]}
         print(json.dumps({"metric": "GPT-3 MLP rounds of stream / rowsync / tilesync", "batch": args.batch, "warmup_rounds": args.warmup,
-                          "rounds": args.steps, "settle_steps": SETTLE_STEPS,
-                          "event_us": {n: round(statistics.fmean(t), 2) for n, t in zip(("stream", "rowsync", "tilesync"), times)}}))
+                          "rounds": args.steps, "settle_steps": SETTLE_STEPS, "wait_kernel_forced": os.environ.get("CUSYNC_WAIT_KERNEL", "0") not in ("", "0"),
+                          "event_us": {n: round(statistics.fmean(t), 2) for n, t in zip(("stream", "rowsync", "tilesync"), times)},
+                          "step_us": {n: dist(t) for n, t in zip(("stream", "rowsync", "tilesync"), times)}}))
         return
     if args.profile_chain == "attention":
         heads, e, seq = 12, 12 * 128, 2048

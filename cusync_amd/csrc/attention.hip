@@ -189,18 +189,17 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   L->cfg = *cfg;
   L->wqkv = wqkv; L->wo = wo;
   L->E = cfg->heads * kHD;
-  // Same per-row-count choice as the MLP chain.  Widths that are multiples of 192 (4608 = 24 x 192, 12288 =
-  // 64 x 192) take the 192-wide direct-to-LDS tiles: 64x192x64 up to 256 rows, where streaming the weights
-  // bounds the projections, 128x192 above (256x192, the MLP's choice from 1024 rows on, gains nothing here: the
-  // QKV projection has only 24 column tiles).  Other widths: tiles that follow the row count up to 128 rows,
-  // 128x128 up to 1024 rows, 128x256 above.
+  // Per-row-count choice, from the tuner's measurements (cusync_amd/tile_sizes_db.py, gpt3_attention_mi355x).
+  // Widths that are multiples of 192 (4608 = 24 x 192, 12288 = 64 x 192) take the 192-wide direct-to-LDS tiles:
+  // 64x192x64 up to 256 rows, where streaming the weights bounds the projections; 128x192 with a CU to itself
+  // while the GEMM has about one tile per CU (QKV projection, 24 column tiles: up to 1024 rows; output projection,
+  // 64: up to 512); 256x192 above (2048 rows: 446 -> 430 us for the chain against 128x192 at two per CU).
+  // Other widths: tiles that follow the row count up to 128 rows, 128x128 up to 1024 rows, 128x256 above.
   const int small = cfg->seq <= 32 ? CUSYNC_TILE_D32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  // 128x192: with a CU to itself, four stages and the pipelined order while the GEMM has about one tile per CU
-  // (QKV projection, 24 column tiles: up to 1024 rows; output projection, 64: up to 512), else two per CU
   auto wide = [&](uint32_t aloneUpTo) {
     return cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64
-           : cfg->seq <= aloneUpTo ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_128x192x32;
+           : cfg->seq <= aloneUpTo ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
   };
   L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide(1024) : dflt;
   L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide(512) : dflt;
@@ -348,7 +347,8 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     // host when the producer's launch takes every workgroup slot of the device (a wait kernel's wave would keep its
     // last workgroup off the device), by the wait kernel otherwise.  eMid1 / eMid2 only serve the stage timing.
     if (overlapped) {
-      if ((e = cusync_gemm_fills_device(&a1) ? cusync_wait_producer_started(&L->st[0], 0) : cusync_invoke_wait_kernel(&L->st[0], s1)) != CUSYNC_SUCCESS) return e;
+      const bool fills = cusync_gemm_fills_device(&a1) != 0 && !cusync::rt::forceWaitKernel();
+      if ((e = fills ? cusync_wait_producer_started(&L->st[0], 0) : cusync_invoke_wait_kernel(&L->st[0], s1)) != CUSYNC_SUCCESS) return e;
     }
     if (CUSYNC_HIP(hipEventRecord(L->eMid1, s1))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_attention_run(&a2, s1)) != CUSYNC_SUCCESS) return e;

@@ -169,12 +169,14 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // silu(gate) * up in GEMM1's epilogue: both GEMMs have plain operands and run the direct-to-LDS tiles at every
     // batch size; the kernels mask the ragged last column tile of the shard's widths (2 * 2752 and 8192).  The
     // policies count columns of the intermediate, half a GEMM1 tile wide, and no width constrains StridedSync.
+    // Measured by the tuner on the LLaMA shard (cusync_amd/tile_sizes_db.py, llama_mlp_mi355x): the 64-row tiles stay
+    // ahead up to 512 rows (232 tiles of 64x192 for GEMM1 against 116 of 128x192: 134 -> 112 us for the pair).
     int a, b;
     if (c.batch <= 32) a = b = CUSYNC_TILE_D32x128x64;
     else if (c.batch <= 64) a = b = CUSYNC_TILE_D64x128x64;
-    else if (c.batch <= 256) a = b = CUSYNC_TILE_D64x192x64;
-    else if (c.batch <= 1024) a = b = CUSYNC_TILE_128x192x32_ALONE;
-    else { a = CUSYNC_TILE_256x192x32; b = CUSYNC_TILE_256x256x32; }
+    else if (c.batch <= 512) { a = CUSYNC_TILE_D64x192x64; b = CUSYNC_TILE_D64x128x64; }
+    else if (c.batch <= 1024) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_128x256x32; }
+    else a = b = CUSYNC_TILE_256x256x32;
     *t1 = c.tile1 >= 0 ? c.tile1 : a;
     *t2 = c.tile2 >= 0 ? c.tile2 : b;
     if (c.one_launch && sync != CUSYNC_SYNC_STREAM && c.tile2 < 0) *t2 = *t1;
@@ -512,7 +514,7 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
       auto holdBack = [&](const cusync_stage_desc* prod, bool fills, hipStream_t s) {
         return fills ? cusync_wait_producer_started(prod, 0) : cusync_invoke_wait_kernel(prod, s);
       };
-      const bool fills1 = cusync_gemm_fills_device(&a1) != 0;
+      const bool fills1 = cusync_gemm_fills_device(&a1) != 0 && !cusync::rt::forceWaitKernel();
       if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a hold-back per edge
         if ((e = holdBack(&m->prod, fills1, m->sMid)) != CUSYNC_SUCCESS) return e;
         if ((e = runActStage(m, h, m->sMid)) != CUSYNC_SUCCESS) return e;

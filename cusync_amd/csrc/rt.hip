@@ -44,6 +44,14 @@ bool forceAcquire() {
   return on;
 }
 
+bool forceWaitKernel() {
+  static const bool on = [] {
+    const char* v = getenv("CUSYNC_WAIT_KERNEL");
+    return v && *v && strcmp(v, "0") != 0;
+  }();
+  return on;
+}
+
 bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t* sum) {
   uint32_t total = 0;
   for (int i = 0; i < count; i++) {

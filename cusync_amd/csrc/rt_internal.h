@@ -16,6 +16,10 @@ int check(hipError_t e, const char* what, const char* file, int line);
 // wait then ends with the agent-scope acquire (cache invalidation), also where the launcher found that the
 // producer's tiles are whole cache lines of the consumer's operand and the invalidation can be skipped.
 bool forceAcquire();
+// True when CUSYNC_WAIT_KERNEL is set to something other than 0: the chain handles then hold every consumer back
+// with the wait kernel, also behind a producer whose launch takes every workgroup slot (where they would wait on
+// the host).  For measuring what the host-side hold is there to prevent.
+bool forceWaitKernel();
 // Adds up the counters of waits that gave up (cusync_stage_desc::spinTimeouts) of the stages given; null
 // entries and stages without a counter are skipped.  Returns false if a copy from the device failed.
 bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t* sum);

@@ -13,6 +13,12 @@ writes the result in the reference's schema:
 plus, per entry, the tile ids of this library ("TileIds") and the measured latencies ("us").
 
     python -m cusync_amd.tuner --model gpt3 --batches 1,16,64,256,512,1024,2048 --out cusync_amd/tile_sizes_db.py
+    python -m cusync_amd.tuner --model llama --out cusync_amd/tile_sizes_db.py        # "tilesync" is StridedSync there
+    python -m cusync_amd.tuner --model attention --batches 256,512,1024,2048 --out cusync_amd/tile_sizes_db.py
+
+(each call appends one table to the file).  The attention table follows the reference's gpt3_attention tables
+(tile_sizes_db.py:364-392: {seqlen: {batch: entry}} with seqlen 0 = no key/value cache); its two tile shapes are
+those of the QKV projection and the output projection, the fused attention kernel between them has one shape.
 """
 import argparse
 import pprint
@@ -32,6 +38,13 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 
 
+def resident_share(tile, M, N, split):
+    """Share of the device's workgroup slots a launch of this GEMM takes (1.0 = every slot)."""
+    g = api.gemm_grid(tile, M, N, split)
+    resident = api._lib.load().cusync_gemm_max_resident(tile)
+    return min(g[0] * g[1] * g[2], resident) / float(resident)
+
+
 def candidates(batch, n1, n2):
     """(tile, split) choices worth timing for a GEMM with `batch` rows."""
     if batch <= 32:
@@ -44,8 +57,13 @@ def candidates(batch, n1, n2):
         tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4]
     else:
         tiles, splits = [api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
-    ok = lambda t, n: n % 192 == 0 or t not in (api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE)
-    return [(t, s) for t in tiles for s in splits if ok(t, n1)], [(t, s) for t in tiles for s in splits if ok(t, n2)]
+    if n1 % 192 or n2 % 192:        # the LLaMA shard (5504 and 8192 columns): also the 256-wide tiles
+        if batch > 512:
+            tiles = tiles + [api.TILE.T256x256x32, api.TILE.T128x192x32_ALONE]
+        elif batch > 32:
+            tiles = tiles + [api.TILE.D64x128x64]
+    # the register-staged tiles have no SwiGLU epilogue path worth timing against the direct-to-LDS ones
+    return [(t, s) for t in tiles for s in splits], [(t, s) for t in tiles for s in splits]
 
 
 def trimmed(times):
@@ -115,12 +133,22 @@ def tune_batch(bench, batch, log):
         row = trimmed(bench.run(batch, api.SYNC.ROW, timed=20, **kw))
         # TileSync with the option bits of the reference's table; AvoidCustomOrder is always safe here, AvoidWaitKernel
         # only when producer and consumer fit on the device together (nothing can then keep a producer workgroup off it)
-        tile_opts = {"AvoidCustomOrder": False, "AvoidWaitKernel": False, "ReorderTileLoads": True, "NoAtomicAdd": True}
-        base = api.OPT.NO_ATOMIC_ADD | api.OPT.REORDER_TILE_LOADS
-        tile = trimmed(bench.run(batch, api.SYNC.TILE, timed=20, opts=base, **kw))
-        t_aco = bench.run(batch, api.SYNC.TILE, timed=20, opts=base | api.OPT.AVOID_CUSTOM_ORDER, **kw)
+        # (the LLaMA chain's tile policy is StridedSync, whose semaphores count to two: atomic adds, TB/mlp.cu:9-14, 109)
+        llama = bench.model == api.MODEL.LLAMA
+        mode = api.SYNC.STRIDED if llama else api.SYNC.TILE
+        tile_opts = {"AvoidCustomOrder": False, "AvoidWaitKernel": False, "ReorderTileLoads": True, "NoAtomicAdd": not llama}
+        base = api.OPT.REORDER_TILE_LOADS | (0 if llama else api.OPT.NO_ATOMIC_ADD)
+        tile = trimmed(bench.run(batch, mode, timed=20, opts=base, **kw))
+        t_aco = bench.run(batch, mode, timed=20, opts=base | api.OPT.AVOID_CUSTOM_ORDER, **kw)
         if t_aco is not None and trimmed(t_aco) < tile:
             tile, tile_opts["AvoidCustomOrder"] = trimmed(t_aco), True
+        share = (resident_share(kw["tile1"], batch, bench.n1, kw["split_k1"]) +
+                 resident_share(kw["tile2"], batch, bench.hidden, kw["split_k2"]))
+        if share <= 1.0:       # both launches are resident together: no wait kernel is needed (CS/cusync.h:193-196, 205-206)
+            o = base | api.OPT.AVOID_WAIT_KERNEL | (api.OPT.AVOID_CUSTOM_ORDER if tile_opts["AvoidCustomOrder"] else 0)
+            t_awk = bench.run(batch, mode, timed=20, opts=o, **kw)
+            if t_awk is not None and trimmed(t_awk) < tile:
+                tile, tile_opts["AvoidWaitKernel"] = trimmed(t_awk), True
         return stream, row, tile, tile_opts
 
     tuned = dict(tile1=best1[1], tile2=best2[1], split_k1=best1[2], split_k2=best2[2])
@@ -155,19 +183,92 @@ def tune_batch(bench, batch, log):
     }
 
 
+def tune_attention(seq, log, hidden=12288, heads=12):
+    """Tile shapes of the two projections and the key/value split of the attention chain at `seq` rows."""
+    import torch
+    e = heads * 128
+    g = torch.Generator(device="cuda").manual_seed(4)
+    wqkv = (torch.randn((hidden, 3 * e), device="cuda", generator=g) * 0.02).half()
+    wo = (torch.randn((e, hidden), device="cuda", generator=g) * 0.02).half()
+    x = (torch.rand((seq, hidden), device="cuda", generator=g) * 2 - 1).half()
+    qkv = torch.empty((seq, 3 * e), dtype=torch.float16, device="cuda")
+    o = torch.empty((seq, e), dtype=torch.float16, device="cuda")
+    y = torch.empty((seq, hidden), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+
+    def run(sync, **kw):
+        layer = api.AttnLayer(seq, hidden, heads, sync, wqkv.data_ptr(), wo.data_ptr(), **kw)
+        try:
+            layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=10)
+            t, st = layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=20, stages=True)
+            return trimmed(t), [trimmed([v[i] for v in st]) for i in range(3)], layer.tiles()
+        finally:
+            layer.destroy()
+
+    if seq <= 256:
+        tiles = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T128x128x32]
+    elif seq <= 1024:
+        tiles = [api.TILE.T128x192x32_ALONE, api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.T128x128x32]
+    else:
+        tiles = [api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.T128x192x32_ALONE]
+    run(api.SYNC.STREAM)        # clocks up
+    best1 = best3 = None
+    for t in tiles:
+        total, st, _ = run(api.SYNC.STREAM, tile1=t, tile3=tiles[0])
+        log("S=%d QKV projection tile %d: %.1f us" % (seq, t, st[0]))
+        if best1 is None or st[0] < best1[0]:
+            best1 = (st[0], t)
+    for t in tiles:
+        total, st, _ = run(api.SYNC.STREAM, tile1=best1[1], tile3=t)
+        log("S=%d output projection tile %d: %.1f us" % (seq, t, st[2]))
+        if best3 is None or st[2] < best3[0]:
+            best3 = (st[2], t)
+    bestkv = None
+    for kv in (0, 8, 16):
+        total, st, _ = run(api.SYNC.STREAM, tile1=best1[1], tile3=best3[1], kv_split_blocks=kv)
+        log("S=%d attention with at most %d key/value blocks per workgroup: %.1f us" % (seq, kv, st[1]))
+        if bestkv is None or st[1] < bestkv[0]:
+            bestkv = (st[1], kv)
+    kw = dict(tile1=best1[1], tile3=best3[1], kv_split_blocks=bestkv[1])
+    us = {}
+    for name, sync in (("baseline", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE), ("consecutivesync", api.SYNC.STRIDED)):
+        us[name] = round(run(sync, **kw)[0], 1)
+    us.update(qkv=round(best1[0], 1), attention=round(bestkv[0], 1), out_proj=round(best3[0], 1))
+    log("S=%d chain: %s" % (seq, us))
+
+    def sizes(t):
+        bm, bn, bk = api.tile_shape(t)
+        wm, wn, _ = WAVES[t]
+        return [bm, bn, bk, bm // wm, bn // wn, bk]
+
+    entry = {"TileSizes": [sizes(best1[1]), sizes(best3[1])], "TileIds": [best1[1], best3[1]],
+             "NumStages": [WAVES[best1[1]][2], WAVES[best3[1]][2]], "KVSplitBlocks": bestkv[1]}
+    for key in ("baseline", "rowsync", "consecutivesync"):
+        entry[key] = {"KVSplitBlocks": bestkv[1]}
+    entry["tilesync"] = {"KVSplitBlocks": bestkv[1], "AvoidCustomOrder": False, "AvoidWaitKernel": False, "ReorderTileLoads": True, "NoAtomicAdd": True}
+    entry["us"] = us
+    return entry
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--model", choices=sorted(SHAPES), default="gpt3")
+    ap.add_argument("--model", choices=sorted(SHAPES) + ["attention"], default="gpt3")
     ap.add_argument("--batches", default="1,16,64,256,512,1024,2048")
     ap.add_argument("--out", default=None, help="file to write the table to (default: stdout)")
     args = ap.parse_args()
-    model, hidden, inner = SHAPES[args.model]
-    bench = Bench(model, hidden, inner)
     log = lambda s: print(s, file=sys.stderr, flush=True)
     db = {}
-    for b in sorted((int(v) for v in args.batches.split(",")), reverse=True):
-        db[b] = tune_batch(bench, b, log)
-    name = "%s_mlp_mi355x" % args.model
+    if args.model == "attention":
+        db[0] = {}
+        for s in sorted((int(v) for v in args.batches.split(",")), reverse=True):
+            db[0][s] = tune_attention(s, log)
+        name = "gpt3_attention_mi355x"
+    else:
+        model, hidden, inner = SHAPES[args.model]
+        bench = Bench(model, hidden, inner)
+        for b in sorted((int(v) for v in args.batches.split(",")), reverse=True):
+            db[b] = tune_batch(bench, b, log)
+        name = "%s_mlp_mi355x" % args.model
     text = ("# Written by `python -m cusync_amd.tuner --model %s`; schema of the reference's tile_sizes_db.py.\n"
             "# Dictionary of tile sizes for each M\n%s = %s\n" % (args.model, name, pprint.pformat(db, width=120, sort_dicts=False)))
     if args.out:

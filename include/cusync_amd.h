@@ -177,7 +177,8 @@ cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc *prod, void
  * place its last workgroup on that CU; the flag is then not raised until another workgroup retires and the chain
  * is one producer tile longer (measured on the 2048-row GPT-3 MLP: 720-790 us against 610 in one run out of ten;
  * per-workgroup timestamps show workgroup 249 of 256 entering at 313 us).  The host holds no CU.  The chain
- * handles of this library use it for exactly those producers and the wait kernel for all others.  No counterpart
+ * handles of this library use it for exactly those producers and the wait kernel for all others (with
+ * CUSYNC_WAIT_KERNEL=1 in the environment they use the wait kernel everywhere, for comparison).  No counterpart
  * in the reference. */
 cusync_error cusync_wait_producer_started(const cusync_stage_desc *prod, uint32_t timeout_ms);
 /* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
