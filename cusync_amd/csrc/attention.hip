@@ -24,24 +24,38 @@ using cusync::rt::setError;
 using namespace cusync::attn;
 
 std::mutex g_attnMutex;
-int g_attnResidentPerCU = -1;
-
+int g_attnResidentPerCU[2] = {-1, -1};      // [0] two stages, [1] four
 int g_attnNumCUs = 0;
 
-int residentAttention() {
+typedef void (*AttnKernel)(AttnParams);
+AttnKernel attnKernel(bool deep) { return deep ? attentionKernel<4> : attentionKernel<2>; }
+int attnLds(bool deep) { return cusync::attn::ldsBytes(deep ? 4 : 2); }
+
+// Four stages where the kernel has the device to itself anyway: as a stage of its own between stream-ordered
+// launches, and from 2048 key rows on, where the projections around it run 256-row tiles that take a whole CU's
+// LDS (measured at 2048 rows x 12 heads: 59 -> 51 us alone; chain under ConsecutiveSync 422 -> 410 us).  Two stages
+// where its workgroups are to sit beside those of its producer and consumer (chains up to 1024 rows: with four
+// stages every gain of the overlapped chains over the stream-ordered ones was gone).
+bool deepPipeline(const cusync_attention_args* a) {
+  const bool alone = a->stage.in.kind == CUSYNC_POLICY_NOSYNC && a->stage.out.kind == CUSYNC_POLICY_NOSYNC;
+  return alone || a->seq + a->cached_rows >= 2048;
+}
+
+int residentAttention(bool deep) {
   std::lock_guard<std::mutex> lock(g_attnMutex);
-  if (g_attnResidentPerCU < 0) {
+  int& perCU = g_attnResidentPerCU[deep ? 1 : 0];
+  if (perCU < 0) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
     g_attnNumCUs = prop.multiProcessorCount;
-    if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attentionKernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes))) return 0;
+    if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attnKernel(deep)),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, attnLds(deep)))) return 0;
     int n = 0;
-    if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attentionKernel, kThreads, kLdsBytes))) return 0;
-    g_attnResidentPerCU = n;
+    if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attnKernel(deep), kThreads, attnLds(deep)))) return 0;
+    perCU = n;
   }
-  return g_attnResidentPerCU * g_attnNumCUs;
+  return perCU * g_attnNumCUs;
 }
 
 cusync_policy_desc noSync() {
@@ -122,6 +136,10 @@ cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
   const cusync_dim3 g = cusync_attention_grid_split(a->seq, a->heads, a->cached_rows, a->kv_split_blocks);
   const cusync_stage_desc& s = a->stage;
   if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("attention: stage grid does not match cusync_attention_grid / cusync_attention_grid_split"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if ((uint64_t)a->seq * a->ldo * 2 >= 0x80000000ull || cusync_attention_workspace_size(a) >= 0x80000000ull) {
+    setError("attention: output or workspace larger than 2 GiB is not addressable by one buffer descriptor");
+    return CUSYNC_ERROR_NOT_INITIALIZED;
+  }
   if (g.z > 1 && (!a->workspace || (uintptr_t)a->workspace % 16)) { setError("attention: a split key range needs a 16-byte aligned workspace of cusync_attention_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (!s.tileOrder || !s.tileCounter || !s.startCounter || !s.spinTimeouts || !s.xcdTickets) { setError("attention: stage not allocated"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (s.out.kind != CUSYNC_POLICY_NOSYNC && !s.tileStatusWrite) { setError("attention: producer stage without semaphores"); return CUSYNC_ERROR_NOT_INITIALIZED; }
@@ -145,12 +163,13 @@ cusync_error cusync_attention_can_implement(const cusync_attention_args* a) {
   return CUSYNC_SUCCESS;
 }
 
-int cusync_attention_max_resident(void) { return residentAttention(); }
+int cusync_attention_max_resident(void) { return residentAttention(false); }
 
 cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) {
   cusync_error e = cusync_attention_can_implement(a);
   if (e != CUSYNC_SUCCESS) return e;
-  const int resident = residentAttention();
+  const bool deep = deepPipeline(a);
+  const int resident = residentAttention(deep);
   if (resident <= 0) { setError("attention: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
   const cusync_stage_desc& s = a->stage;
   uint32_t launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)resident);
@@ -167,14 +186,16 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.scaleLog2 = scale * 1.4426950408889634f;
   p.causal = a->causal ? 1 : 0;
   p.launched = launched;
+  cusync::rt::timeline(&p.timeline, &p.timelineCap);
   if (s.grid.z > 1) {
     const size_t tiles = (size_t)s.grid.x * s.grid.y;
     p.chunk = a->kv_split_blocks;
     p.partO = (float*)a->workspace;
     p.partStat = p.partO + tiles * s.grid.z * 64 * kThreads;
     p.arrivals = (uint32_t*)(p.partStat + tiles * s.grid.z * 2 * kThreads);
+    p.partBytes = (uint32_t)((char*)p.arrivals - (char*)p.partO);
   }
-  hipLaunchKernelGGL(attentionKernel, dim3(launched), dim3(kThreads), kLdsBytes, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(attnKernel(deep), dim3(launched), dim3(kThreads), attnLds(deep), (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }
@@ -204,12 +225,13 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide(1024) : dflt;
   L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide(512) : dflt;
   L->ws1 = L->ws3 = L->ws2 = nullptr;
-  // Key ranges of 16 blocks (1024 rows) or more are cut in two.  Measured alone at 12 heads: 1024 rows 40 -> 35 us,
-  // 2048 rows 73 -> 65 us; finer cuts lose again (four: 71 us, eight: 124 us) — the kernel is bound by the softmax
-  // arithmetic of a CU rather than by its longest workgroup, and every cut adds a tile's fixed cost (Q fragments,
-  // first block, a pass over the partial results).
+  // Key ranges of 8 blocks (512 rows) or more are cut in two: under a causal mask the last row tiles walk the
+  // longest ranges and the launch is as long as its longest workgroup.  Measured alone at 12 heads: 512 rows
+  // 26.7 -> 25.3 us, 1024 rows 37.8 -> 30.8 us, 2048 rows 61 -> 50 us; finer cuts lose again (2048 rows in four:
+  // 62 us, in eight: 89 us): every cut adds a tile's fixed cost (first blocks, Q fragments, a pass over the
+  // partial results) and tickets without work.
   const uint32_t kvBlocks = (cfg->cached_rows + cfg->seq + kBKV - 1) / kBKV;
-  L->kvSplit = cfg->kv_split_blocks >= 0 ? (uint32_t)cfg->kv_split_blocks : kvBlocks >= 16 ? (kvBlocks + 1) / 2 : 0u;
+  L->kvSplit = cfg->kv_split_blocks >= 0 ? (uint32_t)cfg->kv_split_blocks : kvBlocks >= 8 ? (kvBlocks + 1) / 2 : 0u;
   uint32_t tm1 = 0, tn1 = 0;
   if (cusync_gemm_tile_shape(L->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(L->tile3, nullptr, nullptr, nullptr)) {
     setError("attn layer: unknown tile id");

@@ -60,18 +60,24 @@ enum { kAPlain = 0, kAConv = 1 };
 // [1] tile x | y << 16 | z << 32 | tiles this workgroup did before << 48
 // [2..6] constant-rate 100 MHz clock: tile drawn, first loads issued (the waits of the first chunks are over),
 //        main loop done, epilogue and post done, and the clock at kernel entry of this workgroup;  [7] launched
-__device__ __forceinline__ void recordTile(const GemmParams& p, const cusync_dim3& t, uint32_t round,
-                                           unsigned long long tEntry, unsigned long long t0, unsigned long long t1,
-                                           unsigned long long t2, unsigned long long t3) {
-  if (!p.timeline) return;
-  const unsigned long long slot = __hip_atomic_fetch_add(p.timeline, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (slot >= p.timelineCap) return;
-  unsigned long long* r = p.timeline + 1 + slot * 8;
-  const uint32_t role = (p.stage.isProducer() ? 1u : 0u) | (p.stage.isConsumer() ? 2u : 0u);
+__device__ __forceinline__ void recordTileAt(unsigned long long* timeline, uint32_t timelineCap, const cusync::DynStage& stage,
+                                             uint32_t launched, const cusync_dim3& t, uint32_t round,
+                                             unsigned long long tEntry, unsigned long long t0, unsigned long long t1,
+                                             unsigned long long t2, unsigned long long t3) {
+  if (!timeline) return;
+  const unsigned long long slot = __hip_atomic_fetch_add(timeline, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (slot >= timelineCap) return;
+  unsigned long long* r = timeline + 1 + slot * 8;
+  const uint32_t role = (stage.isProducer() ? 1u : 0u) | (stage.isConsumer() ? 2u : 0u);
   const uint32_t xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20);       // HW_REG_XCC_ID, bits 0..3
   r[0] = role | ((unsigned long long)cusync::DynStage::workgroupIndex() << 8) | ((unsigned long long)xcc << 40);
   r[1] = t.x | ((unsigned long long)t.y << 16) | ((unsigned long long)t.z << 32) | ((unsigned long long)round << 48);
-  r[2] = t0; r[3] = t1; r[4] = t2; r[5] = t3; r[6] = tEntry; r[7] = p.launched;
+  r[2] = t0; r[3] = t1; r[4] = t2; r[5] = t3; r[6] = tEntry; r[7] = launched;
+}
+__device__ __forceinline__ void recordTile(const GemmParams& p, const cusync_dim3& t, uint32_t round,
+                                           unsigned long long tEntry, unsigned long long t0, unsigned long long t1,
+                                           unsigned long long t2, unsigned long long t3) {
+  recordTileAt(p.timeline, p.timelineCap, p.stage, p.launched, t, round, tEntry, t0, t1, t2, t3);
 }
 
 // First output column of the tile whose first column of the product is n0: the SwiGLU epilogue folds pairs of
@@ -280,6 +286,8 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
       for (int g = 0; g < 4; g++)
         *reinterpret_cast<floatx4*>(mine + t.z * sliceStride + slot(i, j, g)) =
             floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+  // the release below is the first thread's and covers its own wavefront's stores; the others see theirs through here
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   uint32_t* counter = p.arrivals + t.y * p.stage.d.grid.x + t.x;
   if (threadIdx.x == 0) {

@@ -15,6 +15,7 @@
 //   B stage  [BK rows][BN halfs]:   chunk c of row k lives at slot c ^ 4*(k&1)
 // so that the eight lanes the LDS serves together (A fragments: eight rows;
 // B transpose reads: four k rows x 64 bytes) fall on distinct bank groups.
+// (With BK = 32 the swizzle of A is (r / 4) % 4, see A_SWZ_DIV below.)
 //
 // Pipeline.  STAGES LDS stages; iteration kt waits for its own chunk
 // (s_waitcnt vmcnt), passes one barrier, issues the loads of chunk kt+STAGES-1
@@ -111,7 +112,11 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
 
   // ---- direct-load side: which global chunk this lane fetches ---------------
   // A: load q of this wave fills rows (wave*A_LOADS + q)*A_ROWS_PER_LOAD + lane/A_CPR, slot lane%A_CPR.
-  constexpr int A_SWZ_DIV = 8 / C::A_CPR;                     // rows that share a swizzle value
+  // Rows that share a swizzle value.  A 16-byte-per-lane LDS read is served sixteen lanes at a time over all 64
+  // banks: with 64-byte rows the sixteen rows of such a group cover every bank four times over, so rows r, r+4, r+8
+  // and r+12 must sit in four different slots (four rows per swizzle value: 5.5 clocks per wave instruction on one
+  // CU against 8.0 with two rows per value).
+  constexpr int A_SWZ_DIV = C::A_CPR == 4 ? 4 : 1;
   const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + lane / C::A_CPR;
   const uint32_t aLoadChunk = (lane % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
   // B: the 16-byte slots of a stage are numbered row by row; load q of this wave fills slots

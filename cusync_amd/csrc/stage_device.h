@@ -261,6 +261,9 @@ struct DynStage {
   // one stands for (a workgroup that finished several logical tiles guarded by one semaphore adds them at once).
   __device__ __forceinline__ void post(const cusync_dim3& tile, uint32_t times = 1) const {
     if (!isProducer()) return;
+    // The release is the first thread's and waits for its own wavefront's stores; a workgroup barrier does not wait
+    // for stores to memory.  Every wavefront sees its own stores of the tile through before it reaches the barrier.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
       const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid) * CUSYNC_SEM_STRIDE;

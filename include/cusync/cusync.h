@@ -281,8 +281,9 @@ CUSTAGE_METHOD(CuSyncError) wait(dim3& tile, uint32_t waitingThread, bool callSy
 
 CUSTAGE_METHOD(CuSyncError) post(const dim3& tile, uint32_t postThread) {
   if (!isProducer()) return CuSyncErrorNotProducer;
-  // Barrier: all stores of the workgroup are issued and complete at workgroup
-  // scope; the release below then publishes them device-wide.
+  // Every wavefront sees its own stores through to memory first: a workgroup barrier does not wait for them, and
+  // the release below, issued by one thread, waits for the stores of that thread's wavefront only.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   const uint32_t flat = threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
   if (flat == postThread) {
