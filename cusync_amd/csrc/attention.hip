@@ -186,6 +186,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.scaleLog2 = scale * 1.4426950408889634f;
   p.causal = a->causal ? 1 : 0;
   p.launched = launched;
+  p.stage.prepare(launched);
   cusync::rt::timeline(&p.timeline, &p.timelineCap);
   if (s.grid.z > 1) {
     const size_t tiles = (size_t)s.grid.x * s.grid.y;

@@ -186,6 +186,7 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 &&
                         (a->lda * 2) % 128 == 0 && (wholeLineTiles || canRound);
   p.waitRound = p.stage.lineAligned && !wholeLineTiles ? 64 : 1;
+  p.stage.prepare(launched);
   p.M = a->M; p.N = a->N; p.K = a->K;
   p.A = (const half_t*)a->A; p.lda = a->lda;
   p.B = (const half_t*)a->B; p.ldb = a->ldb;

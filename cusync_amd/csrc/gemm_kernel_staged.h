@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
   // being computed and settled when the tile is done.
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
-  const bool noDraws = stage.allStatic(p.launched);     // every tile is some workgroup's static first tile
+  const bool noDraws = stage.noDraws;     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
     if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kActThreads) void swigluStageKernel(ActParams p) {
   const uint32_t zWait = consumer && stage.d.in.kind == CUSYNC_POLICY_ROWSYNC ? 1 : 0;
   uint32_t dryXcds = 0, nextRaw = 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
-  const bool noDraws = stage.allStatic(p.launched);
+  const bool noDraws = stage.noDraws;
   for (uint32_t round = 0;; round++) {
     if (tid == 0) sTicket = round == 0 ? stage.firstTicket(p.launched, dryXcds, noDraws) : stage.drawFinish(nextRaw, p.launched, round, dryXcds, noDraws);
     __syncthreads();
@@ -155,6 +155,7 @@ cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
   p.G = (const half_t*)h; p.ldg = m->ldh;
   p.A = (half_t*)m->act; p.lda = m->cfg.inner;
   p.launched = std::min<uint32_t>(s.grid.x * s.grid.y * s.grid.z, (uint32_t)resident);
+  p.stage.prepare(p.launched);
   hipLaunchKernelGGL(swigluStageKernel, dim3(p.launched), dim3(kActThreads), 0, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;

@@ -30,11 +30,14 @@ struct DynStage {
   // its wait; the wait can skip the cache invalidation that would also throw
   // away the weights the XCD's workgroups share.
   bool lineAligned;
+  // allStatic(launched) of the launch this object goes to, worked out by the launcher (set by prepare()): in the
+  // kernel it is a loop of eight rounds of integer divisions that every wavefront would run before its first load.
+  bool noDraws;
 
   __device__ __forceinline__ bool isProducer() const { return d.out.kind != CUSYNC_POLICY_NOSYNC; }
   __device__ __forceinline__ bool isConsumer() const { return d.in.kind != CUSYNC_POLICY_NOSYNC; }
   __device__ __forceinline__ uint32_t numTiles() const { return d.grid.x * d.grid.y * d.grid.z; }
-  __device__ __forceinline__ bool customOrder() const { return !(d.opts & CUSYNC_OPT_AVOID_CUSTOM_ORDER); }
+  __host__ __device__ __forceinline__ bool customOrder() const { return !(d.opts & CUSYNC_OPT_AVOID_CUSTOM_ORDER); }
 
   // ---- tickets -------------------------------------------------------------
   // A launch may hold fewer workgroups than the stage has tiles; each workgroup
@@ -73,15 +76,16 @@ struct DynStage {
   //    length is dry for good, the others are tried in turn, so the end of the
   //    launch stays balanced.  The last workgroup to find everything dry
   //    re-arms the dispensers for the next run.
-  __device__ __forceinline__ bool dealtByRows() const { return d.grid.x < 8; }
-  __device__ __forceinline__ uint32_t xcdTiles(uint32_t x) const {
+  __host__ __device__ __forceinline__ bool dealtByRows() const { return d.grid.x < 8; }
+  __host__ __device__ __forceinline__ uint32_t xcdTiles(uint32_t x) const {
     const uint32_t span = dealtByRows() ? d.grid.y : d.grid.x;
     return ((x + 1) * span / 8 - x * span / 8) * (dealtByRows() ? d.grid.x : d.grid.y) * d.grid.z;
   }
   // Positions of XCD x's list that are handed out statically to the first tiles of the workgroups.
-  __device__ __forceinline__ uint32_t xcdStatic(uint32_t x, uint32_t launched) const {
+  __host__ __device__ __forceinline__ uint32_t xcdStatic(uint32_t x, uint32_t launched) const {
     const uint32_t wgs = launched > x ? (launched - x + 7) / 8 : 0;
-    return min(wgs, xcdTiles(x));
+    const uint32_t tiles = xcdTiles(x);
+    return wgs < tiles ? wgs : tiles;
   }
   __device__ __forceinline__ uint32_t xcdTicket(uint32_t x, uint32_t l) const {
     const uint32_t span = dealtByRows() ? d.grid.y : d.grid.x;
@@ -93,12 +97,14 @@ struct DynStage {
   // True when the static first tiles already are all tiles (a launch of one round whose workgroups spread
   // evenly over the lists): nobody then needs a dispenser, a look at the others or the count of workgroups
   // that ran dry, and a workgroup leaves after its tile without a single atomic.
-  __device__ __forceinline__ bool allStatic(uint32_t launched) const {
+  __host__ __device__ __forceinline__ bool allStatic(uint32_t launched) const {
     if (!customOrder()) return false;
     bool all = true;
     for (uint32_t x = 0; x < 8; x++) all = all && xcdStatic(x, launched) == xcdTiles(x);
     return all;
   }
+  // Host side, once the descriptor and lineAligned are in place: what the kernel would otherwise work out per wavefront.
+  __host__ void prepare(uint32_t launched) { noDraws = allStatic(launched); }
   static __device__ __forceinline__ uint32_t workgroupIndex() {
     return blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   }
