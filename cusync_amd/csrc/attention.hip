@@ -187,6 +187,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.causal = a->causal ? 1 : 0;
   p.launched = launched;
   p.stage.prepare(launched);
+  p.descending = p.causal;
   cusync::rt::timeline(&p.timeline, &p.timelineCap);
   if (s.grid.z > 1) {
     const size_t tiles = (size_t)s.grid.x * s.grid.y;

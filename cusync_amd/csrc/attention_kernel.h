@@ -68,6 +68,7 @@ struct AttnParams {
   float* partStat;                   // [heads][row tiles][splits][2][256] row maximum, row sum
   uint32_t* arrivals;                // [heads][row tiles] splits finished; 0 between launches
   uint32_t partBytes;                // bytes of partO and partStat together (they are adjacent)
+  uint32_t descending;               // row tiles are taken last first
   unsigned long long* timeline;      // diagnosis (cusync_rt_set_timeline), records as the GEMM kernels write them
   uint32_t timelineCap;
 };
@@ -153,8 +154,10 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     cusync_dim3 t = stage.ticketToTile(ticket);
     // Tickets are handed out by ascending row tile, and under a causal mask the last row tiles walk the longest key
     // ranges (and are the only ones whose later splits exist at all): taken in descending order the long tiles
-    // start first and the tickets left for a second round are the short and the empty ones.
-    if (p.causal) t.y = stage.d.grid.y - 1 - t.y;
+    // start first and the tickets left for a second round are the short and the empty ones.  (Measured against
+    // the ascending order with every mode of the chain timed in turn: 2048 rows 433 -> 417 us stream-ordered,
+    // 426 -> 415 under RowSync; 512 rows 165 -> 161 and 157 -> 155; 1024 and 256 rows within 2 us either way.)
+    if (p.descending) t.y = stage.d.grid.y - 1 - t.y;
     const unsigned long long tl0 = p.timeline ? wall_clock64() : 0;
     const uint32_t head = t.x, q0 = t.y * kBQ;
     const uint32_t qEnd = min(q0 + (uint32_t)kBQ, p.S);
@@ -190,12 +193,36 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
         loadToLds(rLds, __builtin_amdgcn_readfirstlane(kLds + kStageBytes + q * 1024),
                   valid ? (rowOff + q * 4 * p.ldq + 2 * E + head * kHD + vChunk * 8) * 2 : kOutOfRange);
     };
+    // Key/value rows (counted from the first row the producer writes) below these marks are known to be posted, for
+    // the K and for the V columns of this head.  A poll is a round trip to memory that the direct loads in flight
+    // have to drain behind, so a block that needs rows beyond the mark first looks, without spinning, at all row
+    // blocks of the producer that the rest of this tile's key range meets, and spins only if its own rows are
+    // still missing: a tile that starts after its producer is done polls twice in all.
+    uint32_t seenRows[2] = {0, 0};
     auto waitKV = [&](uint32_t j) {
+      if (!consumer) return;
       // only the rows behind the cache come from the producer; its tiles count rows from there
       const uint32_t lo = max(j * kBKV, p.cached), hi = min(j * kBKV + (uint32_t)kBKV, total);
       if (lo >= hi) return;
-      waitRows(lo - p.cached, hi - p.cached, E + head * kHD);
-      waitRows(lo - p.cached, hi - p.cached, 2 * E + head * kHD);
+      const uint32_t rowLo = lo - p.cached, rowHi = hi - p.cached;             // [rowLo, rowHi)
+      const uint32_t rangeEnd = min(jEnd * kBKV, total) - p.cached;            // end of this tile's key range
+#pragma unroll
+      for (int c = 0; c < 2; c++) {
+        if (rowHi <= seenRows[c]) continue;
+        const uint32_t col = (c + 1) * E + head * kHD;
+        bool oneTile = zWait || col / tnq == (col + kHD - 1) / tnq;           // the head's columns lie in one producer tile
+        if (oneTile) {
+          const uint32_t first = max(rowLo, seenRows[c]);
+          const uint32_t ready = stage.peekWaveRows(first, rangeEnd - 1, tmq, col / tnq * tnq, zWait);
+          if (ready) seenRows[c] = min(rangeEnd, (first / tmq + ready) * tmq);
+        }
+        if (rowHi > seenRows[c]) {
+          waitRows(rowLo, rowHi, col);
+          seenRows[c] = max(seenRows[c], min(rangeEnd, ((rowHi - 1) / tmq + 1) * tmq));
+        }
+        // RowSync guards all columns of a row block with one semaphore: what is known of K holds for V (and for Q)
+        if (stage.d.in.kind == CUSYNC_POLICY_ROWSYNC) { seenRows[1] = seenRows[0]; break; }
+      }
     };
 
     // The first blocks are requested before Q: they are what the tile waits for longest.
@@ -206,7 +233,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     }
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     // Q fragments stay in registers for the whole tile: k-step s is head-dim 16s + 8hi .. + 7 of row myq.
-    waitRows(q0, qEnd, head * kHD);
+    if (!(stage.d.in.kind == CUSYNC_POLICY_ROWSYNC && p.cached == 0 && seenRows[0] >= qEnd)) waitRows(q0, qEnd, head * kHD);
     half8 qf[8];
 #pragma unroll
     for (int s = 0; s < 8; s++)

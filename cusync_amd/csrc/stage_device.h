@@ -235,6 +235,27 @@ struct DynStage {
     if (timedOut && lane == 0) dev::countGiveUp(d.spinTimeouts);
   }
 
+  // Wave-uniform look, without spinning, at the tiles {r, col, z} of the row blocks that meet rowLo..rowHi (at most
+  // 64 of them, one per lane, one round trip): how many of them, counted from the first, are posted.
+  __device__ __forceinline__ uint32_t peekWaveRows(uint32_t rowLo, uint32_t rowHi, uint32_t tileM, uint32_t col, uint32_t z) const {
+    if (!isConsumer()) return 64;
+    const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint32_t b0 = rowLo / tileM;
+    uint32_t blocks = rowHi / tileM - b0 + 1;
+    if (blocks > 64) blocks = 64;
+    const cusync_dim3 mine = {(b0 + (lane < blocks ? lane : 0u)) * tileM, col, z};
+    const bool polls = lane < blocks && needsWait(mine);
+    uint32_t v = 0xffffffffu;
+    if (polls) v = dev::loadRelaxed(&d.tileStatusRead[dyn::tileIndex(d.in, mine, d.prodGrid) * CUSYNC_SEM_STRIDE]);
+    const uint64_t pending = __ballot(lane < blocks && v < waitTarget());
+    const uint32_t ready = pending ? (uint32_t)__builtin_ctzll(pending) : blocks;
+    if (ready) {
+      if (lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      else dev::acquireFence();
+    }
+    return ready;
+  }
+
   // Wave-uniform wait for tile {row, col, 0} that looks ahead: the first poll reads, one per lane, the
   // semaphores of up to `count` (at most 16) tiles {row, col + i * colStep, 0} in one round trip and
   // returns how many of them, counted from the first, are posted.  If the first is not, the wave spins on

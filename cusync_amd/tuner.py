@@ -224,7 +224,7 @@ def tune_attention(seq, log, hidden=12288, heads=12):
         if best3 is None or st[2] < best3[0]:
             best3 = (st[2], t)
     bestkv = None
-    for kv in (0, 8, 16):
+    for kv in (0, 4, 8, 16):
         total, st, _ = run(api.SYNC.STREAM, tile1=best1[1], tile3=best3[1], kv_split_blocks=kv)
         log("S=%d attention with at most %d key/value blocks per workgroup: %.1f us" % (seq, kv, st[1]))
         if bestkv is None or st[1] < bestkv[0]:
