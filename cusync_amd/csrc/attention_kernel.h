@@ -210,12 +210,13 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
       for (int c = 0; c < 2; c++) {
         if (rowHi <= seenRows[c]) continue;
         const uint32_t col = (c + 1) * E + head * kHD;
-        bool oneTile = zWait || col / tnq == (col + kHD - 1) / tnq;           // the head's columns lie in one producer tile
-        if (oneTile) {
-          const uint32_t first = max(rowLo, seenRows[c]);
-          const uint32_t ready = stage.peekWaveRows(first, rangeEnd - 1, tmq, col / tnq * tnq, zWait);
-          if (ready) seenRows[c] = min(rangeEnd, (first / tmq + ready) * tmq);
+        const uint32_t first = max(rowLo, seenRows[c]);
+        uint32_t ready = 64;                       // row blocks posted in every producer column tile the head's columns meet
+        for (uint32_t ct = col / tnq * tnq; ct < col + kHD; ct += tnq) {
+          ready = min(ready, stage.peekWaveRows(first, rangeEnd - 1, tmq, ct, zWait));
+          if (zWait) break;
         }
+        if (ready) seenRows[c] = min(rangeEnd, (first / tmq + ready) * tmq);
         if (rowHi > seenRows[c]) {
           waitRows(rowLo, rowHi, col);
           seenRows[c] = max(seenRows[c], min(rangeEnd, ((rowHi - 1) / tmq + 1) * tmq));

@@ -226,7 +226,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // ---- consumer side (same protocol as the staged kernel) ------------------
     uint32_t nextColTile = (kBegin & ~(p.waitRound - 1)) / tnq;     // the first chunk's line may begin in the tile before
     const bool oneRowBlock = chunkSync && (m0 / tmq == (mEnd - 1) / tmq);
-    uint32_t readyEnd = 0;        // column tiles of the producer below this one are known to be posted (one row block)
+    uint32_t readyEnd = 0;        // column tiles of the producer below this one are known to be posted (for all row blocks of this tile)
     auto waitRows = [&](uint32_t col, uint32_t z) { stage.waitWaveRows(m0, mEnd - 1, tmq, col, z); };
     // Convolution fed by another convolution: the rows of the producer's output
     // this tile reads are its own pixels plus the filter's halo, and a K chunk
@@ -263,8 +263,9 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       const uint32_t kLast = min((min(k0 + (uint32_t)C::BK, kEnd) - 1) | (p.waitRound - 1), p.K - 1);
       for (; nextColTile <= kLast / tnq; nextColTile++) {
         if (nextColTile < readyEnd) continue;            // seen posted by an earlier look-ahead
-        if (oneRowBlock) readyEnd = nextColTile + stage.waitWaveAhead(m0, nextColTile * tnq, tnq, max(kEnd - 1, kLast) / tnq - nextColTile + 1);
-        else waitRows(nextColTile * tnq, 0);
+        const uint32_t left = max(kEnd - 1, kLast) / tnq - nextColTile + 1;      // column tiles this slice still has to see
+        if (oneRowBlock) readyEnd = nextColTile + stage.waitWaveAhead(m0, nextColTile * tnq, tnq, left);
+        else readyEnd = nextColTile + stage.waitWaveAheadRows(m0, mEnd - 1, tmq, nextColTile * tnq, tnq, left);
       }
     };
 

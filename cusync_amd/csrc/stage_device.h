@@ -284,6 +284,36 @@ struct DynStage {
     return ready;
   }
 
+  // The same look-ahead for a consumer tile that meets several row blocks of its producer (rowLo..rowHi, blocks of
+  // tileM rows): one lane per (row block, column tile), as many column tiles as fit into the wave, in one round
+  // trip.  Returns how many column tiles, counted from the first, have all their row blocks posted; if the first
+  // has not, the wave waits for that one (all its row blocks) and returns 1.
+  __device__ __forceinline__ uint32_t waitWaveAheadRows(uint32_t rowLo, uint32_t rowHi, uint32_t tileM, uint32_t col,
+                                                        uint32_t colStep, uint32_t count) const {
+    const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const uint32_t b0 = rowLo / tileM, blocks = rowHi / tileM - b0 + 1;
+    if (blocks > 32) { waitWaveRows(rowLo, rowHi, tileM, col, 0); return 1; }
+    uint32_t n = 64 / blocks;
+    if (n > count) n = count;
+    const uint32_t myCol = lane / blocks, myBlock = lane % blocks;
+    const bool inRange = myCol < n;
+    const cusync_dim3 mine = {(b0 + (inRange ? myBlock : 0u)) * tileM, col + (inRange ? myCol : 0u) * colStep, 0};
+    const bool polls = inRange && needsWait(mine);
+    const uint32_t target = waitTarget();
+    uint32_t v = 0xffffffffu;
+    if (polls) v = dev::loadRelaxed(&d.tileStatusRead[dyn::tileIndex(d.in, mine, d.prodGrid) * CUSYNC_SEM_STRIDE]);
+    const uint64_t pending = __ballot(inRange && v < target);
+    uint32_t ready = pending ? (uint32_t)__builtin_ctzll(pending) / blocks : n;      // lanes are ordered by column tile
+    if (ready > n) ready = n;
+    if (ready == 0) {
+      waitWaveRows(rowLo, rowHi, tileM, col, 0);          // spins, fences, counts a time-out
+      return 1;
+    }
+    if (lineAligned) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    else dev::acquireFence();
+    return ready;
+  }
+
   // Workgroup-wide post; contains a barrier, call from all threads.  `times`: how many posts of the policy this
   // one stands for (a workgroup that finished several logical tiles guarded by one semaphore adds them at once).
   __device__ __forceinline__ void post(const cusync_dim3& tile, uint32_t times = 1) const {
