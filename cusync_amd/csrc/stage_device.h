@@ -257,15 +257,15 @@ struct DynStage {
   }
 
   // Wave-uniform wait for tile {row, col, 0} that looks ahead: the first poll reads, one per lane, the
-  // semaphores of up to `count` (at most 16) tiles {row, col + i * colStep, 0} in one round trip and
+  // semaphores of up to `count` (at most 64) tiles {row, col + i * colStep, 0} in one round trip and
   // returns how many of them, counted from the first, are posted.  If the first is not, the wave spins on
-  // that one alone (sixteen lanes polling for as long as the producer needs would be sixteen times the
+  // that one alone (all lanes polling for as long as the producer needs would be that many times the
   // traffic on the semaphores) and returns 1.  A consumer that is several tiles behind its producer
-  // then polls once per sixteen tiles instead of once per tile; every poll is a round trip to memory
+  // then polls once per sixty-four tiles instead of once per tile; every poll is a round trip to memory
   // that the loads already in flight have to drain behind.
   __device__ __forceinline__ uint32_t waitWaveAhead(uint32_t row, uint32_t col, uint32_t colStep, uint32_t count) const {
     const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    const uint32_t n = count < 16u ? count : 16u;
+    const uint32_t n = count < 64u ? count : 64u;
     const cusync_dim3 mine = {row, col + (lane < n ? lane : 0u) * colStep, 0};
     const bool polls = lane < n && needsWait(mine);
     const uint32_t target = waitTarget();
