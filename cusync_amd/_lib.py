@@ -40,7 +40,7 @@ class GemmArgs(C.Structure):
     _fields_ = [("stage", StageDesc), ("M", u32), ("N", u32), ("K", u32),
                 ("A", vp), ("lda", u32), ("B", vp), ("ldb", u32), ("D", vp), ("ldd", u32),
                 ("epilogue", i32), ("a_mode", i32), ("tile", i32), ("split_k", i32),
-                ("workspace", vp), ("max_workgroups", i32)]
+                ("workspace", vp), ("max_workgroups", i32), ("shared_reduction", i32)]
 
 
 class Conv2dArgs(C.Structure):

@@ -184,7 +184,7 @@ def gemm_grid(tile, M, N, split_k=1):
 
 
 def gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, epilogue=EPI.NONE, a_mode=0, split_k=1,
-              max_workgroups=0, workspace=None):
+              max_workgroups=0, workspace=None, shared_reduction=0):
     a = GemmArgs()
     a.stage = stage.desc
     a.M, a.N, a.K = M, N, K
@@ -192,6 +192,7 @@ def gemm_args(stage, M, N, K, A, lda, B, ldb, D, ldd, tile, epilogue=EPI.NONE, a
     a.epilogue, a.a_mode, a.tile, a.split_k = epilogue, a_mode, tile, split_k
     a.workspace = workspace
     a.max_workgroups = max_workgroups
+    a.shared_reduction = shared_reduction
     return a
 
 

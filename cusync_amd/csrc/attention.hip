@@ -352,7 +352,7 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     a1.stage = L->st[0]; a1.M = S; a1.N = 3 * E; a1.K = H;
     a1.A = x; a1.lda = H; a1.B = L->wqkv; a1.ldb = 3 * E; a1.ldd = 3 * E;
     a1.D = (char*)qkv + (size_t)L->cfg.cached_rows * 3 * E * 2;       // behind the cache rows (attention.cu:289)
-    a1.tile = L->tile1; a1.split_k = L->split1; a1.workspace = L->ws1;
+    a1.tile = L->tile1; a1.split_k = L->split1; a1.workspace = L->ws1; a1.shared_reduction = 1;
     cusync_attention_args a2;
     memset(&a2, 0, sizeof a2);
     a2.stage = L->st[1]; a2.seq = S; a2.heads = L->cfg.heads; a2.head_dim = kHD;
@@ -361,7 +361,7 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     a2.kv_split_blocks = L->kvSplit; a2.workspace = L->ws2;
     a3.stage = L->st[2]; a3.M = S; a3.N = H; a3.K = E;
     a3.A = o; a3.lda = E; a3.B = L->wo; a3.ldb = H; a3.D = y; a3.ldd = H;
-    a3.tile = L->tile3; a3.split_k = L->split3; a3.workspace = L->ws3;
+    a3.tile = L->tile3; a3.split_k = L->split3; a3.workspace = L->ws3; a3.shared_reduction = 1;
 
     hipStream_t s0 = L->stream[0], s1 = overlapped ? L->stream[1] : s0, s2 = overlapped ? L->stream[2] : s0;
     cusync_error e;

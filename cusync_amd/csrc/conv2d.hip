@@ -123,6 +123,7 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
   p.mPad = s.grid.y * ti->bm;
   p.waitRound = 1;
+  p.coopReduce = 0; p.partialBytes = 0;
   p.timeline = nullptr; p.timelineCap = 0;
   // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&

@@ -37,7 +37,13 @@ struct GemmParams {
   // split-K: slice z of a tile covers K columns [z*kPerSlice, (z+1)*kPerSlice)
   uint32_t splitK, kPerSlice;
   float* partials;         // [splitK][m-tiles][n-tiles][BM*BN] fp32 partial sums in register order
-  uint32_t* arrivals;      // [m-tiles * n-tiles] slices finished per output tile; 0 between launches
+  uint32_t* arrivals;      // [2][m-tiles * n-tiles] slices that wrote their partial sums / that stored their share, per output tile; 0 between launches
+  // Split-K where every k-slice of the launch has a workgroup of its own from the start (one round, all resident):
+  // the slices of a tile wait for each other and each adds up and stores a share of the tile (whole 32-row
+  // pieces of it), instead of the slice that arrives last doing all of it while the others' CUs idle.  Set by the
+  // launcher; needs BM/32 to be a multiple of splitK.
+  uint32_t coopReduce;
+  uint32_t partialBytes;   // size of `partials`, for the buffer descriptor of the write-through stores
   uint32_t mPad;           // m-tiles * BM
   // Consumer whose producer's tiles are not whole 128-byte lines of A (a tile policy with a tile width that is
   // not a multiple of 64 halfs): 64, and every wait of a K chunk then covers all producer column tiles that
@@ -167,6 +173,106 @@ __device__ __forceinline__ void schedPass() {
   }
 }
 
+// Stores of an output tile.  Final values go through LDS so that global memory sees whole rows: a lane holds 4
+// consecutive columns of 32 different rows, which stored directly would be 8-byte pieces scattered over 32 cache
+// lines per instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
+// applied) into a [WM*32][BN] buffer (rows padded by 16 bytes against bank conflicts), then all threads copy the
+// buffer out, 16 bytes per lane, consecutive lanes along a row.
+// pass(i, rows, value): MFMA row tile i of every wave, value(j, g) its four floats of tile j, group g; bit w of
+// `rows` set = the waves of wave row w write their 32 rows of this pass and those rows are stored.
+// CUSYNC_EPILOGUE_SWIGLU: the tile's columns are gate and up columns in alternating groups of eight, and in the
+// MFMA result layout group g of a lane is columns 8g + 4*(lane/32) + 0..3 of its 32-column tile: groups 0 and 2
+// are gate values, groups 1 and 3 the up values of the same output columns.  The tile's output is BN/2 wide.
+template<class C>
+struct TileStore {
+  const GemmParams& p;
+  char* lds;
+  uint32_t m0, n0;
+  int wm, wn, lane;
+  bool through;
+  __amdgpu_buffer_rsrc_t rD;
+  static constexpr uint32_t kAllRows = (1u << C::WM) - 1;
+
+  __device__ __forceinline__ TileStore(const GemmParams& p_, const cusync_dim3& t, int wm_, int wn_, int lane_, char* lds_)
+      : p(p_), lds(lds_), m0(t.y * C::BM), n0(t.x * C::BN), wm(wm_), wn(wn_), lane(lane_), through(p_.stage.isProducer()),
+        rD(makeRsrc(p_.D, p_.M * p_.ldd * 2)) {}
+
+  template<class V>
+  __device__ __forceinline__ void passPairs(int i, uint32_t rows, V&& value) const {
+    constexpr int PITCH = C::BN + 16;                 // BN/2 halfs and the pad
+    constexpr int ROWS = C::WM * 32;
+    constexpr int CPR = C::BN / 16;
+    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
+    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
+    constexpr int STEPS = ROWS * CPR / C::THREADS;
+    __syncthreads();
+    if ((rows >> wm) & 1) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int gp = 0; gp < 2; gp++) {
+          const floatx4 vg = value(j, 2 * gp), vu = value(j, 2 * gp + 1);
+          half4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) o[e] = (half_t)(siluf(vg[e]) * vu[e]);
+          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * (C::WTN / 2) + j * 16 + 8 * gp + 4 * (lane >> 5)) * 2) = o;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+      const uint32_t idx = s * C::THREADS + threadIdx.x;
+      const uint32_t lr = idx / CPR, c = idx % CPR;
+      const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 / 2 + c * 8;
+      if (m < p.M && n < p.N / 2 && ((rows >> (lr / 32)) & 1)) {
+        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
+        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
+      }
+    }
+  }
+
+  template<class V>
+  __device__ __forceinline__ void pass(int i, uint32_t rows, V&& value) const {
+    if (p.epilogue == CUSYNC_EPILOGUE_SWIGLU) { passPairs(i, rows, value); return; }
+    constexpr int PITCH = C::BN * 2 + 16;
+    constexpr int ROWS = C::WM * 32;
+    constexpr int CPR = C::BN / 8;
+    constexpr int STEPS = ROWS * CPR / C::THREADS;
+    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
+    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
+    __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
+    if ((rows >> wm) & 1) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const floatx4 v = value(j, g);
+          half4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
+          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = o;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+      const uint32_t idx = s * C::THREADS + threadIdx.x;
+      const uint32_t lr = idx / CPR, c = idx % CPR;
+      const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
+      if (m < p.M && n < p.N && ((rows >> (lr / 32)) & 1)) {
+        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+        // A producer's output is written through to memory (device scope) as it is stored: the release of the
+        // post then finds no dirty lines of it in this XCD's L2.  Left to the post, every one of the workgroups
+        // of an XCD that finish together starts a write-back of the whole L2 (measured: the producer of the
+        // 2048-row MLP runs 5 us longer than the same kernel without a post).
+        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
+        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
+      }
+    }
+  }
+};
+
 // Writes the accumulators of one output tile and tells the caller whether this
 // workgroup completed the tile (and therefore posts it).
 //
@@ -180,116 +286,122 @@ __device__ __forceinline__ void schedPass() {
 // does not depend on arrival order — applies the epilogue, stores, re-arms the
 // counter and posts.  Must be called by all threads of the workgroup.
 template<class C>
+__device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
+                                                const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds);
+
+template<class C>
 __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
                                            const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
-  const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
-  const bool through = p.stage.isProducer();
-  const __amdgpu_buffer_rsrc_t rD = makeRsrc(p.D, p.M * p.ldd * 2);
-  // Final values go through LDS so that global memory sees whole rows: a lane holds 4 consecutive columns of
-  // 32 different rows, which stored directly would be 8-byte pieces scattered over 32 cache lines per
-  // instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
-  // applied) into a [WM*32][BN] buffer (rows padded by 16 bytes against bank conflicts), then all threads
-  // copy the buffer out, 16 bytes per lane, consecutive lanes along a row.
-  // storePass(i, value): MFMA row tile i of every wave, value(j, g) its four floats of tile j, group g.
-  // CUSYNC_EPILOGUE_SWIGLU: the tile's columns are gate and up columns in alternating groups of eight, and in the
-  // MFMA result layout group g of a lane is columns 8g + 4*(lane/32) + 0..3 of its 32-column tile: groups 0 and 2
-  // are gate values, groups 1 and 3 the up values of the same output columns.  The tile's output is BN/2 wide.
-  auto storePassPairs = [&](int i, auto&& value) {
-    constexpr int PITCH = C::BN + 16;                 // BN/2 halfs and the pad
-    constexpr int ROWS = C::WM * 32;
-    constexpr int CPR = C::BN / 16;
-    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
-    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
-    constexpr int STEPS = ROWS * CPR / C::THREADS;
-    __syncthreads();
+  if (p.splitK > 1) return finishTileSplit<C>(p, acc, t, wm, wn, lane, sLast, lds);
+  const TileStore<C> store(p, t, wm, wn, lane, lds);
 #pragma unroll
-    for (int j = 0; j < C::TN; j++)
-#pragma unroll
-      for (int gp = 0; gp < 2; gp++) {
-        const floatx4 vg = value(j, 2 * gp), vu = value(j, 2 * gp + 1);
-        half4 o;
-#pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = (half_t)(siluf(vg[e]) * vu[e]);
-        *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * (C::WTN / 2) + j * 16 + 8 * gp + 4 * (lane >> 5)) * 2) = o;
-      }
-    __syncthreads();
-#pragma unroll
-    for (int s = 0; s < STEPS; s++) {
-      const uint32_t idx = s * C::THREADS + threadIdx.x;
-      const uint32_t lr = idx / CPR, c = idx % CPR;
-      const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 / 2 + c * 8;
-      if (m < p.M && n < p.N / 2) {
-        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
-        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
-        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
-      }
-    }
-  };
-  auto storePass = [&](int i, auto&& value) {
-    if (p.epilogue == CUSYNC_EPILOGUE_SWIGLU) { storePassPairs(i, value); return; }
-    constexpr int PITCH = C::BN * 2 + 16;
-    constexpr int ROWS = C::WM * 32;
-    constexpr int CPR = C::BN / 8;
-    constexpr int STEPS = ROWS * CPR / C::THREADS;
-    static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
-    static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
-    {
-      __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
-#pragma unroll
-      for (int j = 0; j < C::TN; j++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const floatx4 v = value(j, g);
-          half4 o;
-#pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
-          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = o;
-        }
-      __syncthreads();
-#pragma unroll
-      for (int s = 0; s < STEPS; s++) {
-        const uint32_t idx = s * C::THREADS + threadIdx.x;
-        const uint32_t lr = idx / CPR, c = idx % CPR;
-        const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
-        if (m < p.M && n < p.N) {
-          const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
-          // A producer's output is written through to memory (device scope) as it is stored: the release of the
-          // post then finds no dirty lines of it in this XCD's L2.  Left to the post, every one of the workgroups
-          // of an XCD that finish together starts a write-back of the whole L2 (measured: the producer of the
-          // 2048-row MLP runs 5 us longer than the same kernel without a post).
-          if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
-          else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
-        }
-      }
-    }
-  };
-  if (p.splitK <= 1) {
-#pragma unroll
-    for (int i = 0; i < C::TM; i++)
-      storePass(i, [&](int j, int g) {
-        return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-      });
-    return true;
-  }
+  for (int i = 0; i < C::TM; i++)
+    store.pass(i, TileStore<C>::kAllRows, [&](int j, int g) {
+      return floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+    });
+  return true;
+}
+
+// The k-slices' part of finishTile.  Nothing in it may need the accumulators once they are written to the
+// workspace: with them alive next to a slice's worth of loads in flight the compiler runs out of registers and
+// spills in the main loop of the 256-row tiles (the 512-row GEMM1's k loop went from 73 to 162 us).  As a function
+// of its own (not inlined) it costs more still: the kernel then keeps a stack and the same k loop takes 130 us.
+template<class C>
+__device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
+                                                const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
+  const TileStore<C> store(p, t, wm, wn, lane, lds);
+  constexpr uint32_t kAllRows = TileStore<C>::kAllRows;
   // Partial sums live in the workspace in register order: value g of MFMA tile (i, j) of every thread is one
-  // contiguous run (16 bytes per thread), so slices write and the finishing slice reads with fully
-  // coalesced accesses; the padding rows and columns of edge tiles are carried along.
+  // contiguous run (16 bytes per thread), so slices write and read with fully coalesced accesses; the padding rows
+  // and columns of edge tiles are carried along.  They are written through to memory (sc1): the release that
+  // follows then has nothing of them to write back, and the slices that read them do so with device-coherent loads.
   constexpr size_t kTileFloats = (size_t)C::BM * C::BN;
   const size_t sliceStride = (size_t)p.stage.d.grid.x * p.stage.d.grid.y * kTileFloats;
-  float* mine = p.partials + ((size_t)t.y * p.stage.d.grid.x + t.x) * kTileFloats + (size_t)threadIdx.x * 4;
+  const size_t tileOffset = ((size_t)t.y * p.stage.d.grid.x + t.x) * kTileFloats + (size_t)threadIdx.x * 4;      // in floats
+  float* mine = p.partials + tileOffset;
   auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (C::THREADS * 4); };
+  const __amdgpu_buffer_rsrc_t rPart = makeRsrc(p.partials, p.partialBytes);
+  auto partOffset = [&](uint32_t z, int i, int j, int g) { return (uint32_t)((tileOffset + z * sliceStride + slot(i, j, g)) * sizeof(float)); };
 #pragma unroll
   for (int i = 0; i < C::TM; i++)
 #pragma unroll
     for (int j = 0; j < C::TN; j++)
 #pragma unroll
-      for (int g = 0; g < 4; g++)
-        *reinterpret_cast<floatx4*>(mine + t.z * sliceStride + slot(i, j, g)) =
-            floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+      for (int g = 0; g < 4; g++) {
+        const floatx4 v = floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, v), rPart, (int)partOffset(t.z, i, j, g), 0, 16 /* sc1 */);
+      }
   // the release below is the first thread's and covers its own wavefront's stores; the others see theirs through here
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  uint32_t* counter = p.arrivals + t.y * p.stage.d.grid.x + t.x;
+  const uint32_t tileIndex = t.y * p.stage.d.grid.x + t.x;
+  uint32_t* counter = p.arrivals + tileIndex;
+
+  if (p.coopReduce) {
+    // ---- every slice adds up and stores its share ---------------------------------------------------------
+    // The tile is cut into BM/32 pieces of 32 rows (piece u = i * WM + wm: MFMA row tile i of wave row wm); slice z
+    // takes the pieces [z * U/S, (z + 1) * U/S).  A piece is summed over the slices in index order (this slice's
+    // own term read back like the others: see above), so the result is the same, bit for bit, whichever way and
+    // in whatever order of arrival the tile is put together.
+    constexpr uint32_t U = C::TM * C::WM;
+    const uint32_t perSlice = U / p.splitK;
+    uint32_t* departures = p.arrivals + p.stage.d.grid.x * p.stage.d.grid.y + tileIndex;
+    if (threadIdx.x == 0) {
+      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      if (!dev::pollUntilAtLeast(counter, p.splitK)) dev::countGiveUp(p.stage.d.spinTimeouts);     // the siblings are resident: bounded all the same
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+      const uint32_t u = (uint32_t)i * C::WM + (uint32_t)wm;
+      const bool owned = u / perSlice == t.z;                               // uniform per wavefront
+      const uint32_t firstPiece = t.z * perSlice, endPiece = firstPiece + perSlice;
+      // wave rows of this pass that belong to this slice
+      uint32_t rows = 0;
+#pragma unroll
+      for (uint32_t w = 0; w < (uint32_t)C::WM; w++) { const uint32_t q = (uint32_t)i * C::WM + w; if (q >= firstPiece && q < endPiece) rows |= 1u << w; }
+      if (rows == 0) continue;                                              // uniform per workgroup
+      floatx4 sum[C::TN][4];
+      if (owned) {
+        // two slices' worth of loads in flight at a time; this slice's own term is read back like the others
+        for (uint32_t z = 0; z < p.splitK; z += 2) {
+          uint4v v[2][C::TN][4];
+#pragma unroll
+          for (uint32_t q = 0; q < 2; q++) {
+            if (z + q >= p.splitK) break;
+#pragma unroll
+            for (int j = 0; j < C::TN; j++)
+#pragma unroll
+              for (int g = 0; g < 4; g++) v[q][j][g] = __builtin_amdgcn_raw_buffer_load_b128(rPart, (int)partOffset(z + q, i, j, g), 0, 16 /* sc1 */);
+          }
+#pragma unroll
+          for (uint32_t q = 0; q < 2; q++) {
+            if (z + q >= p.splitK) break;
+#pragma unroll
+            for (int j = 0; j < C::TN; j++)
+#pragma unroll
+              for (int g = 0; g < 4; g++) {
+                const floatx4 term = __builtin_bit_cast(floatx4, v[q][j][g]);
+                sum[j][g] = (z + q == 0) ? term : sum[j][g] + term;
+              }
+          }
+        }
+      }
+      store.pass(i, rows, [&](int j, int g) { return sum[j][g]; });
+    }
+    // the slice that stores its share last re-arms the counters and has the tile to post
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t before = __hip_atomic_fetch_add(departures, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = before == p.splitK - 1;
+      if (last) { dev::storeRelaxed(counter, 0); dev::storeRelaxed(departures, 0); }
+      *sLast = last;
+    }
+    __syncthreads();
+    return *sLast != 0;
+  }
+
   if (threadIdx.x == 0) {
     // release only: an acquire here would empty this XCD's L2 once per slice; the finishing slice acquires below
     const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -304,8 +416,7 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
   // of that row for one slice are issued together (TN * 4 of 16 bytes per thread).  One position at a time
   // would be a chain of round trips to memory as long as the GEMM itself; everything at once, accumulated
   // into `acc`, makes the compiler spill in the main loop.  (Letting all slices wait for each other and add
-  // up a share each was measured and is slower: every waiting slice ends with an acquire that empties its
-  // XCD's L2 under the workgroups still streaming weights; the GPT-3 MLP at one row went from 108 to 156 us.)
+  // up a share each is the path above; it needs every slice to have a workgroup of its own from the start.)
   // Narrow wavefront tiles have few loads per slice: several slices are fetched together (G of them, up to 16
   // loads of 16 bytes per thread in flight), still added in index order.
   constexpr int G = C::TN * 4 >= 16 ? 1 : 16 / (C::TN * 4);
@@ -332,7 +443,7 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
           for (int g = 0; g < 4; g++) sum[j][g] = (z + q == 0) ? v[q][j][g] : sum[j][g] + v[q][j][g];
       }
     }
-    storePass(i, [&](int j, int g) { return sum[j][g]; });
+    store.pass(i, kAllRows, [&](int j, int g) { return sum[j][g]; });
   }
   return true;
 }

@@ -117,6 +117,8 @@ cusync_dim3 cusync_gemm_grid(int tile, uint32_t M, uint32_t N, int split_k) {
 
 int cusync_gemm_max_resident(int tile) { return residentWorkgroups(tile); }
 
+static size_t partialBytes(const cusync_gemm_args* a, const TileInfo* ti);
+
 cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   using cusync::rt::setError;
   if (!a) return CUSYNC_ERROR_NOT_INITIALIZED;
@@ -140,6 +142,7 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
     if ((uint32_t)a->split_k > (a->K + ti->bk - 1) / ti->bk) { setError("gemm: more k-slices than K chunks"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (!a->workspace || (uintptr_t)a->workspace % 16) { setError("gemm: split_k > 1 needs a 16-byte aligned workspace of cusync_gemm_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (partialBytes(a, ti) >= 0x80000000ull) { setError("gemm: the partial sums of these k-slices exceed 2 GiB, more than one buffer descriptor addresses"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   }
   if (a->a_mode != CUSYNC_A_PLAIN && a->a_mode != CUSYNC_A_SWIGLU) { setError("gemm: unknown a_mode"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_SWIGLU) { setError("gemm: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
@@ -165,7 +168,7 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
 }
 
 // [split_k][m-tiles][n-tiles][BM*BN] fp32 partial sums (each tile in the order its workgroup holds it in
-// registers), then one arrival counter per output tile.
+// registers), then two counters per output tile (slices that wrote their partial sums, slices that stored their share).
 static size_t partialBytes(const cusync_gemm_args* a, const TileInfo* ti) {
   const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
   return (size_t)a->split_k * g.y * g.x * ti->bm * ti->bn * sizeof(float);
@@ -201,6 +204,11 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   cusync::rt::timeline(&p.timeline, &p.timelineCap);
   p.partials = (float*)a->workspace;
   p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
+  p.partialBytes = a->split_k > 1 ? (uint32_t)partialBytes(a, ti) : 0;
+  // every k-slice has its own workgroup from the start, and the tile's 32-row pieces divide among the slices
+  const bool direct = ti->chainKernel != nullptr;
+  p.coopReduce = a->split_k > 1 && a->shared_reduction != 0 && direct && p.stage.noDraws && launched == s.grid.x * s.grid.y * s.grid.z &&
+                 (ti->bm / 32) % (uint32_t)a->split_k == 0 && !getenv("CUSYNC_NO_COOP_REDUCE");
   return p;
 }
 
@@ -208,7 +216,7 @@ size_t cusync_gemm_workspace_size(const cusync_gemm_args* a) {
   TileInfo* ti = a ? tileInfo(a->tile) : nullptr;
   if (!ti || a->split_k <= 1) return 0;
   const cusync_dim3 g = cusync_gemm_grid(a->tile, a->M, a->N, a->split_k);
-  return partialBytes(a, ti) + (size_t)g.x * g.y * sizeof(uint32_t);
+  return partialBytes(a, ti) + 2 * (size_t)g.x * g.y * sizeof(uint32_t);      // partial sums, then two counters per output tile
 }
 
 // ---- split-K workspace held by the library itself ------------------------------------------------------------
@@ -269,7 +277,7 @@ cusync_error cusync_gemm_run_static_workspace(const cusync_gemm_args* a, void* s
     // call left there is another problem's data.  The partial sums need no clearing (every slice writes its own
     // before anyone adds them up).
     const cusync_dim3 g = cusync_gemm_grid(mine.tile, mine.M, mine.N, mine.split_k);
-    const uint32_t counters = g.x * g.y;
+    const uint32_t counters = 2 * g.x * g.y;
     uint32_t* arrivals = (uint32_t*)((char*)ws + partialBytes(&mine, ti));
     hipLaunchKernelGGL(zeroWordsKernel, dim3((counters + 255) / 256), dim3(256), 0, (hipStream_t)stream, arrivals, counters);
     if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;

@@ -242,6 +242,7 @@ cusync_gemm_args gemmArgs(const cusync_mlp* m, int which, const void* x, void* h
   a.split_k = which == 0 ? m->split1 : m->split2;
   a.workspace = which == 0 ? m->ws1 : m->ws2;
   a.max_workgroups = std::max(0, which == 0 ? m->cfg.max_wg1 : m->cfg.max_wg2);
+  a.shared_reduction = 1;       // a consumer of this handle is launched only after its producer is resident
   if (which == 0) {
     a.stage = m->prod;
     a.N = m->n1; a.K = m->k1;

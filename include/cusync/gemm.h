@@ -187,6 +187,7 @@ class CuSyncGemm {
     a.split_k = split_k;
     a.workspace = workspace;
     a.max_workgroups = max_workgroups;
+    a.shared_reduction = 0;
     return a;
   }
 };

@@ -115,7 +115,7 @@ int main() {
   Gemm1::Arguments args;
   args.problem_size = GemmCoord(2048, 6144, 12288);
   args.split_k_slices = 2;
-  if (Gemm1::get_workspace_size(args) != (size_t)2 * 8 * 48 * 256 * 128 * 4 + 8 * 48 * 4) return 6;
+  if (Gemm1::get_workspace_size(args) != (size_t)2 * 8 * 48 * 256 * 128 * 4 + 2 * 8 * 48 * 4) return 6;      // partial sums, two counters per tile
   typedef CuSyncImplicitGemmConvolution<Cons, CUSYNC_CONV_TILE_128x64x32> Conv;
   const dim3 cg = Conv::get_grid_shape(Conv2dProblemSize(32, 56, 56, 64, 64));
   if (cg.x != 1 || cg.y != 32 * 56 * 56 / 128 || cg.z != 1) return 7;

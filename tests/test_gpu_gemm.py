@@ -19,7 +19,7 @@ def plain_stage(tile, M, N, split_k=1):
     return api.Stage(api.gemm_grid(tile, M, N, split_k), (1, 1, 1), api.no_sync(), api.no_sync())
 
 
-def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups=0, split_k=1, launches=1):
+def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups=0, split_k=1, launches=1, shared_reduction=0):
     import torch
     L = _lib.load()
     M = a.shape[0]
@@ -30,7 +30,8 @@ def run_gemm(a, b, tile, epilogue=api.EPI.NONE, a_mode=0, K=None, max_workgroups
     torch.cuda.synchronize()
     st = plain_stage(tile, M, N, split_k)
     args = api.gemm_args(st, M, N, K, da.data_ptr(), a.shape[1], db.data_ptr(), N, dd.data_ptr(), N, tile,
-                         epilogue=epilogue, a_mode=a_mode, max_workgroups=max_workgroups, split_k=split_k)
+                         epilogue=epilogue, a_mode=a_mode, max_workgroups=max_workgroups, split_k=split_k,
+                         shared_reduction=shared_reduction)
     ws = None
     if split_k > 1:
         ws = torch.zeros(L.cusync_gemm_workspace_size(C.byref(args)), dtype=torch.uint8, device="cuda")   # zeroed once
@@ -118,6 +119,24 @@ def test_gemm_split_k(tile, split):
     b = normal_f16((K, N), 22, std=0.05)
     got = run_gemm(a, b, tile, split_k=split, epilogue=api.EPI.GELU)
     assert_close(got, orc.gemm(a, b, orc.EPI_GELU), "split-k %d tile %d" % (split, tile))
+
+
+@pytest.mark.parametrize("tile,split", [(api.TILE.T256x192x32, 2), (api.TILE.T256x192x32, 4), (api.TILE.T256x192x32, 8),
+                                        (api.TILE.T128x192x32_ALONE, 4), (api.TILE.D64x192x64, 2), (api.TILE.T256x256x32, 4),
+                                        (api.TILE.T256x192x32, 3), (api.TILE.D32x128x64, 4)])
+def test_gemm_split_k_with_the_reduction_shared_among_the_slices(tile, split):
+    # every k-slice has a workgroup of its own, so the slices of a tile each add up and store a share of it (where
+    # the tile's 32-row pieces divide among them: not for 3 slices, not for a 32-row tile, which fall back to the
+    # last slice doing all of it).  Same sums in the same order: bit-identical to the unshared reduction, launch
+    # after launch (the counters re-arm), ragged edges included.
+    print("shared reduction tile", tile, "slices", split, flush=True)
+    M, N, K = 300, 392, 2048
+    a = uniform_f16((M, K), 31)
+    b = normal_f16((K, N), 32, std=0.05)
+    plain = run_gemm(a, b, tile, split_k=split, epilogue=api.EPI.GELU)
+    shared = run_gemm(a, b, tile, split_k=split, epilogue=api.EPI.GELU, shared_reduction=1, launches=3)
+    assert np.array_equal(plain.view(np.uint16), shared.view(np.uint16))
+    assert_close(shared, orc.gemm(a, b, orc.EPI_GELU), "shared reduction, %d slices, tile %d" % (split, tile))
 
 
 def test_gemm_split_k_is_deterministic():
