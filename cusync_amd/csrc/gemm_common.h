@@ -318,7 +318,6 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   constexpr size_t kTileFloats = (size_t)C::BM * C::BN;
   const size_t sliceStride = (size_t)p.stage.d.grid.x * p.stage.d.grid.y * kTileFloats;
   const size_t tileOffset = ((size_t)t.y * p.stage.d.grid.x + t.x) * kTileFloats + (size_t)threadIdx.x * 4;      // in floats
-  float* mine = p.partials + tileOffset;
   auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (C::THREADS * 4); };
   const __amdgpu_buffer_rsrc_t rPart = makeRsrc(p.partials, p.partialBytes);
   auto partOffset = [&](uint32_t z, int i, int j, int g) { return (uint32_t)((tileOffset + z * sliceStride + slot(i, j, g)) * sizeof(float)); };
@@ -411,15 +410,14 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   }
   __syncthreads();
   if (!*sLast) return false;
-  dev::acquireFence();
   // The slice that arrived last adds the slices in index order, one row of MFMA tiles at a time: all loads
   // of that row for one slice are issued together (TN * 4 of 16 bytes per thread).  One position at a time
   // would be a chain of round trips to memory as long as the GEMM itself; everything at once, accumulated
-  // into `acc`, makes the compiler spill in the main loop.  (Letting all slices wait for each other and add
-  // up a share each is the path above; it needs every slice to have a workgroup of its own from the start.)
-  // Narrow wavefront tiles have few loads per slice: several slices are fetched together (G of them, up to 16
-  // loads of 16 bytes per thread in flight), still added in index order.
-  constexpr int G = C::TN * 4 >= 16 ? 1 : 16 / (C::TN * 4);
+  // into `acc`, makes the compiler spill in the main loop.  The loads are coherent at device scope (sc1; the
+  // partial sums were written through), which spares the acquire fence that would empty this XCD's L2.
+  // Narrow wavefront tiles have few loads per slice: several slices are fetched together (G of them), still
+  // added in index order
+  constexpr int G = C::BM <= 64 ? 36 / (C::TN * 4) : C::TN * 4 >= 16 ? 1 : 16 / (C::TN * 4);
 #pragma unroll
   for (int i = 0; i < C::TM; i++) {
     floatx4 sum[C::TN][4];
@@ -428,11 +426,11 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
 #pragma unroll
       for (int q = 0; q < G; q++) {
         if (z + q >= p.splitK) break;
-        const float* src = mine + (z + q) * sliceStride;
 #pragma unroll
         for (int j = 0; j < C::TN; j++)
 #pragma unroll
-          for (int g = 0; g < 4; g++) v[q][j][g] = *reinterpret_cast<const floatx4*>(src + slot(i, j, g));
+          for (int g = 0; g < 4; g++)
+            v[q][j][g] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rPart, (int)partOffset(z + q, i, j, g), 0, 16 /* sc1 */));
       }
 #pragma unroll
       for (int q = 0; q < G; q++) {
