@@ -392,7 +392,11 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
-      const uint32_t before = __hip_atomic_fetch_add(departures, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      // A producer's stores must be out before the count that lets the last slice post (they were written through:
+      // the release has nothing to write back).  No acquire: nobody reads another slice's output, and an acquire
+      // would empty this XCD's L2 under the workgroups that are still in their k loops.
+      const uint32_t before = p.stage.isProducer() ? __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT)
+                                                   : __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = before == p.splitK - 1;
       if (last) { dev::storeRelaxed(counter, 0); dev::storeRelaxed(departures, 0); }
       *sLast = last;

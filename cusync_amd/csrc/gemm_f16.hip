@@ -205,10 +205,13 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   p.partials = (float*)a->workspace;
   p.arrivals = a->split_k > 1 ? (uint32_t*)((char*)a->workspace + partialBytes(a, ti)) : nullptr;
   p.partialBytes = a->split_k > 1 ? (uint32_t)partialBytes(a, ti) : 0;
-  // every k-slice has its own workgroup from the start, and the tile's 32-row pieces divide among the slices
+  // every k-slice has its own workgroup from the start, and the tile's 32-row pieces divide among the slices.
+  // Tiles of 128 rows and more only: with the small tiles of the few-row GEMMs, whose slices finish up to 10 us
+  // apart, the same scheme (also cut finer, into 32x32 pieces) ended every launch 6-12 us later than the slice
+  // that arrives last doing all of it.
   const bool direct = ti->chainKernel != nullptr;
   p.coopReduce = a->split_k > 1 && a->shared_reduction != 0 && direct && p.stage.noDraws && launched == s.grid.x * s.grid.y * s.grid.z &&
-                 (ti->bm / 32) % (uint32_t)a->split_k == 0 && !getenv("CUSYNC_NO_COOP_REDUCE");
+                 ti->bm >= 128 && (ti->bm / 32) % (uint32_t)a->split_k == 0 && !getenv("CUSYNC_NO_COOP_REDUCE");
   return p;
 }
 

@@ -260,7 +260,7 @@ typedef struct cusync_gemm_args {
   int32_t max_workgroups;      /* 0 = as many as stay resident; else cap on launched workgroups */
   int32_t shared_reduction;    /* split_k > 1.  0: the k-slice of a tile that finishes last adds up all slices and stores
                                   the tile.  1: where every k-slice of the launch has a workgroup of its own from the start
-                                  (no more tiles than workgroups stay resident) and tileM/32 is a multiple of split_k, the
+                                  (no more tiles than workgroups stay resident), tileM is at least 128 and tileM/32 is a multiple of split_k, the
                                   slices of a tile wait for each other and each adds up and stores a share; same sums in
                                   the same order, so bit-identical results.  The waiting slices hold their CUs: only for
                                   launches whose workgroups no other kernel keeps off the device while it waits for them

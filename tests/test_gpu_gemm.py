@@ -126,8 +126,8 @@ def test_gemm_split_k(tile, split):
                                         (api.TILE.T256x192x32, 3), (api.TILE.D32x128x64, 4)])
 def test_gemm_split_k_with_the_reduction_shared_among_the_slices(tile, split):
     # every k-slice has a workgroup of its own, so the slices of a tile each add up and store a share of it (where
-    # the tile's 32-row pieces divide among them: not for 3 slices, not for a 32-row tile, which fall back to the
-    # last slice doing all of it).  Same sums in the same order: bit-identical to the unshared reduction, launch
+    # the tile has 128 rows or more and its 32-row pieces divide among them: not for 3 slices, not for the 64- and
+    # 32-row tiles, which fall back to the last slice doing all of it).  Same sums in the same order: bit-identical to the unshared reduction, launch
     # after launch (the counters re-arm), ragged edges included.
     print("shared reduction tile", tile, "slices", split, flush=True)
     M, N, K = 300, 392, 2048
