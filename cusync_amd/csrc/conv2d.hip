@@ -172,7 +172,9 @@ cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
     return CUSYNC_ERROR_NOT_INITIALIZED;
   }
   if (a->K % 8) { setError("conv2d: output channels must be a multiple of 8"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  if ((uint64_t)a->N * a->H * a->W * a->C * 2 >= 0x80000000ull || (uint64_t)a->K * a->R * a->S * a->C * 2 >= 0x80000000ull) {
+  const uint64_t outRows = (uint64_t)((a->H + 2 * a->pad - a->R) / a->stride + 1) * ((a->W + 2 * a->pad - a->S) / a->stride + 1) * a->N;
+  if ((uint64_t)a->N * a->H * a->W * a->C * 2 >= 0x80000000ull || (uint64_t)a->K * a->R * a->S * a->C * 2 >= 0x80000000ull ||
+      outRows * a->K * 2 >= 0x80000000ull) {
     setError("conv2d: operand larger than 2 GiB is not addressable by one buffer descriptor");
     return CUSYNC_ERROR_NOT_INITIALIZED;
   }

@@ -224,11 +224,11 @@ struct TileStore {
       const uint32_t idx = s * C::THREADS + threadIdx.x;
       const uint32_t lr = idx / CPR, c = idx % CPR;
       const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 / 2 + c * 8;
-      if (m < p.M && n < p.N / 2 && ((rows >> (lr / 32)) & 1)) {
-        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
-        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
-        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
-      }
+      const bool inside = m < p.M && n < p.N / 2 && ((rows >> (lr / 32)) & 1);
+      const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+      const int off = inside ? (int)((m * p.ldd + n) * 2) : (int)kOutOfRange;
+      if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, off, 0, 16 /* sc1 */);
+      else __builtin_amdgcn_raw_buffer_store_b128(v, rD, off, 0, 0);
     }
   }
 
@@ -260,15 +260,19 @@ struct TileStore {
       const uint32_t idx = s * C::THREADS + threadIdx.x;
       const uint32_t lr = idx / CPR, c = idx % CPR;
       const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
-      if (m < p.M && n < p.N && ((rows >> (lr / 32)) & 1)) {
-        const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
-        // A producer's output is written through to memory (device scope) as it is stored: the release of the
-        // post then finds no dirty lines of it in this XCD's L2.  Left to the post, every one of the workgroups
-        // of an XCD that finish together starts a write-back of the whole L2 (measured: the producer of the
-        // 2048-row MLP runs 5 us longer than the same kernel without a post).
-        if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, (int)((m * p.ldd + n) * 2), 0, 16 /* sc1 */);
-        else *reinterpret_cast<uint4v*>(p.D + (size_t)m * p.ldd + n) = v;
-      }
+      // Every thread issues every store, those outside the matrix (or outside `rows`) with an offset the buffer
+      // descriptor rejects.  With the stores (and the LDS reads that feed them) under a condition, as plain stores
+      // through a pointer, the compiler serialised each read with its store: the 2048-row MLP step was 13 us
+      // longer (three tiles per workgroup, 4 us each).
+      const bool inside = m < p.M && n < p.N && ((rows >> (lr / 32)) & 1);
+      const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
+      const int off = inside ? (int)((m * p.ldd + n) * 2) : (int)kOutOfRange;
+      // A producer's output is written through to memory (device scope) as it is stored: the release of the
+      // post then finds no dirty lines of it in this XCD's L2.  Left to the post, every one of the workgroups
+      // of an XCD that finish together starts a write-back of the whole L2 (measured: the producer of the
+      // 2048-row MLP runs 5 us longer than the same kernel without a post).
+      if (through) __builtin_amdgcn_raw_buffer_store_b128(v, rD, off, 0, 16 /* sc1 */);
+      else __builtin_amdgcn_raw_buffer_store_b128(v, rD, off, 0, 0);
     }
   }
 };

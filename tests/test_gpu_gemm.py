@@ -103,6 +103,29 @@ def test_gemm_persistent_launch_smaller_than_grid():
     assert_close(got, orc.gemm(a, b), "persistent")
 
 
+@pytest.mark.parametrize("tile", [api.TILE.T256x192x32, api.TILE.T256x256x32, api.TILE.T256x128x32, api.TILE.T128x128x32,
+                                  api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x192x32_ALONE, api.TILE.D64x192x64])
+@pytest.mark.parametrize("K", [24, 200, 1032])
+def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
+    # 3 workgroups for 12 to 88 tiles with ragged edges: every workgroup goes from one tile's stores straight into
+    # the next tile's loads, and the stores outside the matrix are issued all the same (with an offset the buffer
+    # descriptor rejects).  K = 24 is a single, partly filled chunk (fewer chunks than pipeline stages), 200 a
+    # few, 1032 many and a ragged last one.  Two launches, GeLU epilogue.
+    print("several tiles per workgroup, tile", tile, "K", K, flush=True)
+    M, N = 600, 1000
+    a = uniform_f16((M, K), 41)
+    b = normal_f16((K, N), 42, std=0.05)
+    got = run_gemm(a, b, tile, epilogue=api.EPI.GELU, max_workgroups=3, launches=2)
+    assert_close(got, orc.gemm(a, b, orc.EPI_GELU), "tile %d K %d" % (tile, K))
+    # exact arithmetic: any chunk read before it arrived, or read from a stage the next tile's loads had
+    # already overwritten, changes an integer sum
+    rng = np.random.default_rng(tile * 100 + K)
+    a = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    b = rng.integers(-2, 3, (K, N)).astype(np.float16)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float16)
+    assert np.array_equal(run_gemm(a, b, tile, max_workgroups=3), want)
+
+
 @pytest.mark.parametrize("tile", [api.TILE.T128x128x64, api.TILE.T32x128x64, api.TILE.T128x256x32, api.TILE.T256x256x32,
                                   api.TILE.T128x128x32])
 @pytest.mark.parametrize("split", [2, 3, 8])
@@ -243,6 +266,20 @@ def test_two_chained_gemms_config1(policy_kind, opts, tiles):
     assert np.array_equal(ps.sems, want_sems)                 # bit-exact semaphore end state
     assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
     assert ps.kernel_executed == iters
+
+
+@pytest.mark.parametrize("policy_kind", ["row", "tile"])
+@pytest.mark.parametrize("tile", [api.TILE.T256x192x32, api.TILE.T128x128x32])
+def test_chained_direct_to_lds_gemms_with_few_workgroups(policy_kind, tile):
+    # 24 to 72 tiles per GEMM on 5 workgroups each, K with a ragged last chunk: every workgroup works through
+    # several tickets of the producer and of the consumer, and a producer workgroup's post follows all of its
+    # tile's stores.
+    print("chained, few workgroups", policy_kind, tile, flush=True)
+    a, b, d, c, e, ps, cs, want_sems = chained(768, 1536, 520, tile, tile, policy_kind, iters=3, max_wg=5)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d), "E")
+    assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3
+    assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
 
 
 def test_chained_gemms_with_few_workgroups():
