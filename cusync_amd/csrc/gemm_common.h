@@ -261,9 +261,10 @@ struct TileStore {
       const uint32_t lr = idx / CPR, c = idx % CPR;
       const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
       // Every thread issues every store, those outside the matrix (or outside `rows`) with an offset the buffer
-      // descriptor rejects.  With the stores (and the LDS reads that feed them) under a condition, as plain stores
-      // through a pointer, the compiler serialised each read with its store: the 2048-row MLP step was 13 us
-      // longer (three tiles per workgroup, 4 us each).
+      // descriptor rejects.  With the read and the store under a condition (a divergent branch around each) and,
+      // for a stage that is no producer, the store through a 64-bit pointer, the 2048-row MLP step was 13 us
+      // longer (three tiles per workgroup, 4 us each).  Reading all of a pass's pieces from LDS ahead of its
+      // first store was measured too: 2 us slower than one after the other.
       const bool inside = m < p.M && n < p.N && ((rows >> (lr / 32)) & 1);
       const uint4v v = *reinterpret_cast<const uint4v*>(lds + lr * PITCH + c * 16);
       const int off = inside ? (int)((m * p.ldd + n) * 2) : (int)kOutOfRange;
