@@ -135,6 +135,8 @@ def test_conv_can_implement_rejects():
     assert rc(stride=0) != api.ERR.SUCCESS
     assert rc(epilogue=7) != api.ERR.SUCCESS
     assert "conv2d" in api.last_error()
+    # input 0.5 GiB, output 2 GiB (four times the channels): the output no longer fits one buffer descriptor
+    assert rc(N=64, H=256, W=256, Cc=64, K=256) != api.ERR.SUCCESS and "2 GiB" in api.last_error()
     halo = api.CONV_TILE.HALO_256x64x64
     assert rc(tile=halo) == api.ERR.SUCCESS
     assert rc(tile=halo, stride=2) != api.ERR.SUCCESS and rc(tile=halo, pad=0) != api.ERR.SUCCESS
