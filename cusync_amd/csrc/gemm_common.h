@@ -326,15 +326,32 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   auto slot = [](int i, int j, int g) { return (size_t)((i * C::TN + j) * 4 + g) * (C::THREADS * 4); };
   const __amdgpu_buffer_rsrc_t rPart = makeRsrc(p.partials, p.partialBytes);
   auto partOffset = [&](uint32_t z, int i, int j, int g) { return (uint32_t)((tileOffset + z * sliceStride + slot(i, j, g)) * sizeof(float)); };
+  // Shared reduction: the pieces this slice adds up itself (see below) need not travel through memory.  Their
+  // partial sums wait in LDS behind the epilogue's buffer, every lane's own values in a place of its own, if the
+  // workgroup's LDS has room for them (a quarter of the partial-sum traffic with four slices, half with two).
+  constexpr uint32_t kPieces = C::TM * C::WM;                                   // 32-row pieces of a tile
+  constexpr uint32_t kEpiBytes = (C::WM * 32 * (C::BN * 2 + 16) + 1023) / 1024 * 1024;
+  constexpr uint32_t kPieceBytes = C::WN * C::TN * 4 * 1024;                    // 32 rows x BN columns of fp32
+  const uint32_t perSlice = p.coopReduce ? kPieces / p.splitK : 0;
+  const bool ownInLds = p.coopReduce && kEpiBytes + perSlice * kPieceBytes <= (uint32_t)C::LDS_BYTES;
+  auto ownedPiece = [&](int i) { return ((uint32_t)i * C::WM + (uint32_t)wm) / perSlice == t.z; };      // uniform per wavefront
+  auto ownSlot = [&](int i, int j, int g) {
+    const uint32_t o = (uint32_t)i * C::WM + (uint32_t)wm - t.z * perSlice;
+    return lds + kEpiBytes + ((o * C::WN + (uint32_t)wn) * (C::TN * 4) + (uint32_t)(j * 4 + g)) * 1024 + (uint32_t)lane * 16;
+  };
+  if (ownInLds) __syncthreads();         // every wavefront is out of the main loop and its loads have landed
 #pragma unroll
-  for (int i = 0; i < C::TM; i++)
+  for (int i = 0; i < C::TM; i++) {
+    const bool keep = ownInLds && ownedPiece(i);
 #pragma unroll
     for (int j = 0; j < C::TN; j++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const floatx4 v = floatx4{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, v), rPart, (int)partOffset(t.z, i, j, g), 0, 16 /* sc1 */);
+        if (keep) *reinterpret_cast<floatx4*>(ownSlot(i, j, g)) = v;
+        else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, v), rPart, (int)partOffset(t.z, i, j, g), 0, 16 /* sc1 */);
       }
+  }
   // the release below is the first thread's and covers its own wavefront's stores; the others see theirs through here
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -347,8 +364,6 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     // takes the pieces [z * U/S, (z + 1) * U/S).  A piece is summed over the slices in index order (this slice's
     // own term read back like the others: see above), so the result is the same, bit for bit, whichever way and
     // in whatever order of arrival the tile is put together.
-    constexpr uint32_t U = C::TM * C::WM;
-    const uint32_t perSlice = U / p.splitK;
     uint32_t* departures = p.arrivals + p.stage.d.grid.x * p.stage.d.grid.y + tileIndex;
     if (threadIdx.x == 0) {
       __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -357,8 +372,7 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < C::TM; i++) {
-      const uint32_t u = (uint32_t)i * C::WM + (uint32_t)wm;
-      const bool owned = u / perSlice == t.z;                               // uniform per wavefront
+      const bool owned = ownedPiece(i);
       const uint32_t firstPiece = t.z * perSlice, endPiece = firstPiece + perSlice;
       // wave rows of this pass that belong to this slice
       uint32_t rows = 0;
@@ -367,7 +381,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
       if (rows == 0) continue;                                              // uniform per workgroup
       floatx4 sum[C::TN][4];
       if (owned) {
-        // two slices' worth of loads in flight at a time; this slice's own term is read back like the others
+        // two slices' worth of loads in flight at a time; this slice's own term is read back like the others (from
+        // LDS or from memory: kept in registers it costs the main loop its registers, see above)
         for (uint32_t z = 0; z < p.splitK; z += 2) {
           uint4v v[2][C::TN][4];
 #pragma unroll
@@ -376,7 +391,9 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
 #pragma unroll
             for (int j = 0; j < C::TN; j++)
 #pragma unroll
-              for (int g = 0; g < 4; g++) v[q][j][g] = __builtin_amdgcn_raw_buffer_load_b128(rPart, (int)partOffset(z + q, i, j, g), 0, 16 /* sc1 */);
+              for (int g = 0; g < 4; g++)
+                v[q][j][g] = ownInLds && z + q == t.z ? *reinterpret_cast<const uint4v*>(ownSlot(i, j, g))
+                                                      : __builtin_amdgcn_raw_buffer_load_b128(rPart, (int)partOffset(z + q, i, j, g), 0, 16 /* sc1 */);
           }
 #pragma unroll
           for (uint32_t q = 0; q < 2; q++) {

@@ -60,7 +60,13 @@ struct DmaCfg {
   static constexpr int A_ROWS_PER_LOAD = 1024 / A_ROW_BYTES;
   static constexpr bool DUMP = B_TOTAL % WAVES != 0;
   static constexpr int DUMP_OFFSET = STAGES * (A_STAGE + B_STAGE);
-  static constexpr int LDS_BYTES = DUMP_OFFSET + (DUMP ? 1024 : 0);
+  // Beyond the pipeline stages: what a k-slice keeps in LDS while the slices of a tile add it up together (the
+  // epilogue's buffer plus the fp32 partial sums of half a tile, the share of one of two slices), as far as the
+  // workgroup's share of the CU's LDS goes (1 KiB left for the static variables).
+  static constexpr int LDS_SHARE = 160 * 1024 / (WAVES_PER_SIMD * 4 / WAVES > 0 ? WAVES_PER_SIMD * 4 / WAVES : 1) - 1024;
+  static constexpr int REDUCE_BYTES = (WM * 32 * (BN * 2 + 16) + 1023) / 1024 * 1024 + (BM / 2) * BN * 4;
+  static constexpr int PIPE_BYTES = DUMP_OFFSET + (DUMP ? 1024 : 0);
+  static constexpr int LDS_BYTES = PIPE_BYTES > LDS_SHARE ? PIPE_BYTES : REDUCE_BYTES < PIPE_BYTES ? PIPE_BYTES : REDUCE_BYTES < LDS_SHARE ? REDUCE_BYTES : LDS_SHARE;
   static_assert(WAVES == 4 || WAVES == 8, "four or eight wavefronts per workgroup");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile is made of 32x32 MFMA tiles");
   static_assert(A_CPR == 4 || A_CPR == 8, "BK is 32 or 64");
