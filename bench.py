@@ -282,12 +282,16 @@ def main():
             names = ["stream", "rowsync", "tilesync"]
             chains = [Chain(b, api.SYNC.STREAM), Chain(b, api.SYNC.ROW), Chain(b, api.SYNC.TILE)]
             tiles = chains[0].tiles
-            if tiles[0] == tiles[1]:
+            # one launch needs one tile shape for both GEMMs: left to itself the handle gives GEMM2 the tile of GEMM1
+            one_ok = tiles[0] == tiles[1] or args.tile2 < 0
+            one_tiles = None
+            if one_ok:
                 names += ["rowsync_one_launch", "tilesync_one_launch"]
                 chains += [Chain(b, api.SYNC.ROW, one_launch=True), Chain(b, api.SYNC.TILE, one_launch=True)]
+                one_tiles = list(chains[-1].tiles)
             names += ["stream_rp", "rowsync_rp"]
             chains += [Chain(b, api.SYNC.STREAM, repack=True), Chain(b, api.SYNC.ROW, repack=True)]
-            if tiles[0] == tiles[1]:
+            if one_ok:
                 names.append("rowsync_one_launch_rp")
                 chains.append(Chain(b, api.SYNC.ROW, one_launch=True, repack=True))
             times = interleaved(chains, 10, 20, split_first=True)
@@ -311,6 +315,7 @@ def main():
                 "tilesync_gain_pct": round(100 - m["tilesync"][0] / s_us * 100, 2),
                 "rowsync_one_launch_us": round(m["rowsync_one_launch"][0], 2) if "rowsync_one_launch" in m else None,
                 "tilesync_one_launch_us": round(m["tilesync_one_launch"][0], 2) if "tilesync_one_launch" in m else None,
+                "one_launch_tiles": one_tiles,
                 "best_policy": min(in_place, key=lambda k: m[k][0]),
                 "best_gain_pct": round(100 - best / s_us * 100, 2),
                 "repacked_weights": {"stream_us": round(m["stream_rp"][0], 2), "rowsync_us": round(m["rowsync_rp"][0], 2),

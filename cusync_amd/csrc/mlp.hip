@@ -191,9 +191,10 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   // Measured on the GPT-3 shard.  Where the width is a multiple of 192 (6144 and 12288 columns are 32 and
   // 64 tiles: whole rounds on 256 CUs) the 192-wide direct-to-LDS tiles win from 256 rows on.  GEMM1: 256x192
   // with a CU to itself (8 % faster than 128x192 at two workgroups per CU at 1024 and 2048 rows; below that the
-  // k-slices fill the device).  GEMM2: the same from 513 rows on; up to 512 rows, where it has at most one 128-row
-  // tile per CU, 128x192 with four stages in the pipelined order (384 rows: 258 -> 225 us, 512 rows: 254 -> 235 us
-  // for the pair against 128x192 at two workgroups per CU for both).
+  // k-slices fill the device).  GEMM2: the same from 385 rows on (at 512 rows in two k-slices whose workgroups
+  // each add up and store half a tile: 106 us against 117 us for 128x192 without slices); from 257 to 384 rows,
+  // where it has at most one 128-row tile per CU, 128x192 with four stages in the pipelined order (384 rows:
+  // 258 -> 225 us for the pair against 128x192 at two workgroups per CU for both).
   // Other widths (the LLaMA shard: 5504 and 8192 columns; the kernels mask the ragged last column tile): 128x192
   // alone on its CU up to 1024 rows, above that 256x192 for GEMM1 and 256x256 for GEMM2 (at 2048 rows 232 and 256
   // tiles: one round).  Measured against 128x128 / 128x256 at two workgroups per CU: 172 -> 147 us at 512 rows,
@@ -202,7 +203,7 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x256x32;
   if (big && n1 % 192 == 0) a = CUSYNC_TILE_256x192x32;
-  if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 512 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32_ALONE;
+  if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 384 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32_ALONE;
   // Up to 256 rows the GEMMs are bound by streaming the weights: direct-to-LDS tiles with 60-96 KB of loads
   // in flight per workgroup (measured: 104 -> 85 us at 1-32 rows, 127 -> 101 us at 64, 187 -> 158 us at 256).
   // 64x192 makes 32 or 64 column tiles, which 8 or 4 k-slices turn into one workgroup per CU.
