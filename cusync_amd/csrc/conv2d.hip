@@ -124,7 +124,7 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.mPad = s.grid.y * ti->bm;
   p.waitRound = 1;
   p.coopReduce = 0; p.partialBytes = 0;
-  p.timeline = nullptr; p.timelineCap = 0;
+  cusync::rt::timeline(&p.timeline, &p.timelineCap);
   // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
                         (a->C * 2) % 128 == 0 &&

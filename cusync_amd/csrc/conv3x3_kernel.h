@@ -91,6 +91,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
 
   uint32_t dryXcds = 0, nextRaw = 0;
+  const unsigned long long tlEntry = p.timeline ? wall_clock64() : 0;
   const uint32_t startToken = tid == 0 ? stage.beginStart() : 0;
   const bool noDraws = stage.noDraws;     // every tile is some workgroup's static first tile
   for (uint32_t round = 0;; round++) {
@@ -102,6 +103,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
       break;
     }
     const cusync_dim3 t = stage.ticketToTile(ticket);
+    const unsigned long long tl0 = p.timeline ? wall_clock64() : 0;
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
 
     // Which of the nine taps of this lane's output pixels lie inside the image: bit 3r + s.
@@ -155,6 +157,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
 #pragma unroll
     for (uint32_t it = 0; it < C::STAGES - 1; it++) issueB(it);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
+    const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
     floatx16 acc[C::TM][C::TN];
 #pragma unroll
@@ -204,11 +207,13 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     // The loads issued for chunks past the last one (zeros) may still be on their way into LDS, which the
     // epilogue is about to reuse.
     waitVmcnt<0>();
+    const unsigned long long tl2 = p.timeline ? wall_clock64() : 0;
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, 0};
     if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();
+    if (tid == 0) recordTile(p, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }
 }
 

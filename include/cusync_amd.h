@@ -113,7 +113,7 @@ typedef struct cusync_stage_desc {
 
 const char *cusync_rt_last_error(void);            /* text of the last failed HIP call, "" if none */
 /* Diagnosis, off by default.  With a device buffer set (8-byte aligned, zeroed by the caller) the direct-to-LDS GEMM
- * kernels append one record of eight 64-bit words per finished tile behind a record count in word 0: role and
+ * kernels, the 3x3 convolution kernel with the input tile in LDS and the attention kernel append one record of eight 64-bit words per finished tile behind a record count in word 0: role and
  * workgroup and XCD, tile, and the 100 MHz clock at five points of the tile (drawn, first loads issued, main loop
  * done, posted, kernel entry).  This is how the per-workgroup timelines in profiles/ were taken.  NULL switches it
  * off again; when off the kernels pay one test per tile.  No counterpart in the reference. */
