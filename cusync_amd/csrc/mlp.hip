@@ -170,12 +170,15 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // silu(gate) * up in GEMM1's epilogue: both GEMMs have plain operands and run the direct-to-LDS tiles at every
     // batch size; the kernels mask the ragged last column tile of the shard's widths (2 * 2752 and 8192).  The
     // policies count columns of the intermediate, half a GEMM1 tile wide, and no width constrains StridedSync.
-    // Measured by the tuner on the LLaMA shard (cusync_amd/tile_sizes_db.py, llama_mlp_mi355x): the 64-row tiles stay
-    // ahead up to 512 rows (232 tiles of 64x192 for GEMM1 against 116 of 128x192: 134 -> 112 us for the pair).
+    // Measured by the tuner on the LLaMA shard (cusync_amd/tile_sizes_db.py, llama_mlp_mi355x): for GEMM2 the 64-row
+    // tiles stay ahead up to 512 rows; GEMM1 from 129 rows on takes 128x192 with a CU to itself, in as many k-slices
+    // as fill the device, now that the slices share the reduction (256 rows: 54 -> 49 us against 64x192 in two
+    // slices; level at 512 rows).
     int a, b;
     if (c.batch <= 32) a = b = CUSYNC_TILE_D32x128x64;
     else if (c.batch <= 64) a = b = CUSYNC_TILE_D64x128x64;
-    else if (c.batch <= 512) { a = CUSYNC_TILE_D64x192x64; b = CUSYNC_TILE_D64x128x64; }
+    else if (c.batch <= 128) { a = CUSYNC_TILE_D64x192x64; b = CUSYNC_TILE_D64x128x64; }
+    else if (c.batch <= 512) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_D64x128x64; }
     else if (c.batch <= 1024) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_128x256x32; }
     else a = b = CUSYNC_TILE_256x256x32;
     *t1 = c.tile1 >= 0 ? c.tile1 : a;
