@@ -60,6 +60,12 @@ TileInfo* tileInfo(int tile) {
   return &g_tiles[tile];
 }
 
+// A consumer stage of a tile policy waits K chunk by K chunk; the row policies wait once per tile, and a stage
+// without an input policy not at all (same test as in the kernel).
+bool waitsPerChunk(const cusync_stage_desc& s) {
+  return s.in.kind != CUSYNC_POLICY_NOSYNC && s.in.kind != CUSYNC_POLICY_ROWSYNC && s.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC;
+}
+
 int residentWorkgroups(int tile) {
   TileInfo* ti = tileInfo(tile);
   if (!ti) return 0;
@@ -80,11 +86,12 @@ int residentWorkgroups(int tile) {
       if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel[v], (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
     }
-    if (ti->chainKernel) {
+    const void* others[2] = { reinterpret_cast<const void*>(ti->chainKernel), reinterpret_cast<const void*>(ti->kernelNoChunkWaits) };
+    for (const void* k : others) {
+      if (!k) continue;
       int n = 0;
-      if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->chainKernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds)) ||
-          CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->chainKernel, (int)ti->threads, ti->lds))) return 0;
+      if (CUSYNC_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds)) ||
+          CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
     }
     ti->residentPerCU = perCU;
@@ -304,7 +311,14 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
 
   const GemmParams p = gemmParams(a, ti, launched);
-  hipLaunchKernelGGL(ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0], dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
+  void (*kernel)(GemmParams) = ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0];
+  // Which of the two is faster is a matter of what the compiler made of each, and was measured per case on the GPT-3
+  // MLP: without the wait code the k loop is shorter (2048 rows, GEMM2, two tiles per workgroup: 305 -> 295 us; the
+  // few-row tiles: 87 -> 84 us for the 16-row pair), the start and the end of a launch longer (2048 rows, GEMM1, one
+  // tile per workgroup and GeLU: 300 -> 305 us; 1024 rows, GEMM2, one tile per workgroup: 160 -> 161).
+  if (a->a_mode != CUSYNC_A_SWIGLU && ti->kernelNoChunkWaits && !waitsPerChunk(s) && (tiles > launched || ti->bm <= 64))
+    kernel = ti->kernelNoChunkWaits;
+  hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }

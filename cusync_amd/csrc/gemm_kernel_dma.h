@@ -99,8 +99,13 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
   return r;
 }
 
-// One GEMM: all tiles of stage p.stage that this workgroup draws.
-template<class C, int AMODE>
+// One GEMM: all tiles of stage p.stage that this workgroup draws.  CHUNKS: the stage may be a consumer that waits
+// K chunk by K chunk (the tile policies).  The code of those waits is inlined once per pipeline step, and a kernel
+// that carries it without ever running it (stream order, RowSync) is slower for it: 3.5 us of 87 on the 16-row MLP
+// and 4.5 us of 593 on the 2048-row one, so such stages get a kernel compiled without.  (Not the kernel of several
+// GEMMs in one launch: compiled without, it spills more registers, 116 against 76 bytes per lane for the 256x192
+// tile, and the 512-row chain in one launch took 220 us instead of 213.)
+template<class C, int AMODE, bool CHUNKS>
 __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   constexpr bool conv = AMODE == kAConv;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -171,7 +176,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   const uint32_t numTiles = stage.numTiles();
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
-  const bool chunkSync = consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
+  const bool chunkSync = CHUNKS && consumer && stage.d.in.kind != CUSYNC_POLICY_ROWSYNC &&
                          stage.d.in.kind != CUSYNC_POLICY_CONSECUTIVESYNC;
 
   // Thread 0 keeps the ticket state: the start count is issued first and settled after the
@@ -255,6 +260,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       stage.waitWaveRows(lo, hi, tmq, policyCol, z);
     };
     auto waitChunk = [&](uint32_t k0) {
+      if constexpr (!CHUNKS) return;
       if (!chunkSync) return;
       if constexpr (conv) {
         const uint32_t ct = (k0 % p.cvC) / tnq;
@@ -489,9 +495,9 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   }
 }
 
-template<class C, int AMODE = kAPlain>
+template<class C, int AMODE = kAPlain, bool CHUNKS = true>
 __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
-  gemmDmaTiles<C, AMODE>(p);
+  gemmDmaTiles<C, AMODE, CHUNKS>(p);
 }
 
 // Dependent GEMMs of one tile shape in ONE launch: every workgroup works through the tiles of the first
@@ -504,7 +510,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
 template<class C>
 __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaChainKernel(GemmChainParams cp) {
   for (uint32_t g = 0; g < cp.count; g++) {
-    gemmDmaTiles<C, kAPlain>(cp.gemm[g]);
+    gemmDmaTiles<C, kAPlain, true>(cp.gemm[g]);
     __syncthreads();        // everyone has read the last ticket of this GEMM before the next one's is written
   }
 }

@@ -20,6 +20,9 @@ struct TileInfo {
   void (*kernel[2])(GemmParams);   // [plain A, SwiGLU A]
   int residentPerCU;     // filled lazily
   void (*chainKernel)(GemmChainParams);   // several dependent GEMMs in one launch; direct-to-LDS tiles only
+  // kernel[0] compiled without the per-chunk waits of the tile policies, for stages that wait for whole rows or
+  // for nothing (direct-to-LDS tiles only)
+  void (*kernelNoChunkWaits)(GemmParams);
 };
 
 void fillStagedTiles(TileInfo* tiles);     // register-staged tiles (the only ones with a SwiGLU A operand)
@@ -30,12 +33,13 @@ void fillDmaTilesFew(TileInfo* tiles);     // direct-to-LDS, 32 and 64 rows
 // Entry of a register-staged tile.
 #define CUSYNC_TILE(BM, BN, BK, WM, WN) \
   TileInfo{ BM, BN, BK, kThreads, (size_t)TileCfg<BM, BN, BK, WM, WN>::LDS_BYTES, \
-    { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1, nullptr }
+    { gemmKernel<TileCfg<BM, BN, BK, WM, WN>, false>, gemmKernel<TileCfg<BM, BN, BK, WM, WN>, true> }, -1, nullptr, nullptr }
 
 // Entry of a direct-to-LDS tile: no SwiGLU variant (that operand needs arithmetic on its way into LDS).
 #define CUSYNC_TILE_DMA(...) \
   TileInfo{ DmaCfg<__VA_ARGS__>::BM, DmaCfg<__VA_ARGS__>::BN, DmaCfg<__VA_ARGS__>::BK, DmaCfg<__VA_ARGS__>::THREADS, \
-    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1, gemmDmaChainKernel<DmaCfg<__VA_ARGS__>> }
+    (size_t)DmaCfg<__VA_ARGS__>::LDS_BYTES, { gemmDmaKernel<DmaCfg<__VA_ARGS__>>, nullptr }, -1, gemmDmaChainKernel<DmaCfg<__VA_ARGS__>>, \
+    gemmDmaKernel<DmaCfg<__VA_ARGS__>, kAPlain, false> }
 
 }  // namespace gemm
 }  // namespace cusync
