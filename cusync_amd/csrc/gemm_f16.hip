@@ -312,12 +312,8 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
 
   const GemmParams p = gemmParams(a, ti, launched);
   void (*kernel)(GemmParams) = ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0];
-  // Which of the two is faster is a matter of what the compiler made of each, and was measured per case on the GPT-3
-  // MLP: without the wait code the k loop is shorter (2048 rows, GEMM2, two tiles per workgroup: 305 -> 295 us; the
-  // few-row tiles: 87 -> 84 us for the 16-row pair), the start and the end of a launch longer (2048 rows, GEMM1, one
-  // tile per workgroup and GeLU: 300 -> 305 us; 1024 rows, GEMM2, one tile per workgroup: 160 -> 161).
-  if (a->a_mode != CUSYNC_A_SWIGLU && ti->kernelNoChunkWaits && !waitsPerChunk(s) && (tiles > launched || ti->bm <= 64))
-    kernel = ti->kernelNoChunkWaits;
+  // the few-row tiles come with a kernel compiled without the per-chunk waits, for stages that never make them
+  if (a->a_mode != CUSYNC_A_SWIGLU && ti->kernelNoChunkWaits && !waitsPerChunk(s)) kernel = ti->kernelNoChunkWaits;
   hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;

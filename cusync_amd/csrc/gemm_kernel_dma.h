@@ -100,12 +100,16 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
 }
 
 // One GEMM: all tiles of stage p.stage that this workgroup draws.  CHUNKS: the stage may be a consumer that waits
-// K chunk by K chunk (the tile policies).  The code of those waits is inlined once per pipeline step, and a kernel
-// that carries it without ever running it (stream order, RowSync) is slower for it: 3.5 us of 87 on the 16-row MLP
-// and 4.5 us of 593 on the 2048-row one, so such stages get a kernel compiled without.  (Not the kernel of several
-// GEMMs in one launch: compiled without, it spills more registers, 116 against 76 bytes per lane for the 256x192
-// tile, and the 512-row chain in one launch took 220 us instead of 213.)
-template<class C, int AMODE, bool CHUNKS>
+// K chunk by K chunk (the tile policies); without it that code is not compiled in (gemm_tiles.h says for which
+// tiles that is worth a kernel of its own).
+//
+// ROUNDS: a GEMM's chunk waits are made once per round of the pipeline (STAGES chunks ahead) instead of once per
+// chunk.  The wait's code is inlined where it is called; per chunk that is nine copies of it in the kernel, per
+// round two, and the TileSync consumer of the 2048-row MLP is 13 us (2 %) faster for it.  The kernel of several
+// GEMMs in one launch keeps the waits per chunk: compiled the other way it parks ten more registers per lane in
+// scratch around its epilogues (116 against 76 bytes for the 256x192 tile), and the 512-row chain, whose epilogues
+// are the k-slices' reduction, took 222 instead of 212 us.
+template<class C, int AMODE, bool CHUNKS, bool ROUNDS>
 __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   constexpr bool conv = AMODE == kAConv;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -377,7 +381,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       __builtin_amdgcn_s_barrier();      // chunk kt is in LDS for everyone; everyone is done with chunk kt-1
       asm volatile("" ::: "memory");
       const uint32_t ktLoad = kt + C::STAGES - 1;
-      if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
+      if constexpr (conv || !ROUNDS) { if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK); }
       __builtin_amdgcn_sched_barrier(0);
       compute(SP, Parity<(S + C::STAGES - 1) % C::STAGES>{}, ktLoad);
       __builtin_amdgcn_sched_barrier(0);
@@ -425,7 +429,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       __builtin_amdgcn_s_barrier();                // chunk kt+1 is in LDS for everyone; everyone is done with chunk kt-1
       asm volatile("" ::: "memory");
       const uint32_t ktLoad = kt + C::STAGES - 1;
-      if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK);
+      if constexpr (conv || !ROUNDS) { if (ktLoad < nk) waitChunk(kBegin + ktLoad * C::BK); }
       __builtin_amdgcn_sched_barrier(0);
       // k-step 1 while the first fragments of chunk kt+1 arrive and the loads of chunk ktLoad go out
       staticFor<R>([&](auto FP) {
@@ -448,11 +452,18 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     }
 
     // Prologue: chunks 0 .. STAGES-2 (chunks past the end of K load zeros).
-    waitChunk(kBegin);
+    // A GEMM's chunks go through the producer's column tiles in order, so the wait for a chunk covers the chunks
+    // before it: with ROUNDS, one wait for the prologue and one per round of the loop below, each for the last
+    // chunk whose loads it is in front of.  A convolution's chunks come back to the same channel tiles tap after
+    // tap and are always waited for one by one.
+    constexpr bool perChunk = conv || !ROUNDS;
+    auto waitThrough = [&](uint32_t kt) { waitChunk(kBegin + min(kt, nk - 1) * C::BK); };
+    if constexpr (perChunk) waitChunk(kBegin);
+    else waitThrough(C::STAGES - 2);
     issueAll(Parity<0>{}, 0);
-    if constexpr (C::STAGES > 2) { if (nk > 1) waitChunk(kBegin + C::BK); issueAll(Parity<1>{}, 1); }
-    if constexpr (C::STAGES > 3) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); issueAll(Parity<2>{}, 2); }
-    if constexpr (C::STAGES > 4) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); issueAll(Parity<3>{}, 3); }
+    if constexpr (C::STAGES > 2) { if constexpr (perChunk) { if (nk > 1) waitChunk(kBegin + C::BK); } issueAll(Parity<1>{}, 1); }
+    if constexpr (C::STAGES > 3) { if constexpr (perChunk) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); } issueAll(Parity<2>{}, 2); }
+    if constexpr (C::STAGES > 4) { if constexpr (perChunk) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); } issueAll(Parity<3>{}, 3); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 5, "prologue written for 2..5 stages");
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
@@ -463,6 +474,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       asm volatile("" ::: "memory");
       staticFor<C::TM + C::TN>([&](auto FP) { loadFragP(Parity<0>{}, FP, Parity<0>{}, 0); });
       for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
+        if constexpr (!perChunk) waitThrough(kt + 2 * C::STAGES - 2);      // the loads this round issues
         stepP(Parity<0>{}, kt);
         if (kt + 1 < nk) stepP(Parity<1 % C::STAGES>{}, kt + 1);
         if (C::STAGES > 2 && kt + 2 < nk) stepP(Parity<2 % C::STAGES>{}, kt + 2);
@@ -471,6 +483,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       }
     } else {
       for (uint32_t kt = 0; kt < nk; kt += C::STAGES) {
+        if constexpr (!perChunk) waitThrough(kt + 2 * C::STAGES - 2);      // the loads this round issues
         step(Parity<0>{}, kt);
         if (kt + 1 < nk) step(Parity<1 % C::STAGES>{}, kt + 1);
         if (C::STAGES > 2 && kt + 2 < nk) step(Parity<2 % C::STAGES>{}, kt + 2);
@@ -497,7 +510,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
 
 template<class C, int AMODE = kAPlain, bool CHUNKS = true>
 __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(GemmParams p) {
-  gemmDmaTiles<C, AMODE, CHUNKS>(p);
+  gemmDmaTiles<C, AMODE, CHUNKS, true>(p);
 }
 
 // Dependent GEMMs of one tile shape in ONE launch: every workgroup works through the tiles of the first
@@ -510,7 +523,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaKernel(G
 template<class C>
 __global__ __launch_bounds__(C::THREADS, C::WAVES_PER_SIMD) void gemmDmaChainKernel(GemmChainParams cp) {
   for (uint32_t g = 0; g < cp.count; g++) {
-    gemmDmaTiles<C, kAPlain, true>(cp.gemm[g]);
+    gemmDmaTiles<C, kAPlain, true, false>(cp.gemm[g]);
     __syncthreads();        // everyone has read the last ticket of this GEMM before the next one's is written
   }
 }
