@@ -209,7 +209,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     waitVmcnt<0>();
     const unsigned long long tl2 = p.timeline ? wall_clock64() : 0;
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
-    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
+    const bool completed = finishTile<C, false>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, 0};
     if (completed && stage.isProducer()) stage.post(done);
     else __syncthreads();

@@ -294,10 +294,12 @@ template<class C>
 __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
                                                 const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds);
 
-template<class C>
+// SPLIT = false leaves the k-slices' part out of the kernel (the convolutions never slice K, and code a kernel
+// carries without running it still costs it time).
+template<class C, bool SPLIT = true>
 __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[C::TM][C::TN],
                                            const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
-  if (p.splitK > 1) return finishTileSplit<C>(p, acc, t, wm, wn, lane, sLast, lds);
+  if constexpr (SPLIT) { if (p.splitK > 1) return finishTileSplit<C>(p, acc, t, wm, wn, lane, sLast, lds); }
   const TileStore<C> store(p, t, wm, wn, lane, lds);
 #pragma unroll
   for (int i = 0; i < C::TM; i++)
@@ -332,8 +334,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   constexpr uint32_t kPieces = C::TM * C::WM;                                   // 32-row pieces of a tile
   constexpr uint32_t kEpiBytes = (C::WM * 32 * (C::BN * 2 + 16) + 1023) / 1024 * 1024;
   constexpr uint32_t kPieceBytes = C::WN * C::TN * 4 * 1024;                    // 32 rows x BN columns of fp32
-  const uint32_t perSlice = p.coopReduce ? kPieces / p.splitK : 0;
-  const bool ownInLds = p.coopReduce && kEpiBytes + perSlice * kPieceBytes <= (uint32_t)C::LDS_BYTES;
+  const uint32_t perSlice = C::BM >= 128 && p.coopReduce ? kPieces / p.splitK : 0;
+  const bool ownInLds = C::BM >= 128 && p.coopReduce && kEpiBytes + perSlice * kPieceBytes <= (uint32_t)C::LDS_BYTES;
   auto ownedPiece = [&](int i) { return ((uint32_t)i * C::WM + (uint32_t)wm) / perSlice == t.z; };      // uniform per wavefront
   auto ownSlot = [&](int i, int j, int g) {
     const uint32_t o = (uint32_t)i * C::WM + (uint32_t)wm - t.z * perSlice;
@@ -358,7 +360,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   const uint32_t tileIndex = t.y * p.stage.d.grid.x + t.x;
   uint32_t* counter = p.arrivals + tileIndex;
 
-  if (p.coopReduce) {
+  // (the launcher shares the reduction only among tiles of 128 rows and more: the smaller ones do not carry the code)
+  if (C::BM >= 128 && p.coopReduce) {
     // ---- every slice adds up and stores its share ---------------------------------------------------------
     // The tile is cut into BM/32 pieces of 32 rows (piece u = i * WM + wm: MFMA row tile i of wave row wm); slice z
     // takes the pieces [z * U/S, (z + 1) * U/S).  A piece is summed over the slices in index order (this slice's

@@ -497,7 +497,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     waitVmcnt<0>();
     const unsigned long long tl2 = p.timeline ? wall_clock64() : 0;
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
-    const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
+    const bool completed = finishTile<C, !conv>(p, acc, t, wm, wn, lane, &sLast, smem);
 
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
