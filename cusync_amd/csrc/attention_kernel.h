@@ -199,10 +199,10 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     // blocks of the producer that the rest of this tile's key range meets, and spins only if its own rows are
     // still missing: a tile that starts after its producer is done polls twice in all.
     uint32_t seenRows[2] = {0, 0};
-    auto waitKV = [&](uint32_t j) {
+    auto waitKV = [&](uint32_t j, uint32_t jLast) {       // blocks j .. jLast
       if (!consumer) return;
       // only the rows behind the cache come from the producer; its tiles count rows from there
-      const uint32_t lo = max(j * kBKV, p.cached), hi = min(j * kBKV + (uint32_t)kBKV, total);
+      const uint32_t lo = max(j * kBKV, p.cached), hi = min(jLast * kBKV + (uint32_t)kBKV, total);
       if (lo >= hi) return;
       const uint32_t rowLo = lo - p.cached, rowHi = hi - p.cached;             // [rowLo, rowHi)
       const uint32_t rangeEnd = min(jEnd * kBKV, total) - p.cached;            // end of this tile's key range
@@ -226,12 +226,11 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
       }
     };
 
-    // The first blocks are requested before Q: they are what the tile waits for longest.
+    // The first blocks are requested before Q: they are what the tile waits for longest.  One wait for all of them
+    // (the wait's code is inlined where it is called).
+    waitKV(jBegin, min(jBegin + (uint32_t)kStages - 2, jEnd - 1));
 #pragma unroll
-    for (uint32_t a = 0; a < kStages - 1; a++) {
-      if (jBegin + a < jEnd) waitKV(jBegin + a);
-      issue(jBegin + a, a, jBegin + a < jEnd);
-    }
+    for (uint32_t a = 0; a < kStages - 1; a++) issue(jBegin + a, a, jBegin + a < jEnd);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     // Q fragments stay in registers for the whole tile: k-step s is head-dim 16s + 8hi .. + 7 of row myq.
     if (!(stage.d.in.kind == CUSYNC_POLICY_ROWSYNC && p.cached == 0 && seenRows[0] >= qEnd)) waitRows(q0, qEnd, head * kHD);
@@ -353,7 +352,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
         __builtin_amdgcn_s_barrier();       // block j is in LDS for everyone; everyone is done with block j-1
         asm volatile("" ::: "memory");
         const uint32_t ahead = j + kStages - 1;           // goes into the stage block j-1 has left
-        if (ahead < jEnd) waitKV(ahead);
+        if (ahead < jEnd) waitKV(ahead, ahead);
         issue(ahead, (st + kStages - 1) % kStages, ahead < jEnd);
         if (p.causal && j * kBKV > p.cached + qw + 31) continue;       // wholly in this wave's future (wave-uniform)
         computeBlock(MASKED, j, st);
