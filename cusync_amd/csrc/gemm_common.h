@@ -373,7 +373,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
       if (!dev::pollUntilAtLeast(counter, p.splitK)) dev::countGiveUp(p.stage.d.spinTimeouts);     // the siblings are resident: bounded all the same
     }
     __syncthreads();
-#pragma unroll
+    // not unrolled: the sums do not live in the accumulators, so one copy of the pass serves every i
+#pragma unroll 1
     for (int i = 0; i < C::TM; i++) {
       const bool owned = ownedPiece(i);
       const uint32_t firstPiece = t.z * perSlice, endPiece = firstPiece + perSlice;
@@ -447,7 +448,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   // Narrow wavefront tiles have few loads per slice: several slices are fetched together (G of them), still
   // added in index order
   constexpr int G = C::BM <= 64 ? 36 / (C::TN * 4) : C::TN * 4 >= 16 ? 1 : 16 / (C::TN * 4);
-#pragma unroll
+  // (a real loop over i: one copy of the loads and of the pass)
+#pragma unroll 1
   for (int i = 0; i < C::TM; i++) {
     floatx4 sum[C::TN][4];
     for (uint32_t z = 0; z < p.splitK; z += G) {
