@@ -106,9 +106,10 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
 // ROUNDS: a GEMM's chunk waits are made once per round of the pipeline (STAGES chunks ahead) instead of once per
 // chunk.  The wait's code is inlined where it is called; per chunk that is nine copies of it in the kernel, per
 // round two, and the TileSync consumer of the 2048-row MLP is 13 us (2 %) faster for it.  The kernel of several
-// GEMMs in one launch keeps the waits per chunk: compiled the other way it parks ten more registers per lane in
-// scratch around its epilogues (116 against 76 bytes for the 256x192 tile), and the 512-row chain, whose epilogues
-// are the k-slices' reduction, took 222 instead of 212 us.
+// GEMMs in one launch keeps the waits per chunk: compiled the other way the 512-row chain, where one launch is the
+// best mode, took 212 instead of 208 us (and 222 instead of 212 while the k-slices' reduction was still unrolled
+// and the kernel parked ten more registers per lane in scratch for it); it would gain at 2048 rows, 595 -> 588 us,
+// where the two launches are ahead anyway.
 template<class C, int AMODE, bool CHUNKS, bool ROUNDS>
 __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   constexpr bool conv = AMODE == kAConv;
