@@ -376,12 +376,22 @@ def main():
                 row[name + "_us"] = round(trimmed(t)[0], 2)
                 row[name + "_tiles"] = list(m.tiles())
                 m.destroy()
+            # both GEMMs in one launch (the handle gives GEMM2 the tile of GEMM1; the launch has no more workgroups
+            # than the GEMM with fewer tiles, which costs this chain more than it gains except around 64 rows)
+            m = api.Mlp(api.MODEL.LLAMA, b, lh, li, api.SYNC.ROW, lw1.data_ptr(), lw2.data_ptr(), one_launch=True)
+            m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
+            t = m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20)
+            if m.stage_state(1).spin_timeouts:
+                sys.exit("bench.py: LLaMA consumer waits timed out — results invalid")
+            row["rowsync_one_launch_us"] = round(trimmed(t)[0], 2)
+            row["rowsync_one_launch_tiles"] = list(m.tiles())
+            m.destroy()
             for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW)):      # W2's rows are 16 KiB
                 m = api.Mlp(api.MODEL.LLAMA, b, lh, li, sync, lw1.data_ptr(), lw2.data_ptr(), repack_weights=True)
                 m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
                 row[name + "_repacked_us"] = round(trimmed(m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20))[0], 2)
                 m.destroy()
-            best = min(row[k] for k in ("rowsync_us", "tilesync_us", "stridedsync_us"))
+            best = min(row[k] for k in ("rowsync_us", "tilesync_us", "stridedsync_us", "rowsync_one_launch_us"))
             row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)
             row["best_tflops"] = round(2.0 * b * lh * 3 * li / best / 1e6, 1)
             other["llama_mlp"].append(row)
