@@ -376,8 +376,8 @@ def main():
                 row[name + "_us"] = round(trimmed(t)[0], 2)
                 row[name + "_tiles"] = list(m.tiles())
                 m.destroy()
-            # both GEMMs in one launch (the handle gives GEMM2 the tile of GEMM1; the launch has no more workgroups
-            # than the GEMM with fewer tiles, which costs this chain more than it gains except around 64 rows)
+            # both GEMMs in one launch (the handle gives GEMM2 the tile of GEMM1, which from 512 rows on costs this
+            # chain more than the launch saves)
             m = api.Mlp(api.MODEL.LLAMA, b, lh, li, api.SYNC.ROW, lw1.data_ptr(), lw2.data_ptr(), one_launch=True)
             m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
             t = m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20)

@@ -336,7 +336,7 @@ cusync_error cusync_gemm_chain_run(const cusync_gemm_args* args, int count, void
   if (!ti || !ti->chainKernel) { setError("gemm chain: needs a direct-to-LDS tile"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   const int resident = residentWorkgroups(args[0].tile);
   if (resident <= 0) { setError("gemm: kernel does not fit on a CU"); return CUSYNC_ERROR_DEVICE; }
-  uint32_t launched = (uint32_t)resident;
+  uint32_t launched = (uint32_t)resident, mostTiles = 0;
   for (int i = 0; i < count; i++) {
     const cusync_gemm_args& a = args[i];
     if (a.tile != args[0].tile) { setError("gemm chain: all GEMMs must use the same tile"); return CUSYNC_ERROR_NOT_INITIALIZED; }
@@ -344,10 +344,12 @@ cusync_error cusync_gemm_chain_run(const cusync_gemm_args* args, int count, void
     const cusync_error e = cusync_gemm_can_implement(&a);
     if (e != CUSYNC_SUCCESS) return e;
     if (a.stage.in.kind != CUSYNC_POLICY_NOSYNC && i == 0) { setError("gemm chain: the first GEMM cannot wait on a stage outside the launch"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-    // never more workgroups than any of the GEMMs has tiles: a workgroup without a tile of GEMM i would run ahead
-    launched = std::min<uint32_t>(launched, a.stage.grid.x * a.stage.grid.y * a.stage.grid.z);
+    mostTiles = std::max<uint32_t>(mostTiles, a.stage.grid.x * a.stage.grid.y * a.stage.grid.z);
     if (a.max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a.max_workgroups);
   }
+  // As many workgroups as the GEMM with most tiles has (and the device holds at once).  A workgroup without a tile
+  // of GEMM i goes straight on to GEMM i+1 and waits there for tiles that running workgroups hold.
+  launched = std::min<uint32_t>(launched, mostTiles);
   GemmChainParams cp = {};
   cp.count = (uint32_t)count;
   for (int i = 0; i < count; i++) cp.gemm[i] = gemmParams(&args[i], ti, launched);
