@@ -193,6 +193,26 @@ def test_gpt3_mlp_in_one_launch(batch, sync):
     assert np.array_equal(y.view(np.uint16), y0.view(np.uint16))
 
 
+@pytest.mark.parametrize("batch", [1, 64, 512])
+@pytest.mark.parametrize("sync", [api.SYNC.ROW, api.SYNC.STRIDED])
+def test_llama_mlp_in_one_launch(batch, sync):
+    # The two GEMMs of the LLaMA shard have different numbers of tiles (5504 and 8192 columns): the launch has as many
+    # workgroups as the larger one, and a workgroup without a tile of GEMM1 goes straight on to GEMM2 and waits there.
+    # Results bit for bit those of the stream-ordered pair with the same tiles and k-slices, and the oracle's.
+    print("llama one launch", batch, sync, flush=True)
+    x, w1, w2, h, y, prod, cons, tiles, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, 2752, sync, runs=3, one_launch=True)
+    assert tiles[0] == tiles[1]
+    _, _, _, h0, y0, _, _, tiles0, _ = run_mlp(api.MODEL.LLAMA, batch, 8192, 2752, api.SYNC.STREAM, runs=1, tile1=tiles[0], tile2=tiles[1],
+                                               split_k1=tiles[2], split_k2=tiles[3])
+    assert tiles == tiles0
+    assert cons.spin_timeouts == 0 and prod.spin_timeouts == 0
+    assert prod.tile_counter == 0 and cons.tile_counter == 0
+    assert np.array_equal(prod.sems, expected_sems(prod, tiles, 3, True))
+    assert np.array_equal(h.view(np.uint16), h0.view(np.uint16))
+    assert np.array_equal(y.view(np.uint16), y0.view(np.uint16))
+    check_against_oracle(api.MODEL.LLAMA, x, w1, w2, h, y, inner=2752, fused=True)
+
+
 def test_mlp_in_one_launch_rejects():
     w1, w2, dw1, dw2 = weights(api.MODEL.GPT3, 12288, 6144)
     with pytest.raises(RuntimeError):       # two different tiles cannot share a launch
