@@ -282,6 +282,59 @@ def test_chained_direct_to_lds_gemms_with_few_workgroups(policy_kind, tile):
     assert ps.tile_counter == 0 and cs.tile_counter == 0 and ps.start_counter == 0
 
 
+@pytest.mark.parametrize("policy_kind", ["row", "tile"])
+@pytest.mark.parametrize("tile", [api.TILE.T128x192x32, api.TILE.D64x192x64])
+def test_three_gemms_in_one_launch(policy_kind, tile):
+    # cusync_gemm_chain_run: C = A*B, E = C*D, G = E*F in ONE launch, three stages paired as for separate launches
+    # (the middle one waits and posts).  The GEMMs have 6 to 36 tiles each: the launch has as many workgroups as the
+    # largest, and a workgroup without a tile of an earlier GEMM goes straight on to the next and waits there.
+    import torch
+    print("three GEMMs in one launch", policy_kind, tile, flush=True)
+    L = _lib.load()
+    M, K, N1, N2, N3 = 300, 520, 384, 1152, 192
+    a = uniform_f16((M, K), 50)
+    b = uniform_f16((K, N1), 51) * np.float16(0.05)
+    d = uniform_f16((N1, N2), 52) * np.float16(0.05)
+    f = uniform_f16((N2, N3), 53) * np.float16(0.05)
+    da, db, dd, df = to_dev(a), to_dev(b), to_dev(d), to_dev(f)
+    dc, de, dg = (empty_dev((M, n), fill=float("nan")) for n in (N1, N2, N3))
+    torch.cuda.synchronize()
+    tm, tn, _ = api.tile_shape(tile)
+    grids = [api.gemm_grid(tile, M, n, 1) for n in (N1, N2, N3)]
+
+    def policy(g):
+        return api.tile_sync(api.ORDER.TRANSPOSE_XY, tm, tn) if policy_kind == "tile" else api.row_sync(tm, g[0])
+
+    p1, p2 = policy(grids[0]), policy(grids[1])
+    st = [api.Stage(grids[0], (1, 1, 1), api.no_sync(), p1), api.Stage(grids[1], (1, 1, 1), p1, p2),
+          api.Stage(grids[2], (1, 1, 1), p2, api.no_sync())]
+    assert api.set_producer_consumer_pair(st[0], st[1]) == api.ERR.SUCCESS
+    assert api.set_producer_consumer_pair(st[1], st[2]) == api.ERR.SUCCESS
+    args = (_lib.GemmArgs * 3)(
+        api.gemm_args(st[0], M, N1, K, da.data_ptr(), K, db.data_ptr(), N1, dc.data_ptr(), N1, tile),
+        api.gemm_args(st[1], M, N2, N1, dc.data_ptr(), N1, dd.data_ptr(), N2, de.data_ptr(), N2, tile, epilogue=api.EPI.RELU),
+        api.gemm_args(st[2], M, N3, N2, de.data_ptr(), N2, df.data_ptr(), N3, dg.data_ptr(), N3, tile))
+    for it in range(3):
+        for t in (dc, de, dg):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        assert L.cusync_gemm_chain_run(args, 3, None) == api.ERR.SUCCESS, api.last_error()
+        assert L.cusync_rt_device_sync() == 0, api.last_error()
+        for s_ in st:
+            s_.incrementIter()
+        for k in range(3):                  # the descriptors are copied into the arguments: take the new iteration over
+            args[k].stage = st[k].desc
+    states = [s_.read_state() for s_ in st]
+    c, e, g = to_host(dc), to_host(de), to_host(dg)
+    for s_ in st:
+        s_.destroy()
+    assert all(s_.spin_timeouts == 0 for s_ in states)
+    assert all(s_.tile_counter == 0 for s_ in states)
+    assert_close(c, orc.gemm(a, b), "C")
+    assert_close(e, orc.gemm(c, d, orc.EPI_RELU), "E")
+    assert_close(g, orc.gemm(e, f), "G")
+
+
 def test_chained_gemms_with_few_workgroups():
     # both launches hold fewer workgroups than tiles: tickets keep producer rows ahead of consumers
     a, b, d, c, e, ps, cs, want_sems = chained(512, 1024, 512, api.TILE.T128x128x64, api.TILE.T128x128x64,
