@@ -471,7 +471,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
     cusync_dim3 done = {q0, head * kHD, 0};
-    if (completed && stage.isProducer()) stage.post(done);
+    if (completed && stage.isProducer()) stage.post(done, 1, true);
     else __syncthreads();
     if (tid == 0) recordTileAt(p.timeline, p.timelineCap, stage, p.launched, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }

@@ -316,7 +316,10 @@ struct DynStage {
 
   // Workgroup-wide post; contains a barrier, call from all threads.  `times`: how many posts of the policy this
   // one stands for (a workgroup that finished several logical tiles guarded by one semaphore adds them at once).
-  __device__ __forceinline__ void post(const cusync_dim3& tile, uint32_t times = 1) const {
+  // `writtenThrough`: every store of the tile went through to memory as it was made (sc1), so once the wavefronts
+  // have seen their stores acknowledged there is nothing left for a release to write back, and the semaphore is
+  // raised without one (a release at device scope starts a write-back of this XCD's L2 whatever it holds).
+  __device__ __forceinline__ void post(const cusync_dim3& tile, uint32_t times = 1, bool writtenThrough = false) const {
     if (!isProducer()) return;
     // The release is the first thread's and waits for its own wavefront's stores; a workgroup barrier does not wait
     // for stores to memory.  Every wavefront sees its own stores of the tile through before it reaches the barrier.
@@ -325,8 +328,13 @@ struct DynStage {
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
       const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid) * CUSYNC_SEM_STRIDE;
       const uint32_t v = dyn::postValue(d.out) * times;
-      if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::releaseStore(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
-      else dev::releaseAdd(&d.tileStatusWrite[idx], v);
+      if (writtenThrough) {
+        if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::storeRelaxed(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
+        else __hip_atomic_fetch_add((uint32_t*)&d.tileStatusWrite[idx], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::releaseStore(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
+        else dev::releaseAdd(&d.tileStatusWrite[idx], v);
+      }
     }
   }
 };
