@@ -388,13 +388,13 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
       const float scaledMax = rowMax * p.scaleLog2;      // the running maximum is kept unscaled
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, scaledMax), rPart, (int)offS, 0, 16);
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, rowSum), rPart, (int)(offS + kThreads * sizeof(float)), 0, 16);
-      // The release below is the first thread's: it waits for that wavefront's stores only, and a workgroup barrier
-      // does not wait for stores to memory either.  Every wavefront sees its own through first.
+      // The count below is the first thread's, and a workgroup barrier does not wait for stores to memory: every
+      // wavefront sees its own through first.
       waitVmcnt<0>();
       __syncthreads();
       uint32_t* counter = p.arrivals + head * stage.d.grid.y + t.y;
       if (tid == 0) {
-        const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // the shares were written through and are acknowledged
         const bool last = before == splits - 1;
         if (last) cusync::dev::storeRelaxed(counter, 0);
         sLast = last;

@@ -369,7 +369,8 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     // in whatever order of arrival the tile is put together.
     uint32_t* departures = p.arrivals + p.stage.d.grid.x * p.stage.d.grid.y + tileIndex;
     if (threadIdx.x == 0) {
-      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      // not a release: the partial sums were written through and every wavefront has seen its own acknowledged
+      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (!dev::pollUntilAtLeast(counter, p.splitK)) dev::countGiveUp(p.stage.d.spinTimeouts);     // the siblings are resident: bounded all the same
     }
     __syncthreads();
@@ -418,11 +419,10 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
-      // A producer's stores must be out before the count that lets the last slice post (they were written through:
-      // the release has nothing to write back).  No acquire: nobody reads another slice's output, and an acquire
-      // would empty this XCD's L2 under the workgroups that are still in their k loops.
-      const uint32_t before = p.stage.isProducer() ? __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT)
-                                                   : __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // A producer's stores must be out before the count that lets the last slice post: they were written through
+      // and are acknowledged (the wait above), so the count needs no release, which would only start a write-back of
+      // this XCD's L2.  No acquire either: nobody reads another slice's output.
+      const uint32_t before = __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = before == p.splitK - 1;
       if (last) { dev::storeRelaxed(counter, 0); dev::storeRelaxed(departures, 0); }
       *sLast = last;
@@ -432,8 +432,9 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   }
 
   if (threadIdx.x == 0) {
-    // release only: an acquire here would empty this XCD's L2 once per slice; the finishing slice acquires below
-    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    // neither release (the partial sums were written through and are acknowledged) nor acquire (the finishing slice
+    // reads them with device-coherent loads): either would work on this XCD's whole L2
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const bool last = before == p.splitK - 1;
     if (last) dev::storeRelaxed(counter, 0);
     *sLast = last;
