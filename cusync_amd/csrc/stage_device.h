@@ -121,8 +121,11 @@ struct DynStage {
     if (!isProducer() || (d.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL)) return;
     if (token == launched - 1) {
       dev::storeRelaxed(d.startCounter, 0);
-      dev::releaseStore(d.kernelExecuted, (uint32_t)d.iter);
-      dev::releaseStoreSystem(d.spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, (uint32_t)d.iter);     // mirror for a host that holds the consumer back itself
+      // The flag says that every producer workgroup is on the device and publishes no data (a consumer reads the
+      // producer's output behind the tiles' semaphores): relaxed stores.  As releases they wrote this XCD's L2 back,
+      // the second one as far as the host, on the critical path of the one workgroup that raises them.
+      dev::storeRelaxed(d.kernelExecuted, (uint32_t)d.iter);
+      __hip_atomic_store(d.spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, (uint32_t)d.iter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);     // mirror for a host that holds the consumer back itself
     }
   }
 
