@@ -32,6 +32,7 @@
 #include "stage_device.h"
 
 #include "gemm_tiles.h"
+#include "split_choice.h"
 
 namespace {
 
@@ -147,6 +148,7 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
   if (a->split_k < 1) { setError("gemm: split_k must be at least 1"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->split_k > 1) {
     if ((uint32_t)a->split_k > (a->K + ti->bk - 1) / ti->bk) { setError("gemm: more k-slices than K chunks"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (!everySliceHasAChunk(a->K, ti->bk, (uint32_t)a->split_k)) { setError("gemm: split_k leaves the last k-slice without a K chunk (each slice takes ceil(chunks / split_k) chunks)"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (!a->workspace || (uintptr_t)a->workspace % 16) { setError("gemm: split_k > 1 needs a 16-byte aligned workspace of cusync_gemm_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (partialBytes(a, ti) >= 0x80000000ull) { setError("gemm: the partial sums of these k-slices exceed 2 GiB, more than one buffer descriptor addresses"); return CUSYNC_ERROR_NOT_INITIALIZED; }

@@ -213,9 +213,15 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   if (c.batch <= 32) {
     a = CUSYNC_TILE_D32x128x64;
     if (!swiglu) b = CUSYNC_TILE_D32x128x64;
-  } else if (c.batch <= 256) {
+  } else if (c.batch <= 192) {
     if (n1 % 192 == 0) a = CUSYNC_TILE_D64x192x64;
     if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_D64x192x64;
+  } else if (c.batch <= 256) {
+    // two row tiles of 128: 128x192 at two workgroups per CU, in four and two k-slices (256 rows: 78.5 and 72.4 us
+    // against 82.7 and 73.5 for 64x192 in two slices and one; the pair 151 against 156 us stream-ordered, 140
+    // against 142 under TileSync), now that a slice's arrival no longer writes its XCD's L2 back
+    if (n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
+    if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
   }
   // StridedSync needs the gate|up split on a column-tile boundary of GEMM1: 128- or 256-wide tiles where the
   // 192-wide ones do not divide `inner`, 64-wide ones where nothing else does (2752 = 43 * 64)

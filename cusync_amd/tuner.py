@@ -48,13 +48,13 @@ def resident_share(tile, M, N, split):
 def candidates(batch, n1, n2):
     """(tile, split) choices worth timing for a GEMM with `batch` rows."""
     if batch <= 32:
-        tiles, splits = [api.TILE.D32x128x64, api.TILE.T32x128x64], [2, 4, 8]
+        tiles, splits = [api.TILE.D32x128x64, api.TILE.T32x128x64], [2, 4, 8, 16]
     elif batch <= 64:
-        tiles, splits = [api.TILE.D64x192x64, api.TILE.D32x128x64, api.TILE.T64x128x64], [2, 4, 8]
+        tiles, splits = [api.TILE.D64x192x64, api.TILE.D32x128x64, api.TILE.T64x128x64], [2, 4, 8, 16]
     elif batch <= 128:
         tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x128x64, api.TILE.T128x128x32], [1, 2, 4, 8]
     elif batch <= 512:
-        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4]
+        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4, 8]
     else:
         tiles, splits = [api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
     if n1 % 192 or n2 % 192:        # the LLaMA shard (5504 and 8192 columns): also the 256-wide tiles
@@ -94,6 +94,8 @@ class Bench:
             out = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=timed, split=(sync == api.SYNC.STREAM))
             if m.stage_state(1).spin_timeouts:
                 return None
+        except api.CuSyncError:      # a candidate the library refuses (k-slices that do not fit this K)
+            return None
         finally:
             m.destroy()
         return out
@@ -115,12 +117,16 @@ def tune_batch(bench, batch, log):
     bench.run(batch, api.SYNC.STREAM, warm=30, timed=1, tile1=c1[0][0], tile2=c2[0][0], split_k1=c1[0][1], split_k2=c2[0][1])   # clocks up
     for (t, s) in c1:
         r = bench.run(batch, api.SYNC.STREAM, tile1=t, tile2=c2[0][0], split_k1=s, split_k2=c2[0][1])
+        if r is None:
+            continue
         us = trimmed(r[1])
         log("B=%d GEMM1 tile %d split %d: %.1f us" % (batch, t, s, us))
         if best1 is None or us < best1[0]:
             best1 = (us, t, s)
     for (t, s) in c2:
         r = bench.run(batch, api.SYNC.STREAM, tile1=best1[1], tile2=t, split_k1=best1[2], split_k2=s)
+        if r is None:
+            continue
         us = trimmed(r[2])
         log("B=%d GEMM2 tile %d split %d: %.1f us" % (batch, t, s, us))
         if best2 is None or us < best2[0]:

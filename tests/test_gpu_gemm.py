@@ -177,6 +177,11 @@ def test_gemm_can_implement_rejects():
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "multiples of 8" in api.last_error()
     bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=2)   # more slices than K chunks
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "k-slices" in api.last_error()
+    # 2816 / 64 = 44 chunks in 16 slices of three: the sixteenth would begin past the end of K
+    st16 = plain_stage(api.TILE.T64x128x64, 64, 128, split_k=16)
+    bad = api.gemm_args(st16, 64, 128, 2816, 16, 2816, 16, 128, 16, 128, api.TILE.T64x128x64, split_k=16)
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "without a K chunk" in api.last_error()
+    st16.destroy()
     bad = api.gemm_args(st, 64, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64, split_k=0)
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED
     bad = api.gemm_args(st, 300, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # grid mismatch
