@@ -176,7 +176,7 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // slices; level at 512 rows).
     int a, b;
     if (c.batch <= 32) a = b = CUSYNC_TILE_D32x128x64;
-    else if (c.batch <= 64) a = b = CUSYNC_TILE_D64x128x64;
+    else if (c.batch <= 64) { a = CUSYNC_TILE_D64x128x64; b = CUSYNC_TILE_D32x128x64; }     // GEMM2 at 64 rows: 17 us in two slices against 20 on 64x128
     else if (c.batch <= 128) { a = CUSYNC_TILE_D64x192x64; b = CUSYNC_TILE_D64x128x64; }
     else if (c.batch <= 512) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_D64x128x64; }
     else if (c.batch <= 1024) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_128x256x32; }

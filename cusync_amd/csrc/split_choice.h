@@ -8,11 +8,12 @@ namespace cusync {
 namespace gemm {
 
 // k-slices for a GEMM of `tiles` output tiles: double while the launch stays
-// within one and a half workgroups per CU and every slice keeps at least eight
+// within one workgroup per CU (256 of them) and every slice keeps at least eight
 // K chunks.  Small batches are bound by streaming the weights, and without
-// slices a 32-row problem occupies 48 workgroups on 256 CUs; beyond about 384
-// workgroups the cost of adding the slices' partial sums outweighs the gain
-// (measured: M=16, N=6144, K=12288 takes 121 / 49 / 52 / 72 us with 1 / 4 / 8 / 16 slices).
+// slices a 32-row problem occupies 48 workgroups on 256 CUs; a launch of more
+// than one round of workgroups pays more for adding the slices' partial sums than
+// the extra loads in flight gain (M=16, N=6144, K=12288 on 32x128 tiles, 48 of them: 51 / 36 / 41 / 46 us
+// with 2 / 4 / 8 / 16 slices; M=64, N=5504, K=8192 on 64x128 tiles, 43 of them: 34 / 29 / 34 / 41 us).
 // Every slice takes ceil(chunks / slices) chunks of K, so a count that does not divide the chunks can leave the
 // last slices without any (44 chunks in 16 slices: three each, and the sixteenth would begin past the end).
 inline bool everySliceHasAChunk(uint32_t K, uint32_t bk, uint32_t slices) {
@@ -22,7 +23,7 @@ inline bool everySliceHasAChunk(uint32_t K, uint32_t bk, uint32_t slices) {
 
 inline int pickSplit(int requested, uint32_t tiles, uint32_t K, uint32_t bk, int resident) {
   if (requested > 0) return requested;
-  const uint32_t target = (uint32_t)std::min(resident, 384);
+  const uint32_t target = (uint32_t)std::min(resident, 256);
   int s = 1;
   while (tiles * (uint32_t)s * 2 <= target && K / ((uint32_t)s * 2) >= 8 * bk && everySliceHasAChunk(K, bk, (uint32_t)s * 2)) s *= 2;
   return s;
