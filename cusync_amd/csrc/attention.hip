@@ -262,6 +262,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
       sync1.tileM = tm1; sync1.tileN = 1; sync1.waitValue = g1.x; sync1.postValue = 1;
       sync2 = sync1;
       sync2.tileM = kBQ; sync2.waitValue = g2.x;
+      opts = CUSYNC_OPT_REORDER_TILE_LOADS;      // defined for every policy, attention.cu:13
       break;
     case CUSYNC_SYNC_TILE:      // TileSync on both edges, attention.cu:91-97
       sync1.kind = CUSYNC_POLICY_TILESYNC; sync1.order = CUSYNC_ORDER_TRANSPOSE_XY;
@@ -277,6 +278,7 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
       sync1.waitValue = L->E / tn1; sync1.postValue = 1;
       sync2.kind = CUSYNC_POLICY_ROWSYNC; sync2.order = CUSYNC_ORDER_TRANSPOSE_XY;
       sync2.tileM = kBQ; sync2.tileN = 1; sync2.waitValue = g2.x; sync2.postValue = 1;
+      opts = CUSYNC_OPT_REORDER_TILE_LOADS;
       break;
     default:
       setError("attn layer: unknown sync mode");

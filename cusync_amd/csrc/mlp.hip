@@ -363,6 +363,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
     case CUSYNC_SYNC_ROW:        // RowSync(gridDim1.n()), src/ml-bench/transformer/mlp.cu:1032-1034
       pol.kind = CUSYNC_POLICY_ROWSYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
       pol.tileM = tm1; pol.tileN = 1; pol.waitValue = g1.x; pol.postValue = 1;
+      opts = CUSYNC_OPT_REORDER_TILE_LOADS;      // defined for every policy, mlp.cu:15
       break;
     case CUSYNC_SYNC_TILE:       // TileSync<TransposeXY,kM,kN> + NoAtomicAdd + ReorderTileLoads, mlp.cu:9-16,111
       pol.kind = CUSYNC_POLICY_TILESYNC; pol.order = CUSYNC_ORDER_TRANSPOSE_XY;
