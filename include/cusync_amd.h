@@ -255,7 +255,9 @@ typedef struct cusync_gemm_args {
   int32_t epilogue;            /* CUSYNC_EPILOGUE_* */
   int32_t a_mode;              /* CUSYNC_A_* */
   int32_t tile;                /* CUSYNC_TILE_* */
-  int32_t split_k;             /* k-slices (grid z); > 1 adds the slices' fp32 partial sums through `workspace` */
+  int32_t split_k;             /* k-slices (grid z); > 1 adds the slices' fp32 partial sums through `workspace`.  Every slice takes
+                                  ceil(chunks / split_k) K chunks of the tile's depth, and a count that leaves the last slice without
+                                  a chunk is refused by cusync_gemm_can_implement (44 chunks in 16 slices) */
   void *workspace;             /* split_k > 1: cusync_gemm_workspace_size bytes, zeroed once by the caller */
   int32_t max_workgroups;      /* 0 = as many as stay resident; else cap on launched workgroups */
   int32_t shared_reduction;    /* split_k > 1.  0: the k-slice of a tile that finishes last adds up all slices and stores
