@@ -194,10 +194,9 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   // Measured on the GPT-3 shard.  Where the width is a multiple of 192 (6144 and 12288 columns are 32 and
   // 64 tiles: whole rounds on 256 CUs) the 192-wide direct-to-LDS tiles win from 256 rows on.  GEMM1: 256x192
   // with a CU to itself (8 % faster than 128x192 at two workgroups per CU at 1024 and 2048 rows; below that the
-  // k-slices fill the device).  GEMM2: the same from 385 rows on (at 512 rows in two k-slices whose workgroups
-  // each add up and store half a tile: 106 us against 117 us for 128x192 without slices); from 257 to 384 rows,
-  // where it has at most one 128-row tile per CU, 128x192 with four stages in the pipelined order (384 rows:
-  // 258 -> 225 us for the pair against 128x192 at two workgroups per CU for both).
+  // k-slices fill the device).  GEMM2: the same (from 257 to 512 rows in two k-slices whose workgroups each add up
+  // and store half a tile: at 512 rows 106 us against 117 us for 128x192 without slices, at 384 rows 96 against
+  // 110 us for 128x192 alone on its CU, which led there while a k-slice's arrival still wrote an L2 back).
   // Other widths (the LLaMA shard: 5504 and 8192 columns; the kernels mask the ragged last column tile): 128x192
   // alone on its CU up to 1024 rows, above that 256x192 for GEMM1 and 256x256 for GEMM2 (at 2048 rows 232 and 256
   // tiles: one round).  Measured against 128x128 / 128x256 at two workgroups per CU: 172 -> 147 us at 512 rows,
@@ -206,20 +205,25 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   int a = !big ? small : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
   int b = !big ? small : swiglu ? CUSYNC_TILE_256x128x64 : c.batch <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x256x32;
   if (big && n1 % 192 == 0) a = CUSYNC_TILE_256x192x32;
-  if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 384 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32_ALONE;
+  // (1025 to 1536 rows are five or six row tiles of 256, 320 or 384 tiles of GEMM2 for 256 CUs: there 128x192 at
+  // two workgroups per CU fills the second round better: 1152 rows 230 -> 212 us, 1280: 233 -> 217, 1536: 246 -> 236;
+  // from 1664 rows on 256x192 leads again, 258 against 285 us)
+  if (big && n2 % 192 == 0 && !swiglu) b = c.batch > 1024 && c.batch <= 1536 ? CUSYNC_TILE_128x192x32 : CUSYNC_TILE_256x192x32;
   // Up to 256 rows the GEMMs are bound by streaming the weights: direct-to-LDS tiles with 60-96 KB of loads
   // in flight per workgroup (measured: 104 -> 85 us at 1-32 rows, 127 -> 101 us at 64, 187 -> 158 us at 256).
   // 64x192 makes 32 or 64 column tiles, which 8 or 4 k-slices turn into one workgroup per CU.
   if (c.batch <= 32) {
     a = CUSYNC_TILE_D32x128x64;
     if (!swiglu) b = CUSYNC_TILE_D32x128x64;
-  } else if (c.batch <= 192) {
+  } else if (c.batch <= 128) {
     if (n1 % 192 == 0) a = CUSYNC_TILE_D64x192x64;
     if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_D64x192x64;
   } else if (c.batch <= 256) {
     // two row tiles of 128: 128x192 at two workgroups per CU, in four and two k-slices (256 rows: 78.5 and 72.4 us
     // against 82.7 and 73.5 for 64x192 in two slices and one; the pair 151 against 156 us stream-ordered, 140
-    // against 142 under TileSync), now that a slice's arrival no longer writes its XCD's L2 back
+    // against 142 under TileSync; 160 rows, where 64x192 makes three row tiles: 130 against 148 us), now that a
+    // slice's arrival no longer writes its XCD's L2 back.  At 128 rows 64x192 in four and two slices still leads
+    // (106 against 120 us for one row tile of 128 in eight and four).
     if (n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
     if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
   }

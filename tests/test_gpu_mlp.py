@@ -84,7 +84,9 @@ def expected_sems(prod, tiles, iters, fused=False):
     return orc.expected_sems_gemm(p, prod.grid, tm, tn // 2 if fused else tn, iters, d.opts)
 
 
-@pytest.mark.parametrize("batch", [1, 16, 64, 256, 512])
+# 160, 320 and 1280 rows are not whole tiles: 160 is two tiles of 128 rows with the second one ragged, 320 two of 256,
+# and at 1280 the producer's tiles have 256 rows and the consumer's 128
+@pytest.mark.parametrize("batch", [1, 16, 64, 160, 256, 320, 512, 1280])
 def test_gpt3_mlp_all_sync_modes(batch):
     print("gpt3 batch", batch, flush=True)
     outs = {}
