@@ -212,20 +212,24 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   L->cfg = *cfg;
   L->wqkv = wqkv; L->wo = wo;
   L->E = cfg->heads * kHD;
-  // Per-row-count choice, from the tuner's measurements (cusync_amd/tile_sizes_db.py, gpt3_attention_mi355x).
-  // Widths that are multiples of 192 (4608 = 24 x 192, 12288 = 64 x 192) take the 192-wide direct-to-LDS tiles:
-  // 64x192x64 up to 256 rows, where streaming the weights bounds the projections; 128x192 with a CU to itself
-  // while the GEMM has about one tile per CU (QKV projection, 24 column tiles: up to 1024 rows; output projection,
-  // 64: up to 512); 256x192 above (2048 rows: 446 -> 430 us for the chain against 128x192 at two per CU).
+  // Per-row-count choice, from the tuner's measurements (cusync_amd/tile_sizes_db.py, gpt3_attention_mi355x) and
+  // sweeps between its row counts.  Widths that are multiples of 192 (4608 = 24 x 192, 12288 = 64 x 192) take the
+  // 192-wide direct-to-LDS tiles.  QKV projection (24 column tiles): 64x192x64 in k-slices while the projection
+  // streams the weights, up to 320 rows (five row tiles in two slices are 240 workgroups: 56 us against 69 for
+  // 128x192); 128x192 with a CU to itself up to 1024 rows, except from 641 to 768 rows, which are three whole row
+  // tiles of 256x192 in two slices (105 against 124 us); 256x192 above.  Output projection (64 column tiles):
+  // 64x192x64 up to 256 rows, 128x192 alone up to 512, 256x192 up to 1024, and above that 128x192 at two workgroups
+  // per CU, whose tiles fill the last round better (1280 rows: 79 -> 69 us, 1536: 80 -> 72, level at 2048).
   // Other widths: tiles that follow the row count up to 128 rows, 128x128 up to 1024 rows, 128x256 above.
   const int small = cfg->seq <= 32 ? CUSYNC_TILE_D32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
-  auto wide = [&](uint32_t aloneUpTo) {
-    return cfg->seq <= 32 ? small : cfg->seq <= 256 ? CUSYNC_TILE_D64x192x64
-           : cfg->seq <= aloneUpTo ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
-  };
-  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide(1024) : dflt;
-  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide(512) : dflt;
+  const uint32_t S = cfg->seq;
+  const int wide1 = S <= 32 ? small : S <= 320 ? CUSYNC_TILE_D64x192x64 : S > 640 && S <= 768 ? CUSYNC_TILE_256x192x32
+                    : S <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
+  const int wide3 = S <= 32 ? small : S <= 256 ? CUSYNC_TILE_D64x192x64 : S <= 512 ? CUSYNC_TILE_128x192x32_ALONE
+                    : S <= 1024 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;
+  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide1 : dflt;
+  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide3 : dflt;
   L->ws1 = L->ws3 = L->ws2 = nullptr;
   // Key ranges of 8 blocks (512 rows) or more are cut in two: under a causal mask the last row tiles walk the
   // longest ranges and the launch is as long as its longest workgroup.  Measured alone at 12 heads: 512 rows

@@ -174,7 +174,8 @@ def test_attention_layer_small(S, tile):
     check_layer(S, 512, 2, sampled=False, tile1=tile, tile3=tile)
 
 
-@pytest.mark.parametrize("S", [256, 512, 1024, 2048])
+# 320, 768 and 1280 rows fall between the tuned lengths: ragged row tiles, and tile shapes that differ from one stage to the next
+@pytest.mark.parametrize("S", [256, 320, 512, 768, 1024, 1280, 2048])
 def test_attention_layer_gpt3_shard(S):
     print("attn layer gpt3", S, flush=True)
     check_layer(S, 12288, 12, sampled=True)
