@@ -1,0 +1,62 @@
+"""The k-slice rule of the GEMM launcher and of the chains (cusync_amd/csrc/split_choice.h), host code only.
+
+The kernel gives slice z the K chunks [z * per, (z + 1) * per) with per = ceil(chunks / slices): a slice count is
+usable only if the last slice still begins inside K.  The closed form the library uses is checked against that
+definition by brute force, and the automatic choice against the cases the design was measured on."""
+import os
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+SRC = r"""
+#include <cstdio>
+#include "split_choice.h"
+using namespace cusync::gemm;
+int main() {
+  // every (chunks, slices) pair of a small range: 1 if the library accepts it
+  for (uint32_t chunks = 1; chunks <= 96; chunks++)
+    for (uint32_t slices = 1; slices <= 40; slices++)
+      std::printf("E %u %u %d\n", chunks, slices, everySliceHasAChunk(chunks * 64 - 8, 64, slices) ? 1 : 0);
+  const uint32_t cases[][4] = {
+    {48, 12288, 64, 256}, {96, 6144, 64, 256}, {32, 12288, 64, 256}, {64, 6144, 64, 256},     // GPT-3 shard, few rows
+    {43, 8192, 64, 512}, {64, 2752, 64, 256}, {64, 2816, 64, 256},                               // LLaMA shard
+    {64, 12288, 32, 256}, {128, 6144, 32, 256}, {256, 12288, 32, 256}, {512, 6144, 32, 256},    // 512 and 2048 rows on 256x192
+    {1, 8256, 64, 256}, {1, 64, 64, 256}};
+  for (auto& c : cases) std::printf("P %u %u %u %u %d\n", c[0], c[1], c[2], c[3], pickSplit(0, c[0], c[1], c[2], (int)c[3]));
+  std::printf("R %d\n", pickSplit(7, 48, 12288, 64, 256));
+  return 0;
+}
+"""
+
+
+def test_split_choice(tmp_path):
+    src = tmp_path / "split_choice_test.cpp"
+    src.write_text(SRC)
+    exe = tmp_path / "split_choice_test"
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "cusync_amd", "csrc"), str(src), "-o", str(exe)])
+    out = subprocess.check_output([str(exe)], text=True).split("\n")
+    picks = {}
+    for line in out:
+        f = line.split()
+        if not f:
+            continue
+        if f[0] == "E":
+            chunks, slices, got = int(f[1]), int(f[2]), int(f[3])
+            per = -(-chunks // slices)
+            # the definition: every slice z < slices begins before the end of K (K = chunks * 64 - 8: a ragged last chunk)
+            want = all(z * per * 64 < chunks * 64 - 8 for z in range(slices))
+            assert got == int(want), (chunks, slices)
+        elif f[0] == "P":
+            picks[tuple(int(v) for v in f[1:5])] = int(f[5])
+        elif f[0] == "R":
+            assert int(f[1]) == 7                     # a requested count is passed through (and validated by the GEMM)
+    # one workgroup per CU at most, and at least eight chunks per slice
+    assert picks[(48, 12288, 64, 256)] == 4 and picks[(96, 6144, 64, 256)] == 2
+    assert picks[(32, 12288, 64, 256)] == 8 and picks[(64, 6144, 64, 256)] == 4
+    assert picks[(43, 8192, 64, 512)] == 4            # 344 workgroups would be a second round
+    assert picks[(64, 2752, 64, 256)] == 4 and picks[(64, 2816, 64, 256)] == 4
+    assert picks[(64, 12288, 32, 256)] == 4 and picks[(128, 6144, 32, 256)] == 2
+    assert picks[(256, 12288, 32, 256)] == 1 and picks[(512, 6144, 32, 256)] == 1
+    # 129 chunks: sixteen slices of nine would leave the last one empty, and the doubling stops at eight
+    assert picks[(1, 8256, 64, 256)] == 8
+    assert picks[(1, 64, 64, 256)] == 1
