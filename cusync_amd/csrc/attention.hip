@@ -26,6 +26,7 @@ using namespace cusync::attn;
 std::mutex g_attnMutex;
 int g_attnResidentPerCU[2] = {-1, -1};      // [0] two stages, [1] four
 int g_attnNumCUs = 0;
+int g_attnLdsPerCU = 0;
 
 typedef void (*AttnKernel)(AttnParams);
 AttnKernel attnKernel(bool deep) { return deep ? attentionKernel<4> : attentionKernel<2>; }
@@ -49,8 +50,9 @@ int residentAttention(bool deep) {
     hipDeviceProp_t prop;
     if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
     g_attnNumCUs = prop.multiProcessorCount;
+    g_attnLdsPerCU = (int)prop.maxSharedMemoryPerMultiProcessor;
     if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attnKernel(deep)),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, attnLds(deep)))) return 0;
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, std::max(attnLds(deep), g_attnLdsPerCU / 2)))) return 0;
     int n = 0;
     if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attnKernel(deep), kThreads, attnLds(deep)))) return 0;
     perCU = n;
@@ -197,7 +199,15 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
     p.arrivals = (uint32_t*)(p.partStat + tiles * s.grid.z * 2 * kThreads);
     p.partBytes = (uint32_t)((char*)p.arrivals - (char*)p.partO);
   }
-  hipLaunchKernelGGL(attnKernel(deep), dim3(launched), dim3(kThreads), attnLds(deep), (hipStream_t)stream, p);
+  // A consumer launch of no more workgroups than CUs asks for half a CU's LDS, so that the dispatcher spreads it one
+  // to a CU instead of packing pairs onto the CUs its producer left free (see cusync_gemm_run): 1280 rows, 240
+  // workgroups, 264 -> 244 us for the chain under every policy.  Not a launch of up to half as many workgroups as
+  // CUs: packed, those are all resident beside the producer early and leave whole CUs to the output projection's
+  // workgroups (512 rows, 96 workgroups: 124 us packed, 129 spread).
+  int lds = attnLds(deep);
+  if (s.in.kind != CUSYNC_POLICY_NOSYNC && launched <= (uint32_t)g_attnNumCUs && launched > (uint32_t)g_attnNumCUs / 2 && resident > g_attnNumCUs)
+    lds = std::max(lds, g_attnLdsPerCU / 2);
+  hipLaunchKernelGGL(attnKernel(deep), dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }

@@ -47,6 +47,7 @@ std::once_flag g_tilesOnce;
 
 std::mutex g_mutex;
 int g_numCUs = 0;
+uint32_t g_ldsPerCU = 0;
 
 // The kernels are instantiated in several translation units (they take minutes to compile); each fills in
 // the entries of the tiles it holds.
@@ -77,12 +78,13 @@ int residentWorkgroups(int tile) {
       hipDeviceProp_t prop;
       if (CUSYNC_HIP(hipGetDevice(&dev)) || CUSYNC_HIP(hipGetDeviceProperties(&prop, dev))) return 0;
       g_numCUs = prop.multiProcessorCount;
+      g_ldsPerCU = (uint32_t)prop.maxSharedMemoryPerMultiProcessor;
     }
     int perCU = 1 << 30;
     for (int v = 0; v < 2; v++) {
       if (!ti->kernel[v]) continue;
       if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->kernel[v]),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds))) return 0;
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)std::max<size_t>(ti->lds, g_ldsPerCU / 2)))) return 0;
       int n = 0;
       if (CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ti->kernel[v], (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
@@ -91,7 +93,7 @@ int residentWorkgroups(int tile) {
     for (const void* k : others) {
       if (!k) continue;
       int n = 0;
-      if (CUSYNC_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ti->lds)) ||
+      if (CUSYNC_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)std::max<size_t>(ti->lds, g_ldsPerCU / 2))) ||
           CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, (int)ti->threads, ti->lds))) return 0;
       perCU = std::min(perCU, n);
     }
@@ -316,7 +318,18 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   void (*kernel)(GemmParams) = ti->kernel[a->a_mode == CUSYNC_A_SWIGLU ? 1 : 0];
   // the few-row tiles come with a kernel compiled without the per-chunk waits, for stages that never make them
   if (a->a_mode != CUSYNC_A_SWIGLU && ti->kernelNoChunkWaits && !waitsPerChunk(s)) kernel = ti->kernelNoChunkWaits;
-  hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), ti->lds, (hipStream_t)stream, p);
+  // A consumer's workgroups are dispatched while the producer's hold their CUs, and where two of them fit a CU the
+  // dispatcher packs them in pairs onto the CUs the producer left free: when the producer is done, half the device
+  // runs the consumer two to a CU and the other half nothing (LLaMA MLP, 640 to 1024 rows under RowSync: 144-175 us
+  // against 140-164 stream-ordered).  A launch of no more workgroups than CUs therefore asks for half a CU's LDS,
+  // which with the kernel's few static bytes lets one workgroup onto a CU and leaves the other half to the producer
+  // (the same chains: 132-159 us).  A launch of at most half as many workgroups as CUs is left to be packed: it is
+  // resident beside the producer at once and leaves whole CUs to the stage after it (measured on the attention
+  // kernel, see cusync_attention_run).
+  size_t lds = ti->lds;
+  if (s.in.kind != CUSYNC_POLICY_NOSYNC && launched <= (uint32_t)g_numCUs && launched > (uint32_t)g_numCUs / 2 && ti->residentPerCU > 1)
+    lds = std::max<size_t>(lds, g_ldsPerCU / 2);
+  hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   return CUSYNC_SUCCESS;
 }
