@@ -32,14 +32,21 @@ typedef void (*AttnKernel)(AttnParams);
 AttnKernel attnKernel(bool deep) { return deep ? attentionKernel<4> : attentionKernel<2>; }
 int attnLds(bool deep) { return cusync::attn::ldsBytes(deep ? 4 : 2); }
 
+int residentAttention(bool deep);
+
 // Four stages where the kernel has the device to itself anyway: as a stage of its own between stream-ordered
 // launches, and from 2048 key rows on, where the projections around it run 256-row tiles that take a whole CU's
 // LDS (measured at 2048 rows x 12 heads: 59 -> 51 us alone; chain under ConsecutiveSync 422 -> 410 us).  Two stages
 // where its workgroups are to sit beside those of its producer and consumer (chains up to 1024 rows: with four
-// stages every gain of the overlapped chains over the stream-ordered ones was gone).
+// stages every gain of the overlapped chains over the stream-ordered ones was gone) -- as long as the launch has
+// no more workgroups than CUs: beyond that the two-stage workgroups end up two to a CU on the CUs that came free
+// first, and four stages with a CU each are faster again (1408 rows, 264 workgroups: 291 -> 281 us under
+// ConsecutiveSync, 1792 rows: 357 -> 337; 1280 rows, 240 workgroups, stay at two stages: 237 against 246 us).
 bool deepPipeline(const cusync_attention_args* a) {
   const bool alone = a->stage.in.kind == CUSYNC_POLICY_NOSYNC && a->stage.out.kind == CUSYNC_POLICY_NOSYNC;
-  return alone || a->seq + a->cached_rows >= 2048;
+  if (alone || a->seq + a->cached_rows >= 2048) return true;
+  if (g_attnNumCUs == 0) residentAttention(false);      // reads the device's CU count
+  return g_attnNumCUs > 0 && a->stage.grid.x * a->stage.grid.y * a->stage.grid.z > (uint32_t)g_attnNumCUs;
 }
 
 int residentAttention(bool deep) {

@@ -175,7 +175,7 @@ def test_attention_layer_small(S, tile):
 
 
 # 320, 768 and 1280 rows fall between the tuned lengths: ragged row tiles, and tile shapes that differ from one stage to the next
-@pytest.mark.parametrize("S", [256, 320, 512, 768, 1024, 1280, 2048])
+@pytest.mark.parametrize("S", [256, 320, 512, 768, 1024, 1280, 1536, 2048])
 def test_attention_layer_gpt3_shard(S):
     print("attn layer gpt3", S, flush=True)
     check_layer(S, 12288, 12, sampled=True)
