@@ -212,7 +212,8 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   // CUs: packed, those are all resident beside the producer early and leave whole CUs to the output projection's
   // workgroups (512 rows, 96 workgroups: 124 us packed, 129 spread).
   int lds = attnLds(deep);
-  if (s.in.kind != CUSYNC_POLICY_NOSYNC && launched <= (uint32_t)g_attnNumCUs && launched > (uint32_t)g_attnNumCUs / 2 && resident > g_attnNumCUs)
+  if (s.in.kind != CUSYNC_POLICY_NOSYNC && !(s.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) && launched <= (uint32_t)g_attnNumCUs &&
+      launched > (uint32_t)g_attnNumCUs / 2 && resident > g_attnNumCUs)
     lds = std::max(lds, g_attnLdsPerCU / 2);
   hipLaunchKernelGGL(attnKernel(deep), dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;

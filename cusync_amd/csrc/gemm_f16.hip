@@ -325,9 +325,11 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
   // which with the kernel's few static bytes lets one workgroup onto a CU and leaves the other half to the producer
   // (the same chains: 132-159 us).  A launch of at most half as many workgroups as CUs is left to be packed: it is
   // resident beside the producer at once and leaves whole CUs to the stage after it (measured on the attention
-  // kernel, see cusync_attention_run).
+  // kernel, see cusync_attention_run).  Nor a launch under AvoidWaitKernel, which may reach the device before its
+  // producer: holding half of every CU it could keep a producer that needs more than the other half off the device.
   size_t lds = ti->lds;
-  if (s.in.kind != CUSYNC_POLICY_NOSYNC && launched <= (uint32_t)g_numCUs && launched > (uint32_t)g_numCUs / 2 && ti->residentPerCU > 1)
+  if (s.in.kind != CUSYNC_POLICY_NOSYNC && !(s.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) && launched <= (uint32_t)g_numCUs &&
+      launched > (uint32_t)g_numCUs / 2 && ti->residentPerCU > 1)
     lds = std::max<size_t>(lds, g_ldsPerCU / 2);
   hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;

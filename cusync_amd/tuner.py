@@ -38,18 +38,11 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 
 
-def resident_share(tile, M, N, split, consumer=False):
+def resident_share(tile, M, N, split):
     """Share of the device's workgroup slots a launch of this GEMM takes (1.0 = every slot)."""
-    import torch
     g = api.gemm_grid(tile, M, N, split)
     resident = api._lib.load().cusync_gemm_max_resident(tile)
-    wgs = min(g[0] * g[1] * g[2], resident)
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    # a consumer launch of more than half as many workgroups as CUs, and no more than CUs, takes half a CU's LDS per
-    # workgroup whatever its kernel needs (cusync_gemm_run)
-    if consumer and resident > cus and cus // 2 < wgs <= cus:
-        return wgs / (2.0 * cus)
-    return wgs / float(resident)
+    return min(g[0] * g[1] * g[2], resident) / float(resident)
 
 
 def candidates(batch, n1, n2):
@@ -156,7 +149,7 @@ def tune_batch(bench, batch, log):
         if t_aco is not None and trimmed(t_aco) < tile:
             tile, tile_opts["AvoidCustomOrder"] = trimmed(t_aco), True
         share = (resident_share(kw["tile1"], batch, bench.n1, kw["split_k1"]) +
-                 resident_share(kw["tile2"], batch, bench.hidden, kw["split_k2"], consumer=True))
+                 resident_share(kw["tile2"], batch, bench.hidden, kw["split_k2"]))
         if share <= 1.0:       # both launches are resident together: no wait kernel is needed (CS/cusync.h:193-196, 205-206)
             o = base | api.OPT.AVOID_WAIT_KERNEL | (api.OPT.AVOID_CUSTOM_ORDER if tile_opts["AvoidCustomOrder"] else 0)
             t_awk = bench.run(batch, mode, timed=20, opts=o, **kw)
