@@ -58,6 +58,7 @@ TileInfo* tileInfo(int tile) {
     fillDmaTilesWide(g_tiles);
     fillDmaTilesMid(g_tiles);
     fillDmaTilesFew(g_tiles);
+    fillDmaTilesXWide(g_tiles);
   });
   return &g_tiles[tile];
 }
@@ -155,6 +156,7 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
     if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (partialBytes(a, ti) >= 0x80000000ull) { setError("gemm: the partial sums of these k-slices exceed 2 GiB, more than one buffer descriptor addresses"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   }
+  if (a->tile == CUSYNC_TILE_256x384x32 && a->K % 32) { setError("gemm: the 256x384x32 tile takes K in whole chunks: K must be a multiple of 32"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->a_mode != CUSYNC_A_PLAIN && a->a_mode != CUSYNC_A_SWIGLU) { setError("gemm: unknown a_mode"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_SWIGLU) { setError("gemm: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue == CUSYNC_EPILOGUE_SWIGLU && a->N % 16) { setError("gemm: the SwiGLU epilogue pairs groups of eight columns: N must be a multiple of 16"); return CUSYNC_ERROR_NOT_INITIALIZED; }
@@ -219,10 +221,11 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   // every k-slice has its own workgroup from the start, and the tile's 32-row pieces divide among the slices.
   // Tiles of 128 rows and more only: with the small tiles of the few-row GEMMs, whose slices finish up to 10 us
   // apart, the same scheme (also cut finer, into 32x32 pieces) ended every launch 6-12 us later than the slice
-  // that arrives last doing all of it.
+  // that arrives last doing all of it.  Never under AvoidWaitKernel (see slicesShareReduction).
   const bool direct = ti->chainKernel != nullptr;
-  p.coopReduce = a->split_k > 1 && a->shared_reduction != 0 && direct && p.stage.noDraws && launched == s.grid.x * s.grid.y * s.grid.z &&
-                 ti->bm >= 128 && (ti->bm / 32) % (uint32_t)a->split_k == 0 && !getenv("CUSYNC_NO_COOP_REDUCE");
+  p.coopReduce = slicesShareReduction(a->split_k, a->shared_reduction != 0, direct, p.stage.noDraws, launched,
+                                      s.grid.x * s.grid.y * s.grid.z, ti->bm, (s.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) != 0) &&
+                 !getenv("CUSYNC_NO_COOP_REDUCE");
   return p;
 }
 

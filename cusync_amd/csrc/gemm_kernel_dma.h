@@ -31,6 +31,18 @@
 // barrier sits between the two k-steps of chunk kt and already covers chunk
 // kt+1, so that the fragments of (kt+1, k-step 0) are read under the MFMAs of
 // (kt, k-step 1); the loads of chunk kt+STAGES-1 go into the stage of chunk kt-1.
+//
+// Alternating order (DmaCfg::PINGPONG, for the tiles whose accumulators leave no registers for a second set of
+// fragments: 256x384 is 192 accumulator registers per lane).  What binds these GEMMs is data moved per MFMA — bytes
+// from L2 into LDS through the CU's one vector memory path, bytes from LDS into registers, and the power both
+// cost — so the tile is made as large as the register file allows, and the overlap that a second set of fragments
+// gave a wavefront comes from its neighbour instead.  The eight wavefronts are two groups of four, one wavefront
+// of each group per SIMD.  A wavefront alternates a load phase (the fragments of one k-step from LDS, all at
+// once, into its only set of fragment registers) and a compute phase (that k-step's MFMAs, raised priority, the
+// direct loads of a later chunk issued between them); the second group runs one phase behind the first, so that
+// on every SIMD one wavefront computes while the other loads.  One barrier per chunk keeps the groups in step:
+// the first group meets it between two chunks, the second between the load and the compute phase of a chunk's
+// second k-step.
 #pragma once
 
 #include "gemm_tiles.h"
@@ -38,9 +50,10 @@
 namespace cusync {
 namespace gemm {
 
-template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false, bool PIPE_ = false>
+template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false, bool PIPE_ = false, bool PINGPONG_ = false>
 struct DmaCfg {
   static constexpr bool PIPE = PIPE_;                      // barrier in the middle of a chunk, fragments prefetched across chunks
+  static constexpr bool PINGPONG = PINGPONG_;              // two groups of wavefronts half a k-step apart, fragments held once (see below)
   static constexpr bool BT = BT_;                          // B given as [N][K] (k contiguous), e.g. KRSC filters
   static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // register budget: 512 / this per lane
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
@@ -77,6 +90,7 @@ struct DmaCfg {
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
   static_assert(KS >= 2, "the loads of the next chunk ride on the LDS reads of k-step 1");
   static_assert(!PIPE || (KS == 2 && STAGES >= 3), "the pipelined order is written for two k-steps per chunk");
+  static_assert(!PINGPONG || (KS == 2 && STAGES >= 3 && WAVES == 8 && !PIPE && !BT), "the alternating order is written for eight wavefronts and two k-steps per chunk");
 };
 
 // One direct load: 64 lanes x 16 bytes from buffer `rsrc` at per-lane byte offset
@@ -98,6 +112,18 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
   r.w = 0x00020000u;
   return r;
 }
+
+// What the assembly K loop of the 256x384x32 tile works on (gemm_wide_steps.inc, written by gen_wide_steps.py): LDS
+// addresses of this lane's fragments, byte offsets of its direct loads at K = 0, the operands' descriptors and the
+// LDS addresses its wavefront's loads of stage 0 go to.
+struct WideOperands {
+  uint32_t vA, vB[3];
+  uint32_t a[2], b[3];
+  uint4v rA, rB;
+  uint32_t m0A, m0B;
+  uint32_t dB;            // bytes from one chunk's rows of B to the next chunk's
+};
+#include "gemm_wide_steps.inc"
 
 // One GEMM: all tiles of stage p.stage that this workgroup draws.  CHUNKS: the stage may be a consumer that waits
 // K chunk by K chunk (the tile policies); without it that code is not compiled in (gemm_tiles.h says for which
@@ -126,58 +152,6 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
   const uint4v rB = rawRsrc(p.B, (C::BT ? p.N : p.K) * p.ldb * 2);
   const uint32_t ldsBase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
-  // ---- direct-load side: which global chunk this lane fetches ---------------
-  // A: load q of this wave fills rows (wave*A_LOADS + q)*A_ROWS_PER_LOAD + lane/A_CPR, slot lane%A_CPR.
-  // Rows that share a swizzle value.  A 16-byte-per-lane LDS read is served sixteen lanes at a time over all 64
-  // banks: with 64-byte rows the sixteen rows of such a group cover every bank four times over, so rows r, r+4, r+8
-  // and r+12 must sit in four different slots (four rows per swizzle value: 5.5 clocks per wave instruction on one
-  // CU against 8.0 with two rows per value).
-  constexpr int A_SWZ_DIV = C::A_CPR == 4 ? 4 : 1;
-  const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + lane / C::A_CPR;
-  const uint32_t aLoadChunk = (lane % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
-  // B: the 16-byte slots of a stage are numbered row by row; load q of this wave fills slots
-  // (wave*B_LOADS + q)*64 + lane, i.e. row slot / B_CPR, position slot % B_CPR (a row need not be a
-  // power of two long: 192 columns are 24 slots).  With B given k-contiguous ([N][K]) its stage is laid
-  // out and swizzled exactly like A's.
-  uint32_t bLoadRow[C::B_LOADS], bLoadChunk[C::B_LOADS];
-#pragma unroll
-  for (int q = 0; q < C::B_LOADS; q++) {
-    const uint32_t slot = (wave * C::B_LOADS + q) * 64 + lane;
-    bLoadRow[q] = slot / C::B_CPR;                 // >= B_ROWS for a spare load
-    const uint32_t pos = slot % C::B_CPR;
-    bLoadChunk[q] = C::BT ? pos ^ ((bLoadRow[q] / A_SWZ_DIV) & (C::B_CPR - 1)) : pos ^ (4 * (bLoadRow[q] & 1));
-  }
-  static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
-
-  // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
-  // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
-  uint32_t aFrag[C::KS];
-  {
-    const uint32_t row = wm * C::WTM + (lane & 31);
-    const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
-#pragma unroll
-    for (int kk = 0; kk < C::KS; kk++)
-      aFrag[kk] = row * C::A_ROW_BYTES + (((2 * kk + (lane >> 5)) ^ swz) * 16);
-  }
-  // B fragment: transpose read of rows kk*16 + 8*(lane/32) + 4*t + (lane&15)/4,
-  // 4 halfs at column wn*WTN + j*32 + 16*((lane/16)&1) + 4*(lane&3).
-  // A stage row is kept as 64-byte groups; the group of MFMA tile j is swapped with its neighbour on odd rows.
-  const uint32_t bFlip = (lane >> 2) & 1;                      // parity of the row this lane reads
-  const uint32_t bRowOff = (8 * (lane >> 5) + ((lane & 15) >> 2)) * C::B_ROW_BYTES;
-  const uint32_t bInGroup = (2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 + (lane & 1) * 8;
-  uint32_t bFrag[C::TN];
-#pragma unroll
-  for (int j = 0; j < C::TN; j++) bFrag[j] = bRowOff + (((wn * C::TN + j) ^ bFlip) * 64) + bInGroup;
-  // k-contiguous B: same addressing as the A fragment, rows are output columns.
-  uint32_t bFragT[C::KS];
-  {
-    const uint32_t row = wn * C::WTN + (lane & 31);
-    const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
-#pragma unroll
-    for (int kk = 0; kk < C::KS; kk++)
-      bFragT[kk] = row * C::A_ROW_BYTES + (((2 * kk + (lane >> 5)) ^ swz) * 16);
-  }
-
   const uint32_t numTiles = stage.numTiles();
   const bool consumer = stage.isConsumer();
   const uint32_t tmq = consumer ? stage.d.in.tileM : 1, tnq = consumer ? stage.d.in.tileN : 1;
@@ -205,6 +179,63 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     const uint32_t mEnd = min(m0 + (uint32_t)C::BM, p.M);
     const uint32_t kBegin = t.z * p.kPerSlice, kEnd = min(p.K, kBegin + p.kPerSlice);
     const uint32_t nk = (kEnd - kBegin + C::BK - 1) / C::BK;
+
+    // Where this lane's loads and fragments sit.  Worked out per tile from a lane id the compiler cannot see
+    // through where the tile's accumulators fill the register file (PINGPONG): it would otherwise keep these
+    // fifteen values alive across the main loop for the next tile and reload others from scratch inside it.
+    int laneL = lane;
+    if constexpr (C::PINGPONG) asm volatile("" : "+v"(laneL));
+    // ---- direct-load side: which global chunk this lane fetches ---------------
+    // A: load q of this wave fills rows (wave*A_LOADS + q)*A_ROWS_PER_LOAD + lane/A_CPR, slot lane%A_CPR.
+    // Rows that share a swizzle value.  A 16-byte-per-lane LDS read is served sixteen lanes at a time over all 64
+    // banks: with 64-byte rows the sixteen rows of such a group cover every bank four times over, so rows r, r+4, r+8
+    // and r+12 must sit in four different slots (four rows per swizzle value: 5.5 clocks per wave instruction on one
+    // CU against 8.0 with two rows per value).
+    constexpr int A_SWZ_DIV = C::A_CPR == 4 ? 4 : 1;
+    const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + laneL / C::A_CPR;
+    const uint32_t aLoadChunk = (laneL % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
+    // B: the 16-byte slots of a stage are numbered row by row; load q of this wave fills slots
+    // (wave*B_LOADS + q)*64 + lane, i.e. row slot / B_CPR, position slot % B_CPR (a row need not be a
+    // power of two long: 192 columns are 24 slots).  With B given k-contiguous ([N][K]) its stage is laid
+    // out and swizzled exactly like A's.
+    uint32_t bLoadRow[C::B_LOADS], bLoadChunk[C::B_LOADS];
+#pragma unroll
+    for (int q = 0; q < C::B_LOADS; q++) {
+      const uint32_t slot = (wave * C::B_LOADS + q) * 64 + laneL;
+      bLoadRow[q] = slot / C::B_CPR;                 // >= B_ROWS for a spare load
+      const uint32_t pos = slot % C::B_CPR;
+      bLoadChunk[q] = C::BT ? pos ^ ((bLoadRow[q] / A_SWZ_DIV) & (C::B_CPR - 1)) : pos ^ (4 * (bLoadRow[q] & 1));
+    }
+    static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
+
+    // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
+    // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
+    uint32_t aFrag[C::KS];
+    {
+      const uint32_t row = wm * C::WTM + (laneL & 31);
+      const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
+#pragma unroll
+      for (int kk = 0; kk < C::KS; kk++)
+        aFrag[kk] = row * C::A_ROW_BYTES + (((2 * kk + (laneL >> 5)) ^ swz) * 16);
+    }
+    // B fragment: transpose read of rows kk*16 + 8*(lane/32) + 4*t + (lane&15)/4,
+    // 4 halfs at column wn*WTN + j*32 + 16*((lane/16)&1) + 4*(lane&3).
+    // A stage row is kept as 64-byte groups; the group of MFMA tile j is swapped with its neighbour on odd rows.
+    const uint32_t bFlip = (laneL >> 2) & 1;                      // parity of the row this lane reads
+    const uint32_t bRowOff = (8 * (laneL >> 5) + ((laneL & 15) >> 2)) * C::B_ROW_BYTES;
+    const uint32_t bInGroup = (2 * ((laneL >> 4) & 1) + ((laneL & 3) >> 1)) * 16 + (laneL & 1) * 8;
+    uint32_t bFrag[C::TN];
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) bFrag[j] = bRowOff + (((wn * C::TN + j) ^ bFlip) * 64) + bInGroup;
+    // k-contiguous B: same addressing as the A fragment, rows are output columns.
+    uint32_t bFragT[C::KS];
+    {
+      const uint32_t row = wn * C::WTN + (laneL & 31);
+      const uint32_t swz = (row / A_SWZ_DIV) & (C::A_CPR - 1);
+#pragma unroll
+      for (int kk = 0; kk < C::KS; kk++)
+        bFragT[kk] = row * C::A_ROW_BYTES + (((2 * kk + (laneL >> 5)) ^ swz) * 16);
+    }
 
     floatx16 acc[C::TM][C::TN];
 #pragma unroll
@@ -459,7 +490,9 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // tap and are always waited for one by one.
     constexpr bool perChunk = conv || !ROUNDS;
     auto waitThrough = [&](uint32_t kt) { waitChunk(kBegin + min(kt, nk - 1) * C::BK); };
-    if constexpr (perChunk) waitChunk(kBegin);
+    // (the assembly K loop has no place for waits: a stage of a tile policy waits for all its producer tiles here)
+    if constexpr (C::PINGPONG) waitThrough(nk - 1);
+    else if constexpr (perChunk) waitChunk(kBegin);
     else waitThrough(C::STAGES - 2);
     issueAll(Parity<0>{}, 0);
     if constexpr (C::STAGES > 2) { if constexpr (perChunk) { if (nk > 1) waitChunk(kBegin + C::BK); } issueAll(Parity<1>{}, 1); }
@@ -469,7 +502,29 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
-    if constexpr (C::PIPE) {
+    if constexpr (C::PINGPONG) {
+      // The K loop is assembly (gemm_wide_steps.inc); what it is handed is set up here.
+      static_assert(C::BM == 256 && C::BN == 384 && C::BK == 32 && C::WM == 2 && C::WN == 4 && C::STAGES == 3 && !conv,
+                    "the assembly K loop is written for this tile");
+      WideOperands w;
+      w.vA = ldsBase + aFrag[0];
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) w.vB[j] = ldsBase + C::STAGES * C::A_STAGE + bFrag[j];
+      w.a[0] = aVoff0; w.a[1] = aVoff0 + aVstep;
+#pragma unroll
+      for (int q = 0; q < C::B_LOADS; q++) w.b[q] = bVoff0[q];
+      w.rA = rA; w.rB = rB;
+      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * C::A_LOADS * 1024);
+      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + C::STAGES * C::A_STAGE + wave * C::B_LOADS * 1024);
+      w.dB = C::BK * p.ldb * 2;
+      // The K loop is one assembly statement per group.  The prologue above has issued chunks 0 and 1; the loop
+      // loads chunk 2 next and moves on chunk by chunk while there is another one (past the end it loads the last
+      // chunk again, into a stage nobody reads any more, so that no address leaves the operands).
+      const uint32_t first = min(2u, nk - 1);
+      const uint32_t soffA = (kBegin + first * C::BK) * 2, soffB = (kBegin + first * C::BK) * p.ldb * 2;
+      if (wave < C::WAVES / 2) wideLoopA(acc, w, soffA, soffB, nk, nk - 1 - first);
+      else wideLoopB(acc, w, soffA, soffB, nk, nk - 1 - first);
+    } else if constexpr (C::PIPE) {
       waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");

@@ -29,6 +29,7 @@ void fillStagedTiles(TileInfo* tiles);     // register-staged tiles (the only on
 void fillDmaTilesWide(TileInfo* tiles);    // direct-to-LDS, 256 rows, eight wavefronts
 void fillDmaTilesMid(TileInfo* tiles);     // direct-to-LDS, 128 to 256 rows, four wavefronts
 void fillDmaTilesFew(TileInfo* tiles);     // direct-to-LDS, 32 and 64 rows
+void fillDmaTilesXWide(TileInfo* tiles);   // direct-to-LDS, 256x384, eight wavefronts in two alternating groups
 
 // Entry of a register-staged tile.
 #define CUSYNC_TILE(BM, BN, BK, WM, WN) \

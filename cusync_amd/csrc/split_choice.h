@@ -29,5 +29,18 @@ inline int pickSplit(int requested, uint32_t tiles, uint32_t K, uint32_t bk, int
   return s;
 }
 
+// Whether the k-slices of a tile add it up together (each waits for its siblings, then sums and stores a share of
+// the tile) instead of leaving all of it to the slice that arrives last.  The waiting slices hold their CUs, so
+// every slice of the launch must have a workgroup of its own from the start (one round, all of them dealt a
+// static first tile) and nothing may keep a sibling off the device: under AvoidWaitKernel the consumer's launch
+// can reach the device before its producer's and take the slots the siblings need, the resident slices would
+// spin until their bound runs out, so there the last-arriver form is kept, whose workgroups retire and free
+// their slots.  Tiles of 128 rows and more whose 32-row pieces divide among the slices only.
+inline bool slicesShareReduction(int splitK, bool requested, bool directToLdsTile, bool everyTileStatic, uint32_t launched,
+                                 uint32_t tiles, uint32_t tileM, bool avoidWaitKernel) {
+  return splitK > 1 && requested && directToLdsTile && everyTileStatic && launched == tiles && tileM >= 128 &&
+         (tileM / 32) % (uint32_t)splitK == 0 && !avoidWaitKernel;
+}
+
 }  // namespace gemm
 }  // namespace cusync

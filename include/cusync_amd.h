@@ -243,7 +243,10 @@ enum {
   CUSYNC_TILE_D64x128x64 = 14,       /* direct-to-LDS, 3 stages */
   CUSYNC_TILE_D64x192x64 = 15,       /* direct-to-LDS, 4 stages, a CU to itself: 32 or 64 column tiles times 8 or 4 k-slices are 256 */
   CUSYNC_TILE_128x192x32_ALONE = 16, /* 128x192x32 with 4 stages in the pipelined order and a CU to itself: for GEMMs of about one tile per CU */
-  CUSYNC_TILE_COUNT = 17
+  CUSYNC_TILE_256x384x32 = 17,       /* direct-to-LDS, eight wavefronts of 128x96 in two alternating groups, 3 stages, a CU to itself:
+                                        a third less data moved per MFMA than 256x192; 12288 columns are 32 tiles.  K must be a
+                                        multiple of 32; a stage of a tile policy waits for all its producer tiles before its first load */
+  CUSYNC_TILE_COUNT = 18
 };
 
 typedef struct cusync_gemm_args {
@@ -267,6 +270,8 @@ typedef struct cusync_gemm_args {
                                   the same order, so bit-identical results.  The waiting slices hold their CUs: only for
                                   launches whose workgroups no other kernel keeps off the device while it waits for them
                                   (the chains of this library launch a consumer only after its producer is resident).
+                                  Ignored (the last-arriver form runs) for a stage with CUSYNC_OPT_AVOID_WAIT_KERNEL: without
+                                  the hold-back a consumer's launch may reach the device first and keep sibling slices off it.
                                   No counterpart in the reference, whose split-K reduction is a kernel of its own
                                   (cusyncgemm.h:525-563). */
 } cusync_gemm_args;

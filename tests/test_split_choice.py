@@ -24,6 +24,16 @@ int main() {
     {1, 8256, 64, 256}, {1, 64, 64, 256}};
   for (auto& c : cases) std::printf("P %u %u %u %u %d\n", c[0], c[1], c[2], c[3], pickSplit(0, c[0], c[1], c[2], (int)c[3]));
   std::printf("R %d\n", pickSplit(7, 48, 12288, 64, 256));
+  // shared reduction: (slices, requested, direct tile, all static, launched, tiles, tileM, AvoidWaitKernel)
+  std::printf("S %d\n", slicesShareReduction(4, true, true, true, 256, 256, 256, false) ? 1 : 0);
+  std::printf("S %d\n", slicesShareReduction(4, true, true, true, 256, 256, 256, true) ? 1 : 0);     // consumer may arrive first
+  std::printf("S %d\n", slicesShareReduction(4, false, true, true, 256, 256, 256, false) ? 1 : 0);   // not asked for
+  std::printf("S %d\n", slicesShareReduction(4, true, true, true, 200, 256, 256, false) ? 1 : 0);    // a second round
+  std::printf("S %d\n", slicesShareReduction(4, true, true, true, 256, 256, 64, false) ? 1 : 0);     // few-row tile
+  std::printf("S %d\n", slicesShareReduction(3, true, true, true, 192, 192, 256, false) ? 1 : 0);    // 8 pieces, 3 slices
+  std::printf("S %d\n", slicesShareReduction(1, true, true, true, 256, 256, 256, false) ? 1 : 0);    // no slices
+  std::printf("S %d\n", slicesShareReduction(2, true, false, true, 256, 256, 256, false) ? 1 : 0);   // register-staged tile
+  std::printf("S %d\n", slicesShareReduction(2, true, true, false, 256, 256, 256, false) ? 1 : 0);   // tiles drawn from a dispenser
   return 0;
 }
 """
@@ -36,6 +46,7 @@ def test_split_choice(tmp_path):
     subprocess.check_call(["g++", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "cusync_amd", "csrc"), str(src), "-o", str(exe)])
     out = subprocess.check_output([str(exe)], text=True).split("\n")
     picks = {}
+    shares = []
     for line in out:
         f = line.split()
         if not f:
@@ -48,6 +59,8 @@ def test_split_choice(tmp_path):
             assert got == int(want), (chunks, slices)
         elif f[0] == "P":
             picks[tuple(int(v) for v in f[1:5])] = int(f[5])
+        elif f[0] == "S":
+            shares.append(int(f[1]))
         elif f[0] == "R":
             assert int(f[1]) == 7                     # a requested count is passed through (and validated by the GEMM)
     # one workgroup per CU at most, and at least eight chunks per slice
@@ -60,3 +73,6 @@ def test_split_choice(tmp_path):
     # 129 chunks: sixteen slices of nine would leave the last one empty, and the doubling stops at eight
     assert picks[(1, 8256, 64, 256)] == 8
     assert picks[(1, 64, 64, 256)] == 1
+    # the slices of a tile wait for each other only where nothing can keep a sibling off the device: never for a stage
+    # under AvoidWaitKernel, whose consumer may be dispatched ahead of its producer
+    assert shares == [1, 0, 0, 0, 0, 0, 0, 0, 0]
