@@ -117,10 +117,10 @@ __device__ __forceinline__ uint4v rawRsrc(const void* base, uint32_t bytes) {
 // addresses of this lane's fragments, byte offsets of its direct loads at K = 0, the operands' descriptors and the
 // LDS addresses its wavefront's loads of stage 0 go to.
 struct WideOperands {
-  uint32_t vA, vB[3];
-  uint32_t a[2], b[3];
+  uint32_t vA, vB[3];     // LDS: this lane's A fragment (slot 0, first k-step, first row tile) and its three B fragments (stage 0)
+  uint32_t a[4], b[3];    // byte offsets of this lane's direct loads at the first column of the tile's K range
   uint4v rA, rB;
-  uint32_t m0A, m0B;
+  uint32_t m0A, m0B;      // LDS addresses this wavefront's loads of slot / stage 0 go to
   uint32_t dB;            // bytes from one chunk's rows of B to the next chunk's
 };
 #include "gemm_wide_steps.inc"
@@ -494,8 +494,8 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     if constexpr (C::PINGPONG) waitThrough(nk - 1);
     else if constexpr (perChunk) waitChunk(kBegin);
     else waitThrough(C::STAGES - 2);
-    issueAll(Parity<0>{}, 0);
-    if constexpr (C::STAGES > 2) { if constexpr (perChunk) { if (nk > 1) waitChunk(kBegin + C::BK); } issueAll(Parity<1>{}, 1); }
+    if constexpr (!C::PINGPONG) issueAll(Parity<0>{}, 0);
+    if constexpr (C::STAGES > 2 && !C::PINGPONG) { if constexpr (perChunk) { if (nk > 1) waitChunk(kBegin + C::BK); } issueAll(Parity<1>{}, 1); }
     if constexpr (C::STAGES > 3) { if constexpr (perChunk) { if (nk > 2) waitChunk(kBegin + 2 * C::BK); } issueAll(Parity<2>{}, 2); }
     if constexpr (C::STAGES > 4) { if constexpr (perChunk) { if (nk > 3) waitChunk(kBegin + 3 * C::BK); } issueAll(Parity<3>{}, 3); }
     static_assert(C::STAGES >= 2 && C::STAGES <= 5, "prologue written for 2..5 stages");
@@ -503,27 +503,48 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
     if constexpr (C::PINGPONG) {
-      // The K loop is assembly (gemm_wide_steps.inc); what it is handed is set up here.
+      // The K loop is assembly (gemm_wide_steps.inc); its LDS layout and what it is handed are set up here.  A is
+      // kept 64 columns of K at a time, [256 rows][128 bytes] in a ring of two slots, so that every piece fetched
+      // from memory is a whole cache line; B in the ring of three 32-row stages behind it.
       static_assert(C::BM == 256 && C::BN == 384 && C::BK == 32 && C::WM == 2 && C::WN == 4 && C::STAGES == 3 && !conv,
                     "the assembly K loop is written for this tile");
+      constexpr uint32_t A_SLOT = 256 * 128, B_BASE = 2 * A_SLOT;
+      static_assert(B_BASE + 3 * C::B_STAGE <= C::LDS_BYTES, "two A slots and three B stages fit the workgroup's LDS");
       WideOperands w;
-      w.vA = ldsBase + aFrag[0];
+      {
+        // fragment side: row (laneL & 31) of the wavefront's first MFMA row tile, 16-byte piece (laneL >> 5) of the
+        // k-step.  The eight pieces of a row are swizzled with bits 1..3 of the row number: an LDS read serves
+        // sixteen lanes at a time, sixteen consecutive rows here, and with 128-byte rows two rows cover all banks once,
+        // so rows 2n and 2n+1 take one position and the eight pairs eight different ones.
+        const uint32_t row = wm * C::WTM + (laneL & 31);
+        w.vA = ldsBase + row * 128 + ((((uint32_t)laneL >> 5) ^ ((row >> 1) & 7)) * 16);
 #pragma unroll
-      for (int j = 0; j < C::TN; j++) w.vB[j] = ldsBase + C::STAGES * C::A_STAGE + bFrag[j];
-      w.a[0] = aVoff0; w.a[1] = aVoff0 + aVstep;
+        for (int j = 0; j < C::TN; j++) w.vB[j] = ldsBase + B_BASE + bFrag[j];
+        // load side: load q of this wavefront fills rows wave * 32 + q * 8 + laneL / 8 of a slot; the lane at piece
+        // position p of a row fetches the piece that belongs there under the swizzle
 #pragma unroll
-      for (int q = 0; q < C::B_LOADS; q++) w.b[q] = bVoff0[q];
+        for (int q = 0; q < 4; q++) {
+          const uint32_t lrow = q * 8 + ((uint32_t)laneL >> 3), piece = ((uint32_t)laneL & 7) ^ ((lrow >> 1) & 7);
+          w.a[q] = ((m0 + wave * 32 + lrow) * p.lda + kBegin + piece * 8) * 2;
+        }
+#pragma unroll
+        for (int q = 0; q < C::B_LOADS; q++) w.b[q] = bVoff0[q] == kOutOfRange ? kOutOfRange : bVoff0[q] + kBegin * p.ldb * 2;
+      }
       w.rA = rA; w.rB = rB;
-      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * C::A_LOADS * 1024);
-      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + C::STAGES * C::A_STAGE + wave * C::B_LOADS * 1024);
+      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * 4096);
+      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + B_BASE + wave * C::B_LOADS * 1024);
       w.dB = C::BK * p.ldb * 2;
-      // The K loop is one assembly statement per group.  The prologue above has issued chunks 0 and 1; the loop
-      // loads chunk 2 next and moves on chunk by chunk while there is another one (past the end it loads the last
-      // chunk again, into a stage nobody reads any more, so that no address leaves the operands).
-      const uint32_t first = min(2u, nk - 1);
-      const uint32_t soffA = (kBegin + first * C::BK) * 2, soffB = (kBegin + first * C::BK) * p.ldb * 2;
-      if (wave < C::WAVES / 2) wideLoopA(acc, w, soffA, soffB, nk, nk - 1 - first);
-      else wideLoopB(acc, w, soffA, soffB, nk, nk - 1 - first);
+      // A slot 0 and chunks 0 and 1 of B (K is a whole number of slots: at least two chunks)
+#pragma unroll
+      for (int q = 0; q < 4; q++) loadToLds(rA, __builtin_amdgcn_readfirstlane(w.m0A + q * 1024), w.a[q]);
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int q = 0; q < C::B_LOADS; q++)
+          loadToLds(rB, __builtin_amdgcn_readfirstlane(w.m0B + c * C::B_STAGE + q * 1024), w.b[q] == kOutOfRange ? kOutOfRange : w.b[q] + c * w.dB);
+      // The loop loads chunk 2 next and moves on chunk by chunk while there is another one.
+      const uint32_t soffA = min(2u, nk - 1) * 64;
+      wideLoop(acc, w, soffA, nk);
     } else if constexpr (C::PIPE) {
       waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
       __builtin_amdgcn_s_barrier();

@@ -70,8 +70,8 @@ def test_gemm_exact_on_integer_data(tile):
 def test_gemm_matches_oracle(tile, shape):
     print("tile", tile, "shape", shape, flush=True)
     M, N, K = shape
-    if tile == api.TILE.T256x384x32 and K % 32:
-        pytest.skip("the 256x384x32 tile takes K in whole chunks of 32 (refused by cusync_gemm_can_implement, see test_gemm_can_implement_rejects)")
+    if tile == api.TILE.T256x384x32 and K % 64:
+        pytest.skip("the 256x384x32 tile takes K 64 columns at a time (refused by cusync_gemm_can_implement, see test_gemm_can_implement_rejects)")
     a = uniform_f16((M, K), 1)
     b = normal_f16((K, N), 2, std=0.05)
     got = run_gemm(a, b, tile)
@@ -115,7 +115,7 @@ def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
     # descriptor rejects).  K = 24 is a single, partly filled chunk (fewer chunks than pipeline stages), 200 a
     # few, 1032 many and a ragged last one.  Two launches, GeLU epilogue.
     if tile == api.TILE.T256x384x32:
-        K = {24: 32, 200: 192, 1032: 1024}[K]        # this tile takes K in whole chunks: one, as many as stages plus a few, many
+        K = {24: 64, 200: 192, 1032: 1024}[K]        # this tile takes K 64 columns at a time: one slot of A, three, many
     print("several tiles per workgroup, tile", tile, "K", K, flush=True)
     M, N = 600, 1000
     a = uniform_f16((M, K), 41)
@@ -136,6 +136,8 @@ def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
 @pytest.mark.parametrize("split", [2, 3, 8])
 def test_gemm_split_k(tile, split):
     print("split-k tile", tile, "slices", split, flush=True)
+    if tile == api.TILE.T256x384x32 and split == 3:
+        pytest.skip("32 chunks in three slices of eleven: the 256x384x32 tile takes whole pairs of chunks per slice")
     rng = np.random.default_rng(tile * 10 + split)
     M, N, K = 200, 392, 1024
     a = rng.integers(-2, 3, (M, K)).astype(np.float16)
@@ -193,10 +195,14 @@ def test_gemm_can_implement_rejects():
     bad = api.gemm_args(st, 300, 64, 64, 16, 64, 16, 64, 16, 64, api.TILE.T128x128x64)   # grid mismatch
     assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "grid" in api.last_error()
     st.destroy()
-    # the 256x384x32 tile walks K in whole chunks of 32
+    # the 256x384x32 tile walks K 64 columns at a time, in every k-slice
     stw = plain_stage(api.TILE.T256x384x32, 64, 64)
-    bad = api.gemm_args(stw, 64, 64, 72, 16, 72, 16, 64, 16, 64, api.TILE.T256x384x32)
-    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "multiple of 32" in api.last_error()
+    bad = api.gemm_args(stw, 64, 64, 96, 16, 96, 16, 64, 16, 64, api.TILE.T256x384x32)
+    assert L.cusync_gemm_can_implement(C.byref(bad)) == api.ERR.NOT_INITIALIZED and "multiple of 64" in api.last_error()
+    stw.destroy()
+    stw = plain_stage(api.TILE.T256x384x32, 64, 64, split_k=3)
+    ws = api.gemm_args(stw, 64, 64, 1024, 16, 1024, 16, 64, 16, 64, api.TILE.T256x384x32, split_k=3, workspace=16)   # 32 chunks in slices of 11
+    assert L.cusync_gemm_can_implement(C.byref(ws)) == api.ERR.NOT_INITIALIZED and "multiple of 64" in api.last_error()
     stw.destroy()
     # NoAtomicAdd with a counting policy is refused (RowSync counts to gN)
     g = api.gemm_grid(api.TILE.T128x128x64, 256, 512)
