@@ -246,8 +246,10 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
                     : S <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
   const int wide3 = S <= 32 ? small : S <= 256 ? CUSYNC_TILE_D64x192x64 : S <= 512 ? CUSYNC_TILE_128x192x32_ALONE
                     : S <= 1024 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;
-  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? wide1 : dflt;
-  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? wide3 : dflt;
+  // (where K is a multiple of 64, the 256x192 tile that fetches both operands 64 columns at a time, K loop in assembly)
+  auto inLines = [](int tile, uint32_t K) { return tile == CUSYNC_TILE_256x192x32 && K % 64 == 0 ? (int)CUSYNC_TILE_256x192x64 : tile; };
+  L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? inLines(wide1, cfg->hidden) : dflt;
+  L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? inLines(wide3, L->E) : dflt;
   L->ws1 = L->ws3 = L->ws2 = nullptr;
   // Key ranges of 8 blocks (512 rows) or more are cut in two: under a causal mask the last row tiles walk the
   // longest ranges and the launch is as long as its longest workgroup.  Measured alone at 12 heads: 512 rows

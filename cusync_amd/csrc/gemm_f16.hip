@@ -156,11 +156,11 @@ cusync_error cusync_gemm_can_implement(const cusync_gemm_args* a) {
     if (a->N % 4) { setError("gemm: split_k needs N % 4 == 0"); return CUSYNC_ERROR_NOT_INITIALIZED; }
     if (partialBytes(a, ti) >= 0x80000000ull) { setError("gemm: the partial sums of these k-slices exceed 2 GiB, more than one buffer descriptor addresses"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   }
-  if (a->tile == CUSYNC_TILE_256x384x32) {
+  if (a->tile == CUSYNC_TILE_256x384x32 || a->tile == CUSYNC_TILE_256x192x64) {
     // A is fetched 64 columns of K at a time, and nothing masks a piece that reaches past the end of a row or of a k-slice
     const uint32_t chunks = a->K / 32, slices = (uint32_t)std::max(a->split_k, 1);
-    if (a->K % 64 || ((chunks + slices - 1) / slices) % 2) {
-      setError("gemm: the 256x384x32 tile takes K 64 columns at a time: K (and with split_k > 1 every k-slice) must be a multiple of 64");
+    if (a->K % 64 || (a->tile == CUSYNC_TILE_256x384x32 && ((chunks + slices - 1) / slices) % 2)) {
+      setError("gemm: the 256x384x32 and 256x192x64 tiles take K 64 columns at a time: K (and with split_k > 1 every k-slice) must be a multiple of 64");
       return CUSYNC_ERROR_NOT_INITIALIZED;
     }
   }

@@ -90,7 +90,7 @@ struct DmaCfg {
   static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
   static_assert(KS >= 2, "the loads of the next chunk ride on the LDS reads of k-step 1");
   static_assert(!PIPE || (KS == 2 && STAGES >= 3), "the pipelined order is written for two k-steps per chunk");
-  static_assert(!PINGPONG || (KS == 2 && STAGES >= 3 && WAVES == 8 && !PIPE && !BT), "the alternating order is written for eight wavefronts and two k-steps per chunk");
+  static_assert(!PINGPONG || (WAVES == 8 && !PIPE && !BT && BM == 256 && ((BN == 384 && BK == 32) || (BN == 192 && BK == 64))), "the assembly K loops are written for two tiles");
 };
 
 // One direct load: 64 lanes x 16 bytes from buffer `rsrc` at per-lane byte offset
@@ -191,7 +191,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // banks: with 64-byte rows the sixteen rows of such a group cover every bank four times over, so rows r, r+4, r+8
     // and r+12 must sit in four different slots (four rows per swizzle value: 5.5 clocks per wave instruction on one
     // CU against 8.0 with two rows per value).
-    constexpr int A_SWZ_DIV = C::A_CPR == 4 ? 4 : 1;
+    constexpr int A_SWZ_DIV = C::A_CPR == 4 ? 4 : C::PINGPONG ? 2 : 1;      // (128-byte rows: two rows cover all banks once)
     const uint32_t aLoadRow = wave * C::A_LOADS * C::A_ROWS_PER_LOAD + laneL / C::A_CPR;
     const uint32_t aLoadChunk = (laneL % C::A_CPR) ^ ((aLoadRow / A_SWZ_DIV) & (C::A_CPR - 1));
     // B: the 16-byte slots of a stage are numbered row by row; load q of this wave fills slots
@@ -206,7 +206,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       const uint32_t pos = slot % C::B_CPR;
       bLoadChunk[q] = C::BT ? pos ^ ((bLoadRow[q] / A_SWZ_DIV) & (C::B_CPR - 1)) : pos ^ (4 * (bLoadRow[q] & 1));
     }
-    static_assert(C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");
+    static_assert(C::PINGPONG || C::A_ROWS_PER_LOAD % (A_SWZ_DIV * C::A_CPR) == 0, "swizzle repeats per load");      // (the assembly loops set their loads up themselves)
 
     // ---- fragment side: where this lane's MFMA operands sit inside a stage -----
     // A fragment of k-step kk: row (lane&31) of the 32-row MFMA tile, chunk 2*kk + lane/32.
@@ -502,7 +502,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
-    if constexpr (C::PINGPONG) {
+    if constexpr (C::PINGPONG && C::BN == 384) {
       // The K loop is assembly (gemm_wide_steps.inc); its LDS layout and what it is handed are set up here.  A is
       // kept 64 columns of K at a time, [256 rows][128 bytes] in a ring of two slots, so that every piece fetched
       // from memory is a whole cache line; B in the ring of three 32-row stages behind it.
@@ -545,6 +545,39 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       // The loop loads chunk 2 next and moves on chunk by chunk while there is another one.
       const uint32_t soffA = min(2u, nk - 1) * 64;
       wideLoop(acc, w, soffA, nk);
+    } else if constexpr (C::PINGPONG) {
+      // 256x192, both operands 64 columns of K at a time: A [256 rows][128 bytes] in a ring of two slots, B
+      // [64 k rows][384 bytes] in a ring of three behind it; the K loop is assembly (gemm_wide_steps.inc).
+      static_assert(C::BN == 192 && C::BK == 64 && C::WM == 4 && C::WN == 2 && !conv, "the assembly K loop is written for this tile");
+      constexpr uint32_t B_BASE = 2 * C::A_STAGE;
+      static_assert(B_BASE + 3 * C::B_STAGE <= C::LDS_BYTES, "two A slots and three B slots fit the workgroup's LDS");
+      WideOperands w;
+      w.vA = ldsBase + aFrag[0];
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) w.vB[j] = ldsBase + B_BASE + bFrag[j];
+      // load q of this wavefront fills rows wave * 32 + q * 8 + laneL / 8 of a slot; the lane at piece position p of a
+      // row fetches the piece that belongs there under the swizzle (which differs from load to load)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const uint32_t lrow = q * 8 + ((uint32_t)laneL >> 3), piece = ((uint32_t)laneL & 7) ^ ((lrow >> 1) & 7);
+        w.a[q] = ((m0 + wave * 32 + lrow) * p.lda + kBegin + piece * 8) * 2;
+      }
+#pragma unroll
+      for (int q = 0; q < C::B_LOADS; q++) w.b[q] = bVoff0[q] == kOutOfRange ? kOutOfRange : bVoff0[q] + kBegin * p.ldb * 2;
+      w.rA = rA; w.rB = rB;
+      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * C::A_LOADS * 1024);
+      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + B_BASE + wave * C::B_LOADS * 1024);
+      w.dB = C::BK * p.ldb * 2;
+      const uint32_t last = nk - 1;
+      // A slot 0, B slots 0 and 1 (the last slot again if there is only one)
+#pragma unroll
+      for (int q = 0; q < 4; q++) loadToLds(rA, __builtin_amdgcn_readfirstlane(w.m0A + q * 1024), w.a[q]);
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int q = 0; q < C::B_LOADS; q++)
+          loadToLds(rB, __builtin_amdgcn_readfirstlane(w.m0B + c * C::B_STAGE + q * 1024), w.b[q] == kOutOfRange ? kOutOfRange : w.b[q] + min((uint32_t)c, last) * w.dB);
+      pairLoop192(acc, w, min(1u, last) * 128, nk, last);
     } else if constexpr (C::PIPE) {
       waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
       __builtin_amdgcn_s_barrier();

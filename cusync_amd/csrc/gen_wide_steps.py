@@ -222,6 +222,128 @@ def loop():
 
 TAIL = ["s_nop 7", "s_nop 4"]        # the last MFMAs' results are not the compiler's to touch before they are written
 
+# ---------------------------------------------------------------------------------------------------------------
+# The 256x192 tile with both operands 64 columns of K at a time (DmaCfg<256, 192, 64, 4, 2, ...>): eight wavefronts of
+# 64x96 (96 accumulator registers), so there is room for two sets of fragments: the reads of a k-step's fragments go
+# out between the MFMAs of the k-step before.  LDS: [A slot 0..1: 256 rows x 128 B][B slot 0..2: 64 k rows x 384 B].
+# One barrier per slot (four k-steps): barrier x, passed when slot x of both operands has landed for everyone, sits in
+# front of the last k-step of slot x-1, whose reads are the first of slot x; behind it everyone issues A slot x+1 (four
+# loads, into the A slot that slot x-1 has just left) and B slot x+2 (three loads).
+F2 = 200                                       # fragment sets: set s at F2 + 20 s: A0, A1 (four registers each), B0..B2
+TMP2 = 240
+A_SLOT2, B_SLOT2 = 256 * 128, 64 * 384
+PERIOD2 = 6
+
+
+def fa2(s, i):
+    return F2 + 20 * s + 4 * i
+
+
+def fb2(s, j):
+    return F2 + 20 * s + 8 + 4 * j
+
+
+def frag_reads2(x, kp, s):
+    """Reads of k-step kp (0..3) of slot x into fragment set s: list of (ins, ...) groups, one group per fragment."""
+    aslot, bslot = x % 2, x % 3
+    groups = []
+    pre = []
+    a_addr = "%[vA]"
+    if kp:
+        pre = ["v_xor_b32 v%d, %d, %%[vA]" % (TMP2, 32 * kp)]
+        a_addr = "v%d" % TMP2
+    for i in range(2):
+        groups.append((pre if i == 0 else []) + ["ds_read_b128 %s, %s offset:%d" % (v(fa2(s, i), 4), a_addr, aslot * A_SLOT2 + i * 4096)])
+    for j in range(3):
+        off = bslot * B_SLOT2 + kp * 16 * 384
+        addr = "%%[vB%d]" % j
+        pre = []
+        if off + 4 * 384 > 65535:              # beyond the instruction's 16-bit offset: through a register
+            pre = ["v_add_u32 v%d, %d, %%[vB%d]" % (TMP2 + 1, bslot * B_SLOT2, j)]
+            addr, off = "v%d" % (TMP2 + 1), kp * 16 * 384
+        groups.append(pre + ["ds_read_b64_tr_b16 %s, %s offset:%d" % (v(fb2(s, j), 2), addr, off),
+                             "ds_read_b64_tr_b16 %s, %s offset:%d" % (v(fb2(s, j) + 2, 2), addr, off + 4 * 384)])
+    return groups
+
+
+def batch2(x):
+    """Direct loads behind barrier x: A slot x+1, B slot x+2."""
+    out = []
+    for q in range(4):
+        pre = ["s_lshr_b32 vcc_hi, %[soffA], 7", "s_add_u32 vcc_hi, vcc_hi, 1", "s_min_u32 vcc_hi, vcc_hi, %[last]",
+               "s_mul_i32 vcc_hi, vcc_hi, %[dB]"] if q == 0 else []
+        out.append(pre + ["s_add_u32 m0, %%[m0A], %d" % (((x + 1) % 2) * A_SLOT2 + q * 1024),
+                          "buffer_load_dwordx4 %%[a%d], %%[rA], %%[soffA] offen lds" % q])
+    for q in range(3):
+        out.append(["s_add_u32 m0, %%[m0B], %d" % (((x + 2) % 3) * B_SLOT2 + q * 1024),
+                    "buffer_load_dwordx4 %%[b%d], %%[rB], vcc_hi offen lds" % q])
+    return out
+
+
+def kstep2(out, x, kp):
+    """Six MFMAs of k-step kp of slot x on fragment set kp % 2; the reads of the next k-step go out between them, and
+    in front of the last k-step of a slot sits barrier x+1 with its loads behind."""
+    s = kp % 2
+    nx, nkp = (x, kp + 1) if kp < 3 else (x + 1, 0)
+    reads = [] if "noread" in OPTS else frag_reads2(nx % PERIOD2, nkp, 1 - s)
+    loads = batch2((x + 1) % PERIOD2) if kp == 3 else []
+    out.append("s_waitcnt lgkmcnt(0)")                       # this k-step's fragments (read a k-step ago)
+    if kp == 3:
+        out += ["s_waitcnt vmcnt(3)", "s_barrier"]           # slot x+1 has landed for everyone; slot x's last reads are done
+    n = 0
+    for j in range(3):
+        for i in range(2):
+            if "nomfma" not in OPTS:
+                out.append("v_mfma_f32_32x32x16_f16 %%[c%d%d], %s, %s, %%[c%d%d]" % (i, j, v(fb2(s, j), 4), v(fa2(s, i), 4), i, j))
+            if n < len(reads):
+                out += reads[n]
+            if loads:
+                out += loads[n]
+                if n == 5:
+                    out += loads[6]
+            n += 1
+    # (five fragment reads on six MFMAs)
+
+
+def loop192():
+    out = ["s_waitcnt vmcnt(3)", "s_barrier"]                # barrier 0: slot 0 of both operands
+    for load in batch2(0):
+        out += load
+    out += ["s_cmp_gt_u32 %[left], 2", "s_cselect_b32 vcc_lo, 128, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo"]
+    for g in ([] if "noread" in OPTS else frag_reads2(0, 0, 0)):
+        out += g
+    out.append("LOOP_%=:")
+    for x in range(PERIOD2):
+        for kp in range(4):
+            kstep2(out, x, kp)
+        # behind the loads of barrier x+1 (A slot x+2, B slot x+3): on while there is another slot
+        out += ["s_cmp_gt_u32 %[left], 3", "s_cselect_b32 vcc_lo, 128, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo",
+                "s_sub_u32 %[left], %[left], 1", "s_cmp_eq_u32 %[left], 0",
+                "s_cbranch_scc1 DONE_%=" if x < PERIOD2 - 1 else "s_cbranch_scc0 LOOP_%="]
+    out += ["DONE_%=:", "s_waitcnt lgkmcnt(0)"]
+    return out + TAIL
+
+
+CLOBBERS2 = ", ".join('"v%d"' % r for r in range(F2, TMP2 + 2)) + ', "vcc", "scc", "memory"'
+ACC_OPS2 = ", ".join('[c%d%d] "+v"(acc[%d][%d])' % (i, j, i, j) for i in range(2) for j in range(3))
+IN_OPS2 = ('[vA] "v"(w.vA), [vB0] "v"(w.vB[0]), [vB1] "v"(w.vB[1]), [vB2] "v"(w.vB[2]), '
+           '[a0] "v"(w.a[0]), [a1] "v"(w.a[1]), [a2] "v"(w.a[2]), [a3] "v"(w.a[3]), [b0] "v"(w.b[0]), [b1] "v"(w.b[1]), [b2] "v"(w.b[2]), '
+           '[rA] "s"(w.rA), [rB] "s"(w.rB), [m0A] "s"(w.m0A), [m0B] "s"(w.m0B), [dB] "s"(w.dB), [last] "s"(last)')
+
+
+def function192(name, body):
+    text = "\\n\\t".join(body)
+    lines = ["// soffA: 128 bytes x the A slot whose loads go out next (A slot 0 and B slots 0 and 1 are the caller's; the B slot that",
+             "// goes out with it is the one after, held at `last`, the last slot there is); left: slots to compute.",
+             "__device__ __forceinline__ void %s(floatx16 (&acc)[2][3], const WideOperands& w, uint32_t soffA, uint32_t left, uint32_t last) {" % name,
+             '  asm volatile("%s"' % text,
+             "               : %s, %s" % (ACC_OPS2, STATE_OPS),
+             "               : %s" % IN_OPS2,
+             "               : %s);" % CLOBBERS2,
+             "}"]
+    return "\n".join(lines)
+
+
 CLOBBERS = ", ".join('"v%d"' % r for r in range(T, TMP + 1)) + ', "vcc", "scc", "memory"'
 ACC_OPS = ", ".join('[c%d%d] "+v"(acc[%d][%d])' % (i, j, i, j) for i in range(4) for j in range(3))
 STATE_OPS = '[soffA] "+s"(soffA), [left] "+s"(left)'
@@ -244,7 +366,7 @@ def function(name, body):
 
 def main():
     out = ["// Generated by gen_wide_steps.py; do not edit.  The K loop of the 256x384x32 tile (see that script).",
-           "#pragma once", "", function("wideLoop", loop()), ""]
+           "#pragma once", "", function("wideLoop", loop()), "", function192("pairLoop192", loop192()), ""]
     path = os.environ.get("WIDE_OUT") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_wide_steps.inc")
     with open(path, "w") as f:
         f.write("\n".join(out))

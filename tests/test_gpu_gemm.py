@@ -70,8 +70,8 @@ def test_gemm_exact_on_integer_data(tile):
 def test_gemm_matches_oracle(tile, shape):
     print("tile", tile, "shape", shape, flush=True)
     M, N, K = shape
-    if tile == api.TILE.T256x384x32 and K % 64:
-        pytest.skip("the 256x384x32 tile takes K 64 columns at a time (refused by cusync_gemm_can_implement, see test_gemm_can_implement_rejects)")
+    if tile in (api.TILE.T256x384x32, api.TILE.T256x192x64) and K % 64:
+        pytest.skip("the tiles with the K loop in assembly take K 64 columns at a time (refused by cusync_gemm_can_implement, see test_gemm_can_implement_rejects)")
     a = uniform_f16((M, K), 1)
     b = normal_f16((K, N), 2, std=0.05)
     got = run_gemm(a, b, tile)
@@ -107,15 +107,15 @@ def test_gemm_persistent_launch_smaller_than_grid():
 
 @pytest.mark.parametrize("tile", [api.TILE.T256x192x32, api.TILE.T256x256x32, api.TILE.T256x128x32, api.TILE.T128x128x32,
                                   api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x192x32_ALONE, api.TILE.D64x192x64,
-                                  api.TILE.T256x384x32])
+                                  api.TILE.T256x384x32, api.TILE.T256x192x64])
 @pytest.mark.parametrize("K", [24, 200, 1032])
 def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
     # 3 workgroups for 12 to 88 tiles with ragged edges: every workgroup goes from one tile's stores straight into
     # the next tile's loads, and the stores outside the matrix are issued all the same (with an offset the buffer
     # descriptor rejects).  K = 24 is a single, partly filled chunk (fewer chunks than pipeline stages), 200 a
     # few, 1032 many and a ragged last one.  Two launches, GeLU epilogue.
-    if tile == api.TILE.T256x384x32:
-        K = {24: 64, 200: 192, 1032: 1024}[K]        # this tile takes K 64 columns at a time: one slot of A, three, many
+    if tile in (api.TILE.T256x384x32, api.TILE.T256x192x64):
+        K = {24: 64, 200: 192, 1032: 1024}[K]        # these tiles take K 64 columns at a time: one slot of A, three, many
     print("several tiles per workgroup, tile", tile, "K", K, flush=True)
     M, N = 600, 1000
     a = uniform_f16((M, K), 41)
@@ -132,7 +132,7 @@ def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
 
 
 @pytest.mark.parametrize("tile", [api.TILE.T128x128x64, api.TILE.T32x128x64, api.TILE.T128x256x32, api.TILE.T256x256x32,
-                                  api.TILE.T128x128x32, api.TILE.T256x384x32])
+                                  api.TILE.T128x128x32, api.TILE.T256x384x32, api.TILE.T256x192x64])
 @pytest.mark.parametrize("split", [2, 3, 8])
 def test_gemm_split_k(tile, split):
     print("split-k tile", tile, "slices", split, flush=True)
@@ -154,7 +154,7 @@ def test_gemm_split_k(tile, split):
 @pytest.mark.parametrize("tile,split", [(api.TILE.T256x192x32, 2), (api.TILE.T256x192x32, 4), (api.TILE.T256x192x32, 8),
                                         (api.TILE.T128x192x32_ALONE, 4), (api.TILE.D64x192x64, 2), (api.TILE.T256x256x32, 4),
                                         (api.TILE.T256x192x32, 3), (api.TILE.D32x128x64, 4), (api.TILE.T256x384x32, 2),
-                                        (api.TILE.T256x384x32, 4)])
+                                        (api.TILE.T256x384x32, 4), (api.TILE.T256x192x64, 2), (api.TILE.T256x192x64, 4)])
 def test_gemm_split_k_with_the_reduction_shared_among_the_slices(tile, split):
     # every k-slice has a workgroup of its own, so the slices of a tile each add up and store a share of it (where
     # the tile has 128 rows or more and its 32-row pieces divide among them: not for 3 slices, not for the 64- and
@@ -275,7 +275,8 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
                                    (api.TILE.D32x128x64, api.TILE.D64x192x64),        # few-row direct-to-LDS tiles
                                    (api.TILE.D64x192x64, api.TILE.T128x192x32),
                                    (api.TILE.T256x192x32, api.TILE.T256x384x32),      # consumer with the K loop in assembly
-                                   (api.TILE.T256x384x32, api.TILE.T256x192x32)])
+                                   (api.TILE.T256x384x32, api.TILE.T256x192x32),
+                                   (api.TILE.T256x192x64, api.TILE.T256x384x32)])     # as the 2048-row MLP runs them
 def test_two_chained_gemms_config1(policy_kind, opts, tiles):
     # BASELINE config 1: M=256, N=K=1024, fp32 accumulate, inputs uniform from a seed
     print("chained", policy_kind, opts, tiles, flush=True)
