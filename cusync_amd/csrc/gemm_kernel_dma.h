@@ -100,6 +100,12 @@ __device__ __forceinline__ void loadToLds(uint4v rsrc, uint32_t ldsAddr, uint32_
                :: "s"(ldsAddr), "v"(voff), "s"(rsrc) : "memory");
 }
 
+// The same for the lower 32 lanes only (512 bytes); the wavefront must be fully active around it.
+__device__ __forceinline__ void loadToLdsLowerHalf(uint4v rsrc, uint32_t ldsAddr, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_mov_b64 exec, 0xffffffff\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds\n\ts_mov_b64 exec, -1"
+               :: "s"(ldsAddr), "v"(voff), "s"(rsrc) : "memory");
+}
+
 template<int N>
 __device__ __forceinline__ void waitVmcnt() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
@@ -546,38 +552,45 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
       const uint32_t soffA = min(2u, nk - 1) * 64;
       wideLoop(acc, w, soffA, nk);
     } else if constexpr (C::PINGPONG) {
-      // 256x192, both operands 64 columns of K at a time: A [256 rows][128 bytes] in a ring of two slots, B
-      // [64 k rows][384 bytes] in a ring of three behind it; the K loop is assembly (gemm_wide_steps.inc).
+      // 256x192 in whole cache lines: A [256 rows][128 bytes = 64 columns of K] in a ring of three slots, B in stages
+      // of [32 k rows][384 bytes] in a ring of four behind it; the K loop is assembly (gemm_wide_steps.inc).
       static_assert(C::BN == 192 && C::BK == 64 && C::WM == 4 && C::WN == 2 && !conv, "the assembly K loop is written for this tile");
-      constexpr uint32_t B_BASE = 2 * C::A_STAGE;
-      static_assert(B_BASE + 3 * C::B_STAGE <= C::LDS_BYTES, "two A slots and three B slots fit the workgroup's LDS");
+      constexpr uint32_t B_BASE = 3 * C::A_STAGE, B_STAGE32 = 32 * C::B_ROW_BYTES;
+      static_assert(B_BASE + 4 * B_STAGE32 <= C::LDS_BYTES, "three A slots and four B stages fit the workgroup's LDS");
       WideOperands w;
       w.vA = ldsBase + aFrag[0];
 #pragma unroll
       for (int j = 0; j < C::TN; j++) w.vB[j] = ldsBase + B_BASE + bFrag[j];
-      // load q of this wavefront fills rows wave * 32 + q * 8 + laneL / 8 of a slot; the lane at piece position p of a
-      // row fetches the piece that belongs there under the swizzle (which differs from load to load)
+      // A: load q of this wavefront fills rows wave * 32 + q * 8 + laneL / 8 of a slot; the lane at piece position p
+      // of a row fetches the piece that belongs there under the swizzle (which differs from load to load)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         const uint32_t lrow = q * 8 + ((uint32_t)laneL >> 3), piece = ((uint32_t)laneL & 7) ^ ((lrow >> 1) & 7);
         w.a[q] = ((m0 + wave * 32 + lrow) * p.lda + kBegin + piece * 8) * 2;
       }
+      // B: a stage is 768 pieces of 16 bytes, 96 per wavefront: a load of all 64 lanes and one of the lower 32
 #pragma unroll
-      for (int q = 0; q < C::B_LOADS; q++) w.b[q] = bVoff0[q] == kOutOfRange ? kOutOfRange : bVoff0[q] + kBegin * p.ldb * 2;
+      for (int q = 0; q < 2; q++) {
+        const uint32_t slot = wave * 96 + q * 64 + (uint32_t)laneL, brow = slot / C::B_CPR, piece = (slot % C::B_CPR) ^ (4 * (brow & 1));
+        w.b[q] = n0 + piece * 8 < p.N ? ((kBegin + brow) * p.ldb + n0 + piece * 8) * 2 : kOutOfRange;
+      }
       w.rA = rA; w.rB = rB;
-      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * C::A_LOADS * 1024);
-      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + B_BASE + wave * C::B_LOADS * 1024);
-      w.dB = C::BK * p.ldb * 2;
-      const uint32_t last = nk - 1;
-      // A slot 0, B slots 0 and 1 (the last slot again if there is only one)
+      w.m0A = __builtin_amdgcn_readfirstlane(ldsBase + wave * 4096);
+      w.m0B = __builtin_amdgcn_readfirstlane(ldsBase + B_BASE + wave * 1536);
+      w.dB = 32 * p.ldb * 2;
+      const uint32_t chunks = 2 * nk, lastSlot = (chunks - 2) * 64;         // nk counts slots of 64 columns
+      auto loadA = [&](uint32_t slot) {
 #pragma unroll
-      for (int q = 0; q < 4; q++) loadToLds(rA, __builtin_amdgcn_readfirstlane(w.m0A + q * 1024), w.a[q]);
-#pragma unroll
-      for (int c = 0; c < 2; c++)
-#pragma unroll
-        for (int q = 0; q < C::B_LOADS; q++)
-          loadToLds(rB, __builtin_amdgcn_readfirstlane(w.m0B + c * C::B_STAGE + q * 1024), w.b[q] == kOutOfRange ? kOutOfRange : w.b[q] + min((uint32_t)c, last) * w.dB);
-      pairLoop192(acc, w, min(1u, last) * 128, nk, last);
+        for (int q = 0; q < 4; q++) loadToLds(rA, __builtin_amdgcn_readfirstlane(w.m0A + slot * C::A_STAGE + q * 1024), w.a[q] + min(slot * 128, lastSlot));
+      };
+      auto loadB = [&](uint32_t c) {
+        const uint32_t off = min(c, chunks - 1) * w.dB;
+        loadToLds(rB, __builtin_amdgcn_readfirstlane(w.m0B + c * B_STAGE32), w.b[0] == kOutOfRange ? kOutOfRange : w.b[0] + off);
+        loadToLdsLowerHalf(rB, __builtin_amdgcn_readfirstlane(w.m0B + c * B_STAGE32 + 1024), w.b[1] == kOutOfRange ? kOutOfRange : w.b[1] + off);
+      };
+      // what the loop finds under way: A slots 0 and 1, chunks 0 to 2 of B, in the order its own loads keep
+      loadA(0); loadB(0); loadB(1); loadA(1); loadB(2);
+      pairLoop192(acc, w, min(3u, chunks - 1) * 64, chunks, lastSlot);
     } else if constexpr (C::PIPE) {
       waitVmcnt<(C::STAGES - 2) * C::LOADS>();     // chunk 0
       __builtin_amdgcn_s_barrier();

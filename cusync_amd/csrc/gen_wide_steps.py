@@ -223,16 +223,18 @@ def loop():
 TAIL = ["s_nop 7", "s_nop 4"]        # the last MFMAs' results are not the compiler's to touch before they are written
 
 # ---------------------------------------------------------------------------------------------------------------
-# The 256x192 tile with both operands 64 columns of K at a time (DmaCfg<256, 192, 64, 4, 2, ...>): eight wavefronts of
-# 64x96 (96 accumulator registers), so there is room for two sets of fragments: the reads of a k-step's fragments go
-# out between the MFMAs of the k-step before.  LDS: [A slot 0..1: 256 rows x 128 B][B slot 0..2: 64 k rows x 384 B].
-# One barrier per slot (four k-steps): barrier x, passed when slot x of both operands has landed for everyone, sits in
-# front of the last k-step of slot x-1, whose reads are the first of slot x; behind it everyone issues A slot x+1 (four
-# loads, into the A slot that slot x-1 has just left) and B slot x+2 (three loads).
+# The 256x192 tile in whole cache lines (DmaCfg<256, 192, 64, 4, 2, ...>): eight wavefronts of 64x96 (96 accumulator
+# registers), so there is room for two sets of fragments: the reads of a k-step's fragments go out between the MFMAs
+# of the k-step before.  LDS: [A slot 0..2: 256 rows x 128 B = 64 columns of K][B stage 0..3: 32 k rows x 384 B].
+# A chunk is 32 columns of K (two k-steps); barrier x, passed when chunk x of B and, x even, A slot x/2 have landed
+# for everyone, sits in front of the second k-step of chunk x-1, whose reads are the first of chunk x; behind it
+# everyone issues chunk x+3 of B (two loads: 1 KiB and, lower half of the wavefront only, 512 bytes) and, x even,
+# A slot x/2+2 (four loads).  Loads therefore have three chunks (B) and four (A) to land in, more than the latency
+# of a miss; with two A slots they had two, and every slot waited for its slowest line.
 F2 = 200                                       # fragment sets: set s at F2 + 20 s: A0, A1 (four registers each), B0..B2
 TMP2 = 240
-A_SLOT2, B_SLOT2 = 256 * 128, 64 * 384
-PERIOD2 = 6
+A_SLOT2, B_STAGE2, B_BASE2 = 256 * 128, 32 * 384, 3 * 256 * 128
+PERIOD2 = 12
 
 
 def fa2(s, i):
@@ -243,98 +245,114 @@ def fb2(s, j):
     return F2 + 20 * s + 8 + 4 * j
 
 
-def frag_reads2(x, kp, s):
-    """Reads of k-step kp (0..3) of slot x into fragment set s: list of (ins, ...) groups, one group per fragment."""
-    aslot, bslot = x % 2, x % 3
+def frag_reads2(c, kk, s):
+    """Reads of k-step kk of chunk c into fragment set s: one group of instructions per fragment (A0, A1, B0, B1, B2)."""
+    aslot, bstage, kp = (c // 2) % 3, c % 4, 2 * (c % 2) + kk
     groups = []
     pre = []
-    a_addr = "%[vA]"
+    a_addr, a_off = "%[vA]", aslot * A_SLOT2
+    if a_off + 4096 > 65535:                     # beyond the instruction's 16-bit offset: through a register
+        pre.append("v_add_u32 v%d, %d, %%[vA]" % (TMP2, a_off))
+        a_addr, a_off = "v%d" % TMP2, 0
     if kp:
-        pre = ["v_xor_b32 v%d, %d, %%[vA]" % (TMP2, 32 * kp)]
+        pre.append("v_xor_b32 v%d, %d, %s" % (TMP2, 32 * kp, a_addr))
         a_addr = "v%d" % TMP2
     for i in range(2):
-        groups.append((pre if i == 0 else []) + ["ds_read_b128 %s, %s offset:%d" % (v(fa2(s, i), 4), a_addr, aslot * A_SLOT2 + i * 4096)])
+        groups.append((pre if i == 0 else []) + ["ds_read_b128 %s, %s offset:%d" % (v(fa2(s, i), 4), a_addr, a_off + i * 4096)])
     for j in range(3):
-        off = bslot * B_SLOT2 + kp * 16 * 384
-        addr = "%%[vB%d]" % j
-        pre = []
-        if off + 4 * 384 > 65535:              # beyond the instruction's 16-bit offset: through a register
-            pre = ["v_add_u32 v%d, %d, %%[vB%d]" % (TMP2 + 1, bslot * B_SLOT2, j)]
-            addr, off = "v%d" % (TMP2 + 1), kp * 16 * 384
-        groups.append(pre + ["ds_read_b64_tr_b16 %s, %s offset:%d" % (v(fb2(s, j), 2), addr, off),
-                             "ds_read_b64_tr_b16 %s, %s offset:%d" % (v(fb2(s, j) + 2, 2), addr, off + 4 * 384)])
+        off = bstage * B_STAGE2 + kk * 16 * 384
+        groups.append(["ds_read_b64_tr_b16 %s, %%[vB%d] offset:%d" % (v(fb2(s, j), 2), j, off),
+                       "ds_read_b64_tr_b16 %s, %%[vB%d] offset:%d" % (v(fb2(s, j) + 2, 2), j, off + 4 * 384)])
     return groups
 
 
 def batch2(x):
-    """Direct loads behind barrier x: A slot x+1, B slot x+2."""
+    """Direct loads behind barrier x: chunk x+3 of B and, x even, A slot x/2+2.  soffA is 64 bytes x the B chunk."""
     out = []
-    for q in range(4):
-        pre = ["s_lshr_b32 vcc_hi, %[soffA], 7", "s_add_u32 vcc_hi, vcc_hi, 1", "s_min_u32 vcc_hi, vcc_hi, %[last]",
-               "s_mul_i32 vcc_hi, vcc_hi, %[dB]"] if q == 0 else []
-        out.append(pre + ["s_add_u32 m0, %%[m0A], %d" % (((x + 1) % 2) * A_SLOT2 + q * 1024),
-                          "buffer_load_dwordx4 %%[a%d], %%[rA], %%[soffA] offen lds" % q])
-    for q in range(3):
-        out.append(["s_add_u32 m0, %%[m0B], %d" % (((x + 2) % 3) * B_SLOT2 + q * 1024),
-                    "buffer_load_dwordx4 %%[b%d], %%[rB], vcc_hi offen lds" % q])
+    if x % 2 == 0:
+        slot = (x // 2 + 2) % 3
+        for q in range(4):
+            pre = ["s_add_u32 vcc_lo, %[soffA], 64", "s_and_b32 vcc_lo, vcc_lo, 0xffffff80", "s_min_u32 vcc_lo, vcc_lo, %[last]"] if q == 0 else []
+            out.append(pre + ["s_add_u32 m0, %%[m0A], %d" % (slot * A_SLOT2 + q * 1024),
+                              "buffer_load_dwordx4 %%[a%d], %%[rA], vcc_lo offen lds" % q])
+    stage = (x + 3) % 4
+    out.append(["s_lshr_b32 vcc_hi, %[soffA], 6", "s_mul_i32 vcc_hi, vcc_hi, %[dB]",
+                "s_add_u32 m0, %%[m0B], %d" % (stage * B_STAGE2),
+                "buffer_load_dwordx4 %[b0], %[rB], vcc_hi offen lds"])
+    out.append(["s_add_u32 m0, %%[m0B], %d" % (stage * B_STAGE2 + 1024),
+                "s_mov_b64 exec, 0xffffffff",
+                "buffer_load_dwordx4 %[b1], %[rB], vcc_hi offen lds",
+                "s_mov_b64 exec, -1"])
     return out
 
 
-def kstep2(out, x, kp):
-    """Six MFMAs of k-step kp of slot x on fragment set kp % 2; the reads of the next k-step go out between them, and
-    in front of the last k-step of a slot sits barrier x+1 with its loads behind."""
-    s = kp % 2
-    nx, nkp = (x, kp + 1) if kp < 3 else (x + 1, 0)
-    reads = [] if "noread" in OPTS else frag_reads2(nx % PERIOD2, nkp, 1 - s)
-    loads = batch2((x + 1) % PERIOD2) if kp == 3 else []
-    out.append("s_waitcnt lgkmcnt(0)")                       # this k-step's fragments (read a k-step ago)
-    if kp == 3:
-        out += ["s_waitcnt vmcnt(3)", "s_barrier"]           # slot x+1 has landed for everyone; slot x's last reads are done
+def kstep2(w, c, kk):
+    """Six MFMAs of k-step kk of chunk c on fragment set kk; the reads of the next k-step go out between them, and
+    in front of a chunk's second k-step sits barrier c+1 with its loads behind."""
+    s = kk
+    nc, nkk = (c, 1) if kk == 0 else (c + 1, 0)
+    reads = [] if "noread" in OPTS else frag_reads2(nc % PERIOD2, nkk, 1 - s)
+    names = ["A0", "A1", "B0", "B1", "B2"]
+    now = []
+    if kk == 1:
+        w.drain()                                            # chunk c's last reads (this k-step's fragments) are done
+        w.emit("s_waitcnt vmcnt(8)", "s_barrier")            # chunk c+1 has landed for everyone
+        now = batch2((c + 1) % PERIOD2)
     n = 0
     for j in range(3):
         for i in range(2):
+            w.need("%s.A%d" % (s, i))
+            w.need("%s.B%d" % (s, j))
             if "nomfma" not in OPTS:
-                out.append("v_mfma_f32_32x32x16_f16 %%[c%d%d], %s, %s, %%[c%d%d]" % (i, j, v(fb2(s, j), 4), v(fa2(s, i), 4), i, j))
+                w.emit("v_mfma_f32_32x32x16_f16 %%[c%d%d], %s, %s, %%[c%d%d]" % (i, j, v(fb2(s, j), 4), v(fa2(s, i), 4), i, j))
             if n < len(reads):
-                out += reads[n]
-            if loads:
-                out += loads[n]
-                if n == 5:
-                    out += loads[6]
+                for ins in reads[n]:
+                    if ins.startswith("ds_read"):
+                        w.read("%s.%s" % (1 - s, names[n]), ins)
+                    else:
+                        w.emit(ins)
+            if n < len(now):
+                w.emit(*now[n])
             n += 1
-    # (five fragment reads on six MFMAs)
 
 
 def loop192():
-    out = ["s_waitcnt vmcnt(3)", "s_barrier"]                # barrier 0: slot 0 of both operands
+    w = Wave()
+    w.emit("s_waitcnt vmcnt(8)", "s_barrier")                # barrier 0: chunk 0 of B, A slot 0
     for load in batch2(0):
-        out += load
-    out += ["s_cmp_gt_u32 %[left], 2", "s_cselect_b32 vcc_lo, 128, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo"]
-    for g in ([] if "noread" in OPTS else frag_reads2(0, 0, 0)):
-        out += g
-    out.append("LOOP_%=:")
-    for x in range(PERIOD2):
-        for kp in range(4):
-            kstep2(out, x, kp)
-        # behind the loads of barrier x+1 (A slot x+2, B slot x+3): on while there is another slot
-        out += ["s_cmp_gt_u32 %[left], 3", "s_cselect_b32 vcc_lo, 128, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo",
-                "s_sub_u32 %[left], %[left], 1", "s_cmp_eq_u32 %[left], 0",
-                "s_cbranch_scc1 DONE_%=" if x < PERIOD2 - 1 else "s_cbranch_scc0 LOOP_%="]
-    out += ["DONE_%=:", "s_waitcnt lgkmcnt(0)"]
-    return out + TAIL
+        w.emit(*load)
+    w.emit("s_cmp_gt_u32 %[left], 4", "s_cselect_b32 vcc_lo, 64, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo")
+    if "noread" not in OPTS:
+        for name, g in zip(["A0", "A1", "B0", "B1", "B2"], frag_reads2(0, 0, 0)):
+            for ins in g:
+                w.read("0." + name, ins)
+    w.emit("LOOP_%=:")
+    entry = list(w.pending)
+    for c in range(PERIOD2):
+        kstep2(w, c, 0)
+        kstep2(w, c, 1)
+        # behind the loads of barrier c+1 (chunk c+4 of B): on while there is another chunk
+        w.emit("s_cmp_gt_u32 %[left], 5", "s_cselect_b32 vcc_lo, 64, 0", "s_add_u32 %[soffA], %[soffA], vcc_lo")
+        w.emit("s_sub_u32 %[left], %[left], 1", "s_cmp_eq_u32 %[left], 0",
+               "s_cbranch_scc1 DONE_%=" if c < PERIOD2 - 1 else "s_cbranch_scc0 LOOP_%=")
+    assert w.pending == entry, (w.pending, entry)
+    w.emit("DONE_%=:", "s_waitcnt lgkmcnt(0)")
+    return w.out + TAIL
 
 
-CLOBBERS2 = ", ".join('"v%d"' % r for r in range(F2, TMP2 + 2)) + ', "vcc", "scc", "memory"'
+STATE_OPS = '[soffA] "+s"(soffA), [left] "+s"(left)'
+CLOBBERS2 = ", ".join('"v%d"' % r for r in range(F2, TMP2 + 1)) + ', "vcc", "scc", "memory"'
 ACC_OPS2 = ", ".join('[c%d%d] "+v"(acc[%d][%d])' % (i, j, i, j) for i in range(2) for j in range(3))
 IN_OPS2 = ('[vA] "v"(w.vA), [vB0] "v"(w.vB[0]), [vB1] "v"(w.vB[1]), [vB2] "v"(w.vB[2]), '
-           '[a0] "v"(w.a[0]), [a1] "v"(w.a[1]), [a2] "v"(w.a[2]), [a3] "v"(w.a[3]), [b0] "v"(w.b[0]), [b1] "v"(w.b[1]), [b2] "v"(w.b[2]), '
+           '[a0] "v"(w.a[0]), [a1] "v"(w.a[1]), [a2] "v"(w.a[2]), [a3] "v"(w.a[3]), [b0] "v"(w.b[0]), [b1] "v"(w.b[1]), '
            '[rA] "s"(w.rA), [rB] "s"(w.rB), [m0A] "s"(w.m0A), [m0B] "s"(w.m0B), [dB] "s"(w.dB), [last] "s"(last)')
 
 
 def function192(name, body):
     text = "\\n\\t".join(body)
-    lines = ["// soffA: 128 bytes x the A slot whose loads go out next (A slot 0 and B slots 0 and 1 are the caller's; the B slot that",
-             "// goes out with it is the one after, held at `last`, the last slot there is); left: slots to compute.",
+    lines = ["// soffA: 64 bytes x the chunk (32 columns of K) of B whose loads go out next (A slots 0 and 1 and chunks 0 to 2 of B are the",
+             "// caller's); the A slot that goes out with every second one begins one chunk later, held at `last`, the byte offset of the",
+             "// last slot there is; left: chunks to compute.",
              "__device__ __forceinline__ void %s(floatx16 (&acc)[2][3], const WideOperands& w, uint32_t soffA, uint32_t left, uint32_t last) {" % name,
              '  asm volatile("%s"' % text,
              "               : %s, %s" % (ACC_OPS2, STATE_OPS),
@@ -346,7 +364,6 @@ def function192(name, body):
 
 CLOBBERS = ", ".join('"v%d"' % r for r in range(T, TMP + 1)) + ', "vcc", "scc", "memory"'
 ACC_OPS = ", ".join('[c%d%d] "+v"(acc[%d][%d])' % (i, j, i, j) for i in range(4) for j in range(3))
-STATE_OPS = '[soffA] "+s"(soffA), [left] "+s"(left)'
 IN_OPS = ('[vA] "v"(w.vA), [vB0] "v"(w.vB[0]), [vB1] "v"(w.vB[1]), [vB2] "v"(w.vB[2]), '
           '[a0] "v"(w.a[0]), [a1] "v"(w.a[1]), [a2] "v"(w.a[2]), [a3] "v"(w.a[3]), [b0] "v"(w.b[0]), [b1] "v"(w.b[1]), [b2] "v"(w.b[2]), '
           '[rA] "s"(w.rA), [rB] "s"(w.rB), [m0A] "s"(w.m0A), [m0B] "s"(w.m0B), [dB] "s"(w.dB)')
