@@ -188,6 +188,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
   p.stage.d = s;
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->qkv % 128 == 0 && (a->ldqkv * 2) % 128 == 0 &&
                         (s.in.kind != CUSYNC_POLICY_TILESYNC || (s.in.tileN * 2) % 128 == 0);
+  p.stage.releaseAll = cusync::rt::forceRelease();
   p.S = a->seq; p.heads = a->heads; p.cached = a->cached_rows;
   p.qkv = (const half_t*)a->qkv; p.ldq = a->ldqkv;
   p.out = (half_t*)a->out; p.ldo = a->ldo;

@@ -394,9 +394,9 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
       __syncthreads();
       uint32_t* counter = p.arrivals + head * stage.d.grid.y + t.y;
       if (tid == 0) {
-        const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // the shares were written through and are acknowledged
+        const uint32_t before = stage.countIn(counter);      // relaxed: the shares were written through and are acknowledged
         const bool last = before == splits - 1;
-        if (last) cusync::dev::storeRelaxed(counter, 0);
+        if (last) { cusync::dev::storeRelaxed(counter, 0); stage.countSeen(); }
         sLast = last;
       }
       __syncthreads();
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
     cusync_dim3 done = {q0, head * kHD, 0};
-    if (completed && stage.isProducer()) stage.post(done, 1, true);
+    if (completed && stage.isProducer()) stage.post(done, 1, stage.storesThrough());
     else __syncthreads();
     if (tid == 0) recordTileAt(p.timeline, p.timelineCap, stage, p.launched, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }

@@ -129,6 +129,7 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
                         (a->C * 2) % 128 == 0 &&
                         (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
+  p.stage.releaseAll = cusync::rt::forceRelease();
   p.stage.prepare(launched);
   return p;
 }

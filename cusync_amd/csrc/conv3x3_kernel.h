@@ -211,7 +211,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
     const bool completed = finishTile<C, false>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, 0};
-    if (completed && stage.isProducer()) stage.post(done, 1, true);
+    if (completed && stage.isProducer()) stage.post(done, 1, stage.storesThrough());
     else __syncthreads();
     if (tid == 0) recordTile(p, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }

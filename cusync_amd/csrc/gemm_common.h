@@ -194,7 +194,7 @@ struct TileStore {
   static constexpr uint32_t kAllRows = (1u << C::WM) - 1;
 
   __device__ __forceinline__ TileStore(const GemmParams& p_, const cusync_dim3& t, int wm_, int wn_, int lane_, char* lds_)
-      : p(p_), lds(lds_), m0(t.y * C::BM), n0(t.x * C::BN), wm(wm_), wn(wn_), lane(lane_), through(p_.stage.isProducer()),
+      : p(p_), lds(lds_), m0(t.y * C::BM), n0(t.x * C::BN), wm(wm_), wn(wn_), lane(lane_), through(p_.stage.storesThrough()),
         rD(makeRsrc(p_.D, p_.M * p_.ldd * 2)) {}
 
   template<class V>
@@ -370,8 +370,9 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
     uint32_t* departures = p.arrivals + p.stage.d.grid.x * p.stage.d.grid.y + tileIndex;
     if (threadIdx.x == 0) {
       // not a release: the partial sums were written through and every wavefront has seen its own acknowledged
-      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      p.stage.countIn(counter);
       if (!dev::pollUntilAtLeast(counter, p.splitK)) dev::countGiveUp(p.stage.d.spinTimeouts);     // the siblings are resident: bounded all the same
+      p.stage.countSeen();
     }
     __syncthreads();
     // not unrolled: the sums do not live in the accumulators, so one copy of the pass serves every i
@@ -422,7 +423,7 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
       // A producer's stores must be out before the count that lets the last slice post: they were written through
       // and are acknowledged (the wait above), so the count needs no release, which would only start a write-back of
       // this XCD's L2.  No acquire either: nobody reads another slice's output.
-      const uint32_t before = __hip_atomic_fetch_add(departures, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t before = p.stage.countIn(departures);
       const bool last = before == p.splitK - 1;
       if (last) { dev::storeRelaxed(counter, 0); dev::storeRelaxed(departures, 0); }
       *sLast = last;
@@ -434,9 +435,9 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   if (threadIdx.x == 0) {
     // neither release (the partial sums were written through and are acknowledged) nor acquire (the finishing slice
     // reads them with device-coherent loads): either would work on this XCD's whole L2
-    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t before = p.stage.countIn(counter);
     const bool last = before == p.splitK - 1;
-    if (last) dev::storeRelaxed(counter, 0);
+    if (last) { dev::storeRelaxed(counter, 0); p.stage.countSeen(); }
     *sLast = last;
   }
   __syncthreads();

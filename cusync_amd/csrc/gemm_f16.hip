@@ -208,6 +208,7 @@ static GemmParams gemmParams(const cusync_gemm_args* a, const TileInfo* ti, uint
   const bool canRound = ti->chainKernel != nullptr && a->a_mode == CUSYNC_A_PLAIN;      // a direct-to-LDS tile
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->A % 128 == 0 &&
                         (a->lda * 2) % 128 == 0 && (wholeLineTiles || canRound);
+  p.stage.releaseAll = cusync::rt::forceRelease();
   p.waitRound = p.stage.lineAligned && !wholeLineTiles ? 64 : 1;
   p.stage.prepare(launched);
   p.M = a->M; p.N = a->N; p.K = a->K;

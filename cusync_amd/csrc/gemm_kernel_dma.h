@@ -625,7 +625,7 @@ __device__ __forceinline__ void gemmDmaTiles(const GemmParams& p) {
     // All waves must be past their last LDS read before the next tile's loads
     // land in stage 0; the post (or this barrier) provides that.
     cusync_dim3 done = {m0, outputColumn(p, n0), t.z};
-    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p), true);
+    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p), stage.storesThrough());
     else __syncthreads();
     if (tid == 0) recordTile(p, t, round, tlEntry, tl0, tl1, tl2, p.timeline ? wall_clock64() : 0);
   }

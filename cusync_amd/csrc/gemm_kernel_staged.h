@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kThreads) void gemmKernel(GemmParams p) {
     const bool completed = finishTile<C>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, outputColumn(p, n0), t.z};
     // the post's barrier (or this one) keeps the next tile's LDS writes behind the epilogue's LDS reads
-    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p), true);
+    if (completed && stage.isProducer()) stage.post(done, postsPerTile(p), stage.storesThrough());
     else __syncthreads();
   }
 }

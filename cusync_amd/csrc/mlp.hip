@@ -150,6 +150,7 @@ cusync_error runActStage(const cusync_mlp* m, const void* h, void* stream) {
   const cusync_stage_desc& s = m->mid;
   ActParams p = {};
   p.stage.d = s;
+  p.stage.releaseAll = cusync::rt::forceRelease();
   p.stage.lineAligned = false;       // every wait is followed by an L2 invalidation: tiles of 128 columns of a 2d-wide matrix are not whole lines for every d
   p.M = m->cfg.batch; p.d = m->cfg.inner;
   p.G = (const half_t*)h; p.ldg = m->ldh;

@@ -44,6 +44,14 @@ bool forceAcquire() {
   return on;
 }
 
+bool forceRelease() {
+  static const bool on = [] {
+    const char* v = getenv("CUSYNC_FORCE_RELEASE");
+    return v && *v && strcmp(v, "0") != 0;
+  }();
+  return on;
+}
+
 bool forceWaitKernel() {
   static const bool on = [] {
     const char* v = getenv("CUSYNC_WAIT_KERNEL");

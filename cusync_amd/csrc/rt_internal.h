@@ -16,6 +16,11 @@ int check(hipError_t e, const char* what, const char* file, int line);
 // wait then ends with the agent-scope acquire (cache invalidation), also where the launcher found that the
 // producer's tiles are whole cache lines of the consumer's operand and the invalidation can be skipped.
 bool forceAcquire();
+// True when CUSYNC_FORCE_RELEASE is set to something other than 0: every post of the library's kernels and every
+// count their k-slices and key-range splits hand partial results over with is a device-scope release (the counts'
+// readers acquire), also where the data was written through and acknowledged and the count is normally relaxed.
+// With CUSYNC_FORCE_ACQUIRE this is the plain release/acquire protocol end to end; results must be the same.
+bool forceRelease();
 // True when CUSYNC_WAIT_KERNEL is set to something other than 0: the chain handles then hold every consumer back
 // with the wait kernel, also behind a producer whose launch takes every workgroup slot (where they would wait on
 // the host).  For measuring what the host-side hold is there to prevent.

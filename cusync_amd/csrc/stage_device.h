@@ -33,8 +33,25 @@ struct DynStage {
   // allStatic(launched) of the launch this object goes to, worked out by the launcher (set by prepare()): in the
   // kernel it is a loop of eight rounds of integer divisions that every wavefront would run before its first load.
   bool noDraws;
+  // Diagnosis (set by the launcher from CUSYNC_FORCE_RELEASE): every post, and every count the k-slices and key-range
+  // splits hand partial results over with, is a release at device scope (and the counts' readers acquire), as the
+  // plain protocol has it, also where the stores were written through and acknowledged and the library normally
+  // raises them relaxed.  Results must not change; only the write-backs and invalidations come back.
+  bool releaseAll;
 
   __device__ __forceinline__ bool isProducer() const { return d.out.kind != CUSYNC_POLICY_NOSYNC; }
+  // Whether this stage's kernels write their output through to memory as they store it (sc1): a producer's do, so
+  // that the post finds nothing to write back.  The epilogues take their store policy from here and hand the same
+  // answer to post(): one flag decides both.
+  __device__ __forceinline__ bool storesThrough() const { return isProducer(); }
+  // A count that hands over data written through and acknowledged (k-slices, key-range splits): relaxed, or a
+  // release under releaseAll.
+  __device__ __forceinline__ uint32_t countIn(uint32_t* counter) const {
+    return releaseAll ? __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT)
+                      : __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // ... and what its reader does before it touches the data (nothing: it reads with device-coherent loads).
+  __device__ __forceinline__ void countSeen() const { if (releaseAll) dev::acquireFence(); }
   __device__ __forceinline__ bool isConsumer() const { return d.in.kind != CUSYNC_POLICY_NOSYNC; }
   __device__ __forceinline__ uint32_t numTiles() const { return d.grid.x * d.grid.y * d.grid.z; }
   __host__ __device__ __forceinline__ bool customOrder() const { return !(d.opts & CUSYNC_OPT_AVOID_CUSTOM_ORDER); }
@@ -331,7 +348,7 @@ struct DynStage {
     if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
       const uint32_t idx = dyn::tileIndex(d.out, tile, d.grid) * CUSYNC_SEM_STRIDE;
       const uint32_t v = dyn::postValue(d.out) * times;
-      if (writtenThrough) {
+      if (writtenThrough && !releaseAll) {
         if (d.opts & CUSYNC_OPT_NO_ATOMIC_ADD) dev::storeRelaxed(&d.tileStatusWrite[idx], v * (uint32_t)d.iter);
         else __hip_atomic_fetch_add((uint32_t*)&d.tileStatusWrite[idx], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
