@@ -22,6 +22,7 @@ import argparse
 import json
 import os
 import statistics
+import subprocess
 import sys
 import time
 
@@ -272,8 +273,23 @@ def main():
         return
 
     per_batch = []
+    launcher = {}
     if not args.no_sweep:
         settle(max(BATCHES))
+        # The reference's own loop (CuStage + CuSyncGemm objects wired by a plain C++ driver, invokeWaitKernel between the
+        # two launches) next to the handle: the driver runs rounds of 20 steps of each in turn, in a process of its own
+        # while this one is idle, and reports medians.
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cusync_amd", "bin", "mlp_stages")
+        if not os.path.exists(exe):
+            sys.exit("bench.py: %s is not built (make -C cusync_amd/drivers)" % exe)
+        drv = subprocess.run([exe, "--batch", ",".join(str(b) for b in BATCHES), "--sync", "both", "--runs", "20", "--rounds", "3"],
+                             capture_output=True, text=True, timeout=600)
+        if drv.returncode != 0:
+            sys.exit("bench.py: mlp_stages failed: " + drv.stderr[-2000:])
+        for line in drv.stdout.splitlines():
+            if line.startswith('{"batch"'):
+                r = json.loads(line)
+                launcher[(r["batch"], r["sync"])] = r
         for b in BATCHES:
             # all modes of this batch size alive together, one step each per round (10 untimed rounds, 20 timed):
             # stream-ordered, RowSync, TileSync, RowSync with both GEMMs in one launch (same stages and semaphores,
@@ -316,6 +332,10 @@ def main():
                 "rowsync_one_launch_us": round(m["rowsync_one_launch"][0], 2) if "rowsync_one_launch" in m else None,
                 "tilesync_one_launch_us": round(m["tilesync_one_launch"][0], 2) if "tilesync_one_launch" in m else None,
                 "one_launch_tiles": one_tiles,
+                # medians of 60 steps in the driver's process: the launcher objects' loop, and the handle beside it there
+                "launcher_rowsync_us": launcher[(b, "rowsync")]["launcher_us"], "launcher_tilesync_us": launcher[(b, "tilesync")]["launcher_us"],
+                "launcher_vs_handle_pct": {k: round(launcher[(b, k)]["launcher_us"] / launcher[(b, k)]["handle_us"] * 100 - 100, 2)
+                                           for k in ("rowsync", "tilesync")},
                 "best_policy": min(in_place, key=lambda k: m[k][0]),
                 "best_gain_pct": round(100 - best / s_us * 100, 2),
                 "repacked_weights": {"stream_us": round(m["stream_rp"][0], 2), "rowsync_us": round(m["rowsync_rp"][0], 2),

@@ -100,6 +100,7 @@ SIGNATURES = {
     "cusync_invoke_wait_kernel": (C.c_int, [C.POINTER(StageDesc), vp]),
     "cusync_invoke_wait_kernel_after": (C.c_int, [C.POINTER(StageDesc), vp, vp]),
     "cusync_wait_producer_started": (C.c_int, [C.POINTER(StageDesc), u32]),
+    "cusync_hold_back": (C.c_int, [C.POINTER(StageDesc), vp]),
     "cusync_wait_kernel": (C.c_int, [vp, u32, vp]),
     "cusync_stage_read_state": (C.c_int, [C.POINTER(StageDesc), vp, vp, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_policy_tile_index": (u32, [C.POINTER(PolicyDesc), Dim3, Dim3]),
@@ -150,6 +151,7 @@ SIGNATURES = {
     "cusync_mlp_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
     "cusync_mlp_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cusync_mlp_splits": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "cusync_mlp_choice": (C.c_int, [C.POINTER(MlpConfig), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
 }
 
 _lib = None

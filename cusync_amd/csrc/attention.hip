@@ -218,6 +218,7 @@ cusync_error cusync_attention_run(const cusync_attention_args* a, void* stream) 
     lds = std::max(lds, g_attnLdsPerCU / 2);
   hipLaunchKernelGGL(attnKernel(deep), dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  cusync::rt::noteLaunch(s, launched >= (uint32_t)resident);
   return CUSYNC_SUCCESS;
 }
 
@@ -395,15 +396,12 @@ cusync_error cusync_attn_layer_run(cusync_attn_layer* L, const void* x, void* qk
     if (CUSYNC_HIP(hipEventRecord(L->eStart, s0))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_gemm_run(&a1, s0)) != CUSYNC_SUCCESS) return e;
     // overlapped: each consumer's stream is held back until every workgroup of its producer has started: from the
-    // host when the producer's launch takes every workgroup slot of the device (a wait kernel's wave would keep its
+    // host when the producer's launch took every workgroup slot of the device (a wait kernel's wave would keep its
     // last workgroup off the device), by the wait kernel otherwise.  eMid1 / eMid2 only serve the stage timing.
-    if (overlapped) {
-      const bool fills = cusync_gemm_fills_device(&a1) != 0 && !cusync::rt::forceWaitKernel();
-      if ((e = fills ? cusync_wait_producer_started(&L->st[0], 0) : cusync_invoke_wait_kernel(&L->st[0], s1)) != CUSYNC_SUCCESS) return e;
-    }
+    if (overlapped && (e = cusync_hold_back(&L->st[0], s1)) != CUSYNC_SUCCESS) return e;
     if (CUSYNC_HIP(hipEventRecord(L->eMid1, s1))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_attention_run(&a2, s1)) != CUSYNC_SUCCESS) return e;
-    if (overlapped) { if ((e = cusync_invoke_wait_kernel(&L->st[1], s2)) != CUSYNC_SUCCESS) return e; }
+    if (overlapped) { if ((e = cusync_hold_back(&L->st[1], s2)) != CUSYNC_SUCCESS) return e; }
     else if (CUSYNC_HIP(hipEventRecord(L->eMid2, s0))) return CUSYNC_ERROR_DEVICE;
     if ((e = cusync_gemm_run(&a3, s2)) != CUSYNC_SUCCESS) return e;
     if (CUSYNC_HIP(hipEventRecord(L->eEnd, s2))) return CUSYNC_ERROR_DEVICE;

@@ -221,6 +221,7 @@ cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   GemmParams p = convParams(a, ti, launched);
   hipLaunchKernelGGL(ti->kernel, dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  cusync::rt::noteLaunch(a->stage, launched >= (uint32_t)resident);
   return CUSYNC_SUCCESS;
 }
 
@@ -397,10 +398,10 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
       hipStream_t s = c->stream[overlapped ? i : 0];
       const cusync_conv2d_args a = layerArgs(i);
       cusync_error e;
-      // overlapped: the reference's wait kernel holds layer i's stream back until layer i - 1 is on the device.  A
-      // layer's launch leaves workgroup slots free (392 tiles on 512 slots for the benchmark shapes; any launch of
-      // fewer workgroups than stay resident), so the wait kernel's wave takes nothing from the producer.
-      if (overlapped && i > 0 && (e = cusync_invoke_wait_kernel(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
+      // overlapped: layer i's stream is held back until layer i - 1 is on the device: by the reference's wait kernel
+      // where that layer's launch left workgroup slots free (392 tiles on 512 slots for the benchmark shapes), so
+      // that the wait kernel's wave takes nothing from the producer; from this thread where the launch took them all.
+      if (overlapped && i > 0 && (e = cusync_hold_back(&c->st[i - 1], s)) != CUSYNC_SUCCESS) return e;
       if ((e = cusync_conv2d_run(&a, s)) != CUSYNC_SUCCESS) return e;
       if ((!overlapped || i + 1 == n) && CUSYNC_HIP(hipEventRecord(c->ev[i + 1], s))) return CUSYNC_ERROR_DEVICE;
     }

@@ -344,6 +344,7 @@ cusync_error cusync_gemm_run(const cusync_gemm_args* a, void* stream) {
     lds = std::max<size_t>(lds, g_ldsPerCU / 2);
   hipLaunchKernelGGL(kernel, dim3(launched), dim3(ti->threads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
+  cusync::rt::noteLaunch(s, launched >= (uint32_t)resident);
   return CUSYNC_SUCCESS;
 }
 

@@ -296,6 +296,34 @@ void discard(cusync_mlp* m) {
   setError(why);
 }
 
+// What a handle for `c` runs with: where the activation is computed, the sync mode after the StridedSync
+// substitution, tiles and k-slices.  False (with the error text set) for a configuration no handle can be made of.
+struct Choice { bool fused, actStage; int aMode2, sync, tile1, tile2, split1, split2; };
+bool choose(const cusync_mlp_config& c, Choice* o) {
+  const bool llama = c.model == CUSYNC_MLP_LLAMA;
+  const uint32_t k1 = c.hidden, n1 = llama ? 2 * c.inner : c.inner, k2 = c.inner, n2 = c.hidden;
+  const bool swiglu = llama && c.activation;
+  // where silu(gate) * up is computed: 2 = GEMM1's epilogue (the built-in choice), -1 = a stage of its own, 1 = GEMM2's A loader
+  const int where = !swiglu ? 0 : c.swiglu_in_gemm2 == 0 ? 2 : c.swiglu_in_gemm2;
+  if (swiglu && where != 2 && where != -1 && where != 1) { setError("mlp: swiglu_in_gemm2 must be -1, 0, 1 or 2"); return false; }
+  o->fused = swiglu && where == 2;
+  o->actStage = swiglu && where == -1;
+  o->aMode2 = (swiglu && where == 1) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  o->sync = c.sync;
+  if (swiglu && !o->fused && o->sync == CUSYNC_SYNC_TILE && c.inner % 128 == 0) o->sync = CUSYNC_SYNC_STRIDED;
+  pickTiles(c, o->sync, o->aMode2 == CUSYNC_A_SWIGLU, o->fused, &o->tile1, &o->tile2);
+  uint32_t bk1 = 0, bk2 = 0;
+  if (cusync_gemm_tile_shape(o->tile1, nullptr, nullptr, &bk1) || cusync_gemm_tile_shape(o->tile2, nullptr, nullptr, &bk2)) {
+    setError("mlp: unknown tile id");
+    return false;
+  }
+  const cusync_dim3 flat1 = cusync_gemm_grid(o->tile1, c.batch, n1, 1);
+  const cusync_dim3 flat2 = cusync_gemm_grid(o->tile2, c.batch, n2, 1);
+  o->split1 = pickSplit(c.split_k1, flat1.x * flat1.y, k1, bk1, cusync_gemm_max_resident(o->tile1));
+  o->split2 = pickSplit(c.split_k2, flat2.x * flat2.y, k2, bk2, cusync_gemm_max_resident(o->tile2));
+  return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -315,12 +343,11 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->w1p = m->w2p = nullptr;
   m->ldw1 = m->n1; m->ldw2 = m->n2;
   const bool swiglu = llama && cfg->activation;
-  // where silu(gate) * up is computed: 2 = GEMM1's epilogue (the built-in choice), -1 = a stage of its own, 1 = GEMM2's A loader
-  const int where = !swiglu ? 0 : cfg->swiglu_in_gemm2 == 0 ? 2 : cfg->swiglu_in_gemm2;
-  if (swiglu && where != 2 && where != -1 && where != 1) { setError("mlp: swiglu_in_gemm2 must be -1, 0, 1 or 2"); discard(m); return nullptr; }
-  m->fused = swiglu && where == 2;
-  m->actStage = swiglu && where == -1;
-  m->aMode2 = (swiglu && where == 1) ? CUSYNC_A_SWIGLU : CUSYNC_A_PLAIN;
+  Choice ch;
+  if (!choose(*cfg, &ch)) { discard(m); return nullptr; }
+  m->fused = ch.fused;
+  m->actStage = ch.actStage;
+  m->aMode2 = ch.aMode2;
   m->epilogue1 = (!llama && cfg->activation) ? CUSYNC_EPILOGUE_GELU : m->fused ? CUSYNC_EPILOGUE_SWIGLU : CUSYNC_EPILOGUE_NONE;
   if (cfg->repack_weights) {
     // rows 256 bytes longer than the data: consecutive k rows of a column tile then fall into consecutive
@@ -348,26 +375,15 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->sMid = nullptr;
   memset(&m->mid, 0, sizeof m->mid);
 
-  int sync = cfg->sync;
-  if (swiglu && !m->fused && sync == CUSYNC_SYNC_TILE && cfg->inner % 128 == 0) sync = CUSYNC_SYNC_STRIDED;
-  pickTiles(*cfg, sync, m->aMode2 == CUSYNC_A_SWIGLU, m->fused, &m->tile1, &m->tile2);
+  const int sync = ch.sync;
+  m->tile1 = ch.tile1; m->tile2 = ch.tile2;
   uint32_t tm1 = 0, tn1 = 0;
-  if (cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr) || cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, nullptr)) {
-    setError("mlp: unknown tile id");
-    discard(m);
-    return nullptr;
-  }
+  cusync_gemm_tile_shape(m->tile1, &tm1, &tn1, nullptr);
 
   cusync_policy_desc pol = noSync();
   int opts = 0;
   const uint32_t tnOut = m->fused ? tn1 / 2 : tn1;      // width of a GEMM1 tile in columns of the intermediate
-  uint32_t bk1 = 0, bk2 = 0;
-  cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk1);
-  cusync_gemm_tile_shape(m->tile2, nullptr, nullptr, &bk2);
-  const cusync_dim3 flat1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, 1);
-  const cusync_dim3 flat2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, 1);
-  m->split1 = pickSplit(cfg->split_k1, flat1.x * flat1.y, m->k1, bk1, cusync_gemm_max_resident(m->tile1));
-  m->split2 = pickSplit(cfg->split_k2, flat2.x * flat2.y, m->k2, bk2, cusync_gemm_max_resident(m->tile2));
+  m->split1 = ch.split1; m->split2 = ch.split2;
   m->ws1 = m->ws2 = nullptr;
   const cusync_dim3 g1 = cusync_gemm_grid(m->tile1, cfg->batch, m->n1, m->split1);
   const cusync_dim3 g2 = cusync_gemm_grid(m->tile2, cfg->batch, m->n2, m->split2);
@@ -538,15 +554,11 @@ cusync_error cusync_mlp_run_split(cusync_mlp* m, const void* x, void* h, void* y
       // that takes every workgroup slot of the device is waited for here on the host (a wait kernel's wave on one
       // of the CUs would keep the last producer workgroup off the device until another retires); for any other
       // the reference's wait kernel goes into the consumer's stream, unordered like the reference's.
-      auto holdBack = [&](const cusync_stage_desc* prod, bool fills, hipStream_t s) {
-        return fills ? cusync_wait_producer_started(prod, 0) : cusync_invoke_wait_kernel(prod, s);
-      };
-      const bool fills1 = cusync_gemm_fills_device(&a1) != 0 && !cusync::rt::forceWaitKernel();
       if (m->actStage) {        // GEMM1 -> activation -> GEMM2, a stream and a hold-back per edge
-        if ((e = holdBack(&m->prod, fills1, m->sMid)) != CUSYNC_SUCCESS) return e;
+        if ((e = cusync_hold_back(&m->prod, m->sMid)) != CUSYNC_SUCCESS) return e;
         if ((e = runActStage(m, h, m->sMid)) != CUSYNC_SUCCESS) return e;
         if ((e = cusync_invoke_wait_kernel(&m->mid, m->sCons)) != CUSYNC_SUCCESS) return e;
-      } else if ((e = holdBack(&m->prod, fills1, m->sCons)) != CUSYNC_SUCCESS) {
+      } else if ((e = cusync_hold_back(&m->prod, m->sCons)) != CUSYNC_SUCCESS) {
         return e;
       }
       if ((e = cusync_gemm_run(&a2, m->sCons)) != CUSYNC_SUCCESS) return e;
@@ -598,6 +610,17 @@ int cusync_mlp_splits(const cusync_mlp* m, int* split_k1, int* split_k2) {
   if (!m) return 1;
   if (split_k1) *split_k1 = m->split1;
   if (split_k2) *split_k2 = m->split2;
+  return 0;
+}
+
+int cusync_mlp_choice(const cusync_mlp_config* cfg, int* tile1, int* tile2, int* split_k1, int* split_k2) {
+  if (!cfg || cfg->batch == 0 || cfg->hidden == 0 || cfg->inner == 0) { setError("mlp: empty shape"); return 1; }
+  Choice ch;
+  if (!choose(*cfg, &ch)) return 1;
+  if (tile1) *tile1 = ch.tile1;
+  if (tile2) *tile2 = ch.tile2;
+  if (split_k1) *split_k1 = ch.split1;
+  if (split_k2) *split_k2 = ch.split2;
   return 0;
 }
 

@@ -270,7 +270,9 @@ cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc* prod, void
   return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
-cusync_error cusync_wait_producer_started(const cusync_stage_desc* prod, uint32_t timeout_ms) {
+// Polls the host-memory mirror of the producer's flag.  *timedOut says whether a failure was the time limit.
+static cusync_error waitStartedOnHost(const cusync_stage_desc* prod, uint32_t timeout_ms, bool* timedOut) {
+  *timedOut = false;
   if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
   if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
   if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
@@ -279,12 +281,47 @@ cusync_error cusync_wait_producer_started(const cusync_stage_desc* prod, uint32_
   const uint32_t want = (uint32_t)prod->iter;
   for (uint32_t spins = 0;; spins++) {
     if (__atomic_load_n(prod->spinTimeouts + CUSYNC_HOST_FLAG_OFFSET, __ATOMIC_ACQUIRE) >= want) return CUSYNC_SUCCESS;
+    __builtin_ia32_pause();      // the flag arrives over the bus: leave the core's other thread and the memory pipeline alone meanwhile
     if ((spins & 1023u) == 1023u &&
         std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(timeout_ms ? timeout_ms : 2000)) {
       cusync::rt::setError("cusync_wait_producer_started: the producer's workgroups did not all start in time");
+      *timedOut = true;
       return CUSYNC_ERROR_DEVICE;
     }
   }
+}
+
+cusync_error cusync_wait_producer_started(const cusync_stage_desc* prod, uint32_t timeout_ms) {
+  bool timedOut;
+  return waitStartedOnHost(prod, timeout_ms, &timedOut);
+}
+
+extern "C++" { namespace cusync { namespace rt {
+void noteLaunch(const cusync_stage_desc& stage, bool fillsDevice) {
+  if (stage.out.kind == CUSYNC_POLICY_NOSYNC || !stage.spinTimeouts) return;
+  __atomic_store_n(stage.spinTimeouts + CUSYNC_HOST_FLAG_OFFSET + 1, fillsDevice ? (uint32_t)stage.iter : 0u, __ATOMIC_RELAXED);
+}
+}} }
+
+cusync_error cusync_hold_back(const cusync_stage_desc* prod, void* stream) {
+  if (!prod) return CUSYNC_ERROR_NOT_INITIALIZED;
+  if (prod->out.kind == CUSYNC_POLICY_NOSYNC) return CUSYNC_ERROR_NOT_PRODUCER;
+  if (prod->opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) return CUSYNC_SUCCESS;
+  if (!prod->kernelExecuted || !prod->spinTimeouts) return CUSYNC_ERROR_NOT_INITIALIZED;
+  const bool filled = __atomic_load_n(prod->spinTimeouts + CUSYNC_HOST_FLAG_OFFSET + 1, __ATOMIC_RELAXED) == (uint32_t)prod->iter;
+  if (filled && !cusync::rt::forceWaitKernel()) {
+    // a stream that is being captured has launched nothing yet: the flag would never rise while this thread waits
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (RT(hipStreamIsCapturing((hipStream_t)stream, &capturing))) return CUSYNC_ERROR_DEVICE;
+    if (capturing == hipStreamCaptureStatusNone) {
+      bool timedOut = false;
+      const cusync_error e = waitStartedOnHost(prod, 0, &timedOut);
+      if (e == CUSYNC_SUCCESS || !timedOut) return e;
+      // The producer is queued behind other work of the device, or its launch was refused: the wait kernel holds
+      // the consumer's stream back from here on, with its own bounded wait and its own count of waits that gave up.
+    }
+  }
+  return launchWaitKernel(prod->kernelExecuted, (uint32_t)prod->iter, prod->spinTimeouts, stream);
 }
 
 cusync_error cusync_stage_read_state(const cusync_stage_desc* d, uint32_t* sems, cusync_dim3* tile_order,

@@ -25,6 +25,10 @@ bool forceRelease();
 // with the wait kernel, also behind a producer whose launch takes every workgroup slot (where they would wait on
 // the host).  For measuring what the host-side hold is there to prevent.
 bool forceWaitKernel();
+// Called by a kernel launcher right after it launched a run of `stage`: records, in the stage's block of host memory,
+// whether that launch took every workgroup slot of the device.  cusync_hold_back reads it.  No-op for a stage that
+// posts nothing.
+void noteLaunch(const cusync_stage_desc& stage, bool fillsDevice);
 // Adds up the counters of waits that gave up (cusync_stage_desc::spinTimeouts) of the stages given; null
 // entries and stages without a counter are skipped.  Returns false if a copy from the device failed.
 bool spinTimeoutsOf(const cusync_stage_desc* const* stages, int count, uint32_t* sum);

@@ -154,7 +154,12 @@ public:
   dim3 grid() { return grid_; }
 
   // Holds `stream` back until the producer kernel of the current run is on the
-  // device (src/include/cusync/cusync.h:203-209).
+  // device (src/include/cusync/cusync.h:203-209).  For a run launched by one of
+  // the library's launchers (CuSyncGemm::run, ...) the library picks the way
+  // that suits that launch (cusync_hold_back): the reference's wait kernel, or,
+  // where the launch took every workgroup slot of the device and a wait kernel's
+  // wave would keep the producer's last workgroup off it, a wait on the calling
+  // thread.  A kernel of the caller's own always gets the wait kernel.
   // `launchEvent` (optional, not in the reference): a hipEvent_t recorded on the
   // producer's stream right before the producer's launch.  `stream` then waits
   // for it first, so that the wait kernel's wave cannot reach the device ahead of
@@ -163,11 +168,9 @@ public:
     if (!isProducer()) return CuSyncErrorNotProducer;
     if (getAvoidWaitKernel()) return CuSyncSuccess;
     if (kernelExecuted_ == nullptr) return CuSyncErrorNotInitialized;
-    if (launchEvent != nullptr) {
-      const cusync_stage_desc d = desc();
-      return (CuSyncError)cusync_invoke_wait_kernel_after(&d, stream, launchEvent);
-    }
-    return (CuSyncError)cusync_wait_kernel(kernelExecuted_, (uint32_t)iter, stream);
+    const cusync_stage_desc d = desc();
+    if (launchEvent != nullptr) return (CuSyncError)cusync_invoke_wait_kernel_after(&d, stream, launchEvent);
+    return (CuSyncError)cusync_hold_back(&d, stream);
   }
 
   void incrementIter() { iter += 1; }

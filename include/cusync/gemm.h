@@ -59,6 +59,33 @@ struct LinearCombinationParams {
   LinearCombinationParams(float a = 1.0f, float b = 0.0f) : alpha(a), beta(b) {}
 };
 
+// ThreadblockShape of a tile id at compile time, for the policies whose tile extents are template arguments
+// (RowSync<kM>, TileSync<Order, kM, kN>: mlp.cu:1026-1037 takes them from ShapeThreadBlock1).  The same numbers as
+// cusync_gemm_tile_shape() returns at run time.
+template<int TileId> struct GemmTileShape;
+#define CUSYNC_GEMM_TILE_SHAPE(ID, M, N, K) \
+  template<> struct GemmTileShape<ID> { static constexpr uint32_t kM = M, kN = N, kK = K; }
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x256x32, 256, 256, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x128x64, 256, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x128x64, 128, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_64x128x64, 64, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_32x128x64, 32, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x256x64, 128, 256, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x64x64, 256, 64, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x64x64, 128, 64, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x128x32, 256, 128, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x256x32, 128, 256, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x128x32, 128, 128, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x192x32, 128, 192, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x192x32, 256, 192, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_D32x128x64, 32, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_D64x128x64, 64, 128, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_D64x192x64, 64, 192, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x192x32_ALONE, 128, 192, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x384x32, 256, 384, 32);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x192x64, 256, 192, 64);
+#undef CUSYNC_GEMM_TILE_SHAPE
+
 // CuSyncGemm<CuStageImpl, TileId, Epilogue>: D = epilogue(A x B), fp16 row-major, fp32 accumulate.
 //   TileId    CUSYNC_TILE_*  (stands in for ThreadblockShape / WarpShape / Stages)
 //   Epilogue  CUSYNC_EPILOGUE_*  (LinearCombination, LinearCombinationGELU, LinearCombinationRelu, ...)
@@ -187,7 +214,9 @@ class CuSyncGemm {
     a.split_k = split_k;
     a.workspace = workspace;
     a.max_workgroups = max_workgroups;
-    a.shared_reduction = 0;
+    // k-slices add their partial sums up among themselves where the library finds that safe for this launch
+    // (cusync_gemm_args::shared_reduction); the reference's reduction is a kernel of its own, cusyncgemm.h:525-563
+    a.shared_reduction = 1;
     return a;
   }
 };

@@ -101,7 +101,8 @@ typedef struct cusync_stage_desc {
   uint32_t *spinTimeouts;     /* number of waits of this stage that gave up, 0 in a healthy chain.  Pinned host memory
                                  that the device writes to, so that the host reads it without a copy; the word
                                  CUSYNC_HOST_FLAG_OFFSET words behind it mirrors the wait-kernel flag for
-                                 cusync_wait_producer_started (written right after the flag itself) */
+                                 cusync_wait_producer_started (written right after the flag itself), and the word after
+                                 that is the launchers' note for cusync_hold_back (host-written only) */
   uint32_t *tileStatusWrite;  /* semaphores this stage posts, CUSYNC_SEM_STRIDE apart */
   uint32_t *tileStatusRead;   /* semaphores this stage waits on (its producer's) */
 } cusync_stage_desc;
@@ -181,6 +182,15 @@ cusync_error cusync_invoke_wait_kernel_after(const cusync_stage_desc *prod, void
  * CUSYNC_WAIT_KERNEL=1 in the environment they use the wait kernel everywhere, for comparison).  No counterpart
  * in the reference. */
 cusync_error cusync_wait_producer_started(const cusync_stage_desc *prod, uint32_t timeout_ms);
+/* CuStage::invokeWaitKernel as the library's own chains do it (CS/cusync.h:203-209): holds `stream` back until every
+ * workgroup of the producer's run prod->iter has started, by whichever of the two ways above suits the producer's last
+ * launch.  cusync_gemm_run, cusync_conv2d_run and cusync_attention_run leave a note in the stage's host memory saying
+ * whether the launch they just made took every workgroup slot of the device (cusync_gemm_fills_device); for such a
+ * launch the calling thread waits (cusync_wait_producer_started) and, should that time out (the producer is queued
+ * behind other work), the wait kernel is enqueued after all; for any other launch, for a stream under capture, or with
+ * CUSYNC_WAIT_KERNEL=1 in the environment, the wait kernel is enqueued at once.  Call it after the producer's launch
+ * call has returned and before the consumer's, as the reference's loop does (src/ml-bench/transformer/mlp.cu:691-699). */
+cusync_error cusync_hold_back(const cusync_stage_desc *prod, void *stream);
 /* cusync::invokeWaitKernel(sem, value, stream) (CS/wait-kernel.h:10). */
 cusync_error cusync_wait_kernel(uint32_t *semaphore, uint32_t value, void *stream);
 /* Reads back device state for tests (the reference reaches it through the
@@ -527,6 +537,11 @@ cusync_error cusync_mlp_run_split(cusync_mlp *mlp, const void *x, void *h, void 
 /* Device state of the two stages for tests (see cusync_stage_read_state). */
 const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer (GEMM1), 1 consumer (GEMM2), 2 the activation stage or NULL */);
 int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
+/* The tile table without a handle: the tiles and k-slices cusync_mlp_create would take for `cfg` on this device
+ * (fields < 0 / 0 in cfg mean "choose", as there).  What a driver that wires its own stages and launchers looks
+ * up per batch size, as the reference's build looks its shapes up in src/ml-bench/transformer/tile_sizes_db.py.
+ * Returns 0, or 1 with cusync_rt_last_error() set. */
+int cusync_mlp_choice(const cusync_mlp_config *cfg, int *tile1, int *tile2, int *split_k1, int *split_k2);
 int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 
 /* ------------------------------------------------------------------------- */

@@ -72,3 +72,40 @@ def test_resnet_driver(shape, layers, sync):
     _, end = between(out, "START-OVERLAP:", "END-OVERLAP")
     assert float(re.search(r"Total: ([0-9.]+)", end).group(1)) > 0
     assert "check: passed" in out
+
+
+def test_mlp_stages_driver_against_oracle(tmp_path):
+    """The reference's own loop (CuStage + CuSyncGemm objects, invokeWaitKernel, incrementIter) at 256 and 2048 rows,
+    both policies, on inputs this test writes; the launchers' H and Y against the CPU oracle on sampled rows, and
+    bit for bit against each other across policies."""
+    import numpy as np
+    import oracle as orc
+    from util import assert_close, normal_f16, sample_rows, uniform_f16
+    hidden, inner, batches = 12288, 6144, (256, 2048)
+    x, w1, w2 = uniform_f16((max(batches), hidden), 1), normal_f16((hidden, inner), 2), normal_f16((inner, hidden), 3)
+    for name, a in (("x", x), ("w1", w1), ("w2", w2)):
+        a.tofile(tmp_path / (name + ".bin"))
+    out = run("mlp_stages", "--batch", ",".join(str(b) for b in batches), "--sync", "both", "--runs", "5", "--check", "true",
+              "--load", str(tmp_path), "--dump", str(tmp_path))
+    assert out.count("check: passed") == 4
+    rows = [json.loads(l) for l in out.splitlines() if l.startswith('{"batch"')]
+    assert [(r["batch"], r["sync"]) for r in rows] == [(256, "rowsync"), (256, "tilesync"), (2048, "rowsync"), (2048, "tilesync")]
+    for r in rows:
+        assert r["runs"] == 5 and r["launcher_us"] > 0 and r["handle_us"] > 0
+    for b in batches:
+        got = {}
+        for sync in ("rowsync", "tilesync"):
+            h = np.fromfile(tmp_path / ("h_%d_%s.bin" % (b, sync)), dtype=np.float16).reshape(b, inner)
+            y = np.fromfile(tmp_path / ("y_%d_%s.bin" % (b, sync)), dtype=np.float16).reshape(b, hidden)
+            got[sync] = (h, y)
+        sel = sample_rows(b)
+        h, y = got["rowsync"]
+        assert_close(h[sel], orc.gemm(np.ascontiguousarray(x[sel]), w1, orc.EPI_GELU), "H rows, %d" % b)
+        assert_close(y[sel], orc.gemm(np.ascontiguousarray(h[sel]), w2), "Y rows, %d" % b)
+        assert np.array_equal(got["tilesync"][0].view(np.uint16), h.view(np.uint16))
+        assert np.array_equal(got["tilesync"][1].view(np.uint16), y.view(np.uint16))
+
+
+def test_mlp_stages_driver_usage_error():
+    p = subprocess.run([os.path.join(BIN, "mlp_stages"), "--batch", "0"], capture_output=True, text=True, timeout=60)
+    assert p.returncode != 0 and "usage" in p.stderr
