@@ -37,22 +37,39 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 SETTLE_STEPS = 40              # untimed steps of the timed shape before anything is measured: after a light load
                                # the device needs about 30 steps of this size until its clock settles
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_by_tile.md")
+MFMA_TABLE = os.path.join(ROOT, "profiles", "gemm_mfma_by_batch.md")
+
+
+def table_row(path, tiles, batch):
+    """The cells of the row of a committed profile table whose first three columns are the tile ids of the two
+    launches and the batch; None if that combination was never profiled."""
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 4 and cells[0].isdigit() and cells[1].isdigit() and cells[2].isdigit():
+                    if (int(cells[0]), int(cells[1]), int(cells[2])) == (tiles[0], tiles[1], batch):
+                        return cells
+    except OSError:
+        pass
+    return None
 
 
 def traffic_bytes(tiles, batch):
     """HBM bytes per GEMM launch from the committed counter runs (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
     plain copy of known size), looked up by the tile ids of the two launches and the batch; None if that
     combination was never profiled."""
-    try:
-        with open(TRAFFIC_TABLE) as f:
-            for line in f:
-                cells = [c.strip() for c in line.strip().strip("|").split("|")]
-                if len(cells) >= 4 and cells[0].isdigit() and cells[1].isdigit() and cells[2].isdigit():
-                    if (int(cells[0]), int(cells[1]), int(cells[2])) == (tiles[0], tiles[1], batch):
-                        return float(cells[3]) * 1e6
-    except OSError:
-        pass
-    return None
+    row = table_row(TRAFFIC_TABLE, tiles, batch)
+    return float(row[3]) * 1e6 if row else None
+
+
+def mfma_busy(tiles, batch):
+    """From the committed SQ counter runs, for the tile ids of the two launches and the batch: the share of SIMD
+    cycles the matrix pipes were busy over the launch, at the clock the launch ran at (SQ_VALU_MFMA_BUSY_CYCLES per
+    SIMD over SQ_BUSY_CYCLES per shader engine), that clock, and the share of wave time spent waiting
+    (SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES).  None if that combination was never profiled."""
+    row = table_row(MFMA_TABLE, tiles, batch)
+    return {"mfma_busy_pct": float(row[3]), "clock_ghz": float(row[4]), "wait_inst_any_pct": float(row[5])} if row else None
 
 
 def trimmed(times):
@@ -113,6 +130,12 @@ def main():
     ap.add_argument("--profile-chain", choices=["attention", "conv", "mlp"], default=None,
                     help="run only the stream-ordered attention chain (S = 2048) or convolution pairs, or (mlp) --steps rounds of "
                          "the GPT-3 MLP at --batch stream-ordered / RowSync / TileSync in turn, for rocprofv3")
+    ap.add_argument("--timeline", action="store_true",
+                    help="with --roofline-only: one more step with the kernels' per-workgroup clock records switched on "
+                         "(cusync_rt_set_timeline); prints where a workgroup's time goes per launch")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="with --roofline-only: X, W1 and W2 all zero.  Same instruction stream, far less switching in the "
+                         "matrix pipes: what the kernels take when the device's power limit does not set the clock")
     ap.add_argument("--tile1", type=int, default=-1)
     ap.add_argument("--tile2", type=int, default=-1)
     args = ap.parse_args()
@@ -135,6 +158,11 @@ def main():
     w1_host, w2_host = normal((HIDDEN, INNER), 2), normal((INNER, HIDDEN), 3)
     x_host = np.random.default_rng(1).uniform(-1, 1, (max(BATCHES), HIDDEN)).astype(np.float32).astype(np.float16)
     w1, w2, x_all = (torch.from_numpy(a).cuda() for a in (w1_host, w2_host, x_host))
+    if args.zero_operands:
+        if not args.roofline_only:
+            sys.exit("bench.py: --zero-operands is a diagnosis of the --roofline-only leg")
+        for t in (w1, w2, x_all):
+            t.zero_()
     torch.cuda.synchronize()
 
     class Chain:
@@ -169,6 +197,20 @@ def main():
                 times[i].append(c.step(split=split_first and i == 0))
         return times
 
+    def rounds(objs, step, warm=10, timed=20):
+        """The same turn-taking for the other chains' handles: `step(obj)` runs one pass and returns ([us], extra).
+        Returns the step times and the extras, one list per object."""
+        for _ in range(warm):
+            for o in objs:
+                step(o)
+        times, extras = [[] for _ in objs], [[] for _ in objs]
+        for _ in range(timed):
+            for i, o in enumerate(objs):
+                t, e = step(o)
+                times[i].append(t[0])
+                extras[i].append(e[0] if e else None)
+        return times, extras
+
     def settle(batch, steps=SETTLE_STEPS):
         """Untimed steps of the timed shape: brings the clock to where it stays under this load."""
         c = Chain(batch, api.SYNC.STREAM)
@@ -181,6 +223,38 @@ def main():
         c = Chain(B, api.SYNC.STREAM)
         (t3,) = interleaved([c], warm, timed, split_first=True)
         tiles = c.tiles
+        timeline = None
+        if args.timeline:
+            # one record per finished tile: 100 MHz clock at kernel entry of the workgroup, tile drawn, first loads
+            # issued, main loop done, epilogue (and post) done
+            from cusync_amd import _lib
+            buf = torch.zeros(1 + 8 * 8192, dtype=torch.int64, device="cuda")
+            torch.cuda.synchronize()
+            _lib.load().cusync_rt_set_timeline(buf.data_ptr(), buf.numel() * 8)
+            c.step()
+            _lib.load().cusync_rt_set_timeline(None, 0)
+            r = buf.cpu().numpy()
+            rec = r[1:1 + 8 * int(r[0])].reshape(-1, 8)
+            entry = np.sort(np.unique(rec[:, 6]))
+            cut = entry[int(np.argmax(np.diff(entry))) + 1] if len(entry) > 1 else entry[0] + 1      # first workgroup of GEMM2
+            timeline = {}
+            for name, m in (("gemm1", rec[:, 6] < cut), ("gemm2", rec[:, 6] >= cut)):
+                q = rec[m]
+                if len(q) == 0:
+                    continue
+                t0 = q[:, 6].min()
+                first = q[(q[:, 1] >> 48) == 0]          # a workgroup's first tile: its prologue starts at kernel entry
+                def med(v):
+                    return round(float(np.median(v)) / 100.0, 2)
+                timeline[name] = {
+                    "tiles": int(len(q)), "workgroups": int(len(np.unique(q[:, 0] >> 8 & 0xffffffff))),
+                    "entry_spread_us": round(float(q[:, 6].max() - t0) / 100.0, 2),
+                    "entry_to_first_loads_us": med(first[:, 3] - first[:, 6]),
+                    "k_loop_us": {"median": med(q[:, 4] - q[:, 3]), "min": round(float((q[:, 4] - q[:, 3]).min()) / 100.0, 2),
+                                  "max": round(float((q[:, 4] - q[:, 3]).max()) / 100.0, 2)},
+                    "epilogue_us": med(q[:, 5] - q[:, 4]),
+                    "last_tile_done_us": round(float(q[:, 5].max() - t0) / 100.0, 2),
+                }
         c.close()
         t_s, g1, g2 = [v[0] for v in t3], [v[1] for v in t3], [v[2] for v in t3]
         k_us = (statistics.fmean(g1) + statistics.fmean(g2)) / 2
@@ -201,7 +275,10 @@ def main():
                 if hbm_bound else
                 {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                  "frac": round(achieved / PEAK_FP16_TFLOPS, 4)})
-        return {**head, "traffic": traffic_bytes(tiles, B),
+        busy = mfma_busy(tiles, B)
+        return {**head, "traffic": traffic_bytes(tiles, B), "mfma_busy_pct": busy["mfma_busy_pct"] if busy else None,
+                "clock_ghz_under_load": busy["clock_ghz"] if busy else None, **({"timeline": timeline} if timeline else {}),
+                **({"operands": "all zero"} if args.zero_operands else {}),
                 "kernel": "gemmDmaKernel, mean of the two launches of the step: GEMM1 tile %s %.1f us, GEMM2 tile %s %.1f us "
                           "(stream-ordered, %.1f GFLOP per launch)" % (shapes[0], statistics.fmean(g1), shapes[1], statistics.fmean(g2),
                                                                        flops_per_launch / 1e9),
@@ -344,6 +421,8 @@ def main():
                 "best_tflops": round(mlp_flops(b) / best / 1e6, 1),
                 "bound": "mfma" if mlp_flops(b) / (PEAK_FP16_TFLOPS * 1e12) > mlp_bytes(b) / (PEAK_HBM_GBS * 1e9) else "hbm",
                 "roofline_frac": round(ideal_us(b) / best, 4),
+                # stream-ordered launches of these tiles at this batch, from the committed counter runs
+                "mfma_busy_pct": (mfma_busy(tiles, b) or {}).get("mfma_busy_pct"),
             })
 
     # ---- the other chains of the benchmark set: self-attention and the convolution pair --------
@@ -361,16 +440,16 @@ def main():
             y = torch.empty((seq, HIDDEN), dtype=torch.float16, device="cuda")
             torch.cuda.synchronize()
             row = {"S": seq}
-            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE),
-                               ("consecutivesync", api.SYNC.STRIDED)):
-                layer = api.AttnLayer(seq, HIDDEN, heads, sync, wqkv.data_ptr(), wo.data_ptr())
-                layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=10)
-                t, st = layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=20, stages=True)
+            # all modes alive together, one step each per round (10 untimed rounds, 20 timed), like the GPT-3 sweep
+            modes = (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE), ("consecutivesync", api.SYNC.STRIDED))
+            layers = [api.AttnLayer(seq, HIDDEN, heads, sync, wqkv.data_ptr(), wo.data_ptr()) for _, sync in modes]
+            t, st = rounds(layers, lambda l: l.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=1, stages=True))
+            for (name, sync), layer, tt, ss in zip(modes, layers, t, st):
                 if any(layer.stage_state(i).spin_timeouts for i in range(3)):
                     sys.exit("bench.py: attention chain waits timed out — results invalid")
-                row[name + "_us"] = round(trimmed(t)[0], 2)
+                row[name + "_us"] = round(trimmed(tt)[0], 2)
                 if sync == api.SYNC.STREAM:
-                    row["stage_us"] = [round(trimmed([v[i] for v in st])[0], 2) for i in range(3)]
+                    row["stage_us"] = [round(trimmed([v[i] for v in ss])[0], 2) for i in range(3)]
                     row["tiles"] = list(layer.tiles())
                 layer.destroy()
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "consecutivesync_us"))
@@ -387,29 +466,19 @@ def main():
             ly = torch.empty((b, lh), dtype=torch.float16, device="cuda")
             torch.cuda.synchronize()
             row = {"B": b}
-            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE), ("stridedsync", api.SYNC.STRIDED)):
-                m = api.Mlp(api.MODEL.LLAMA, b, lh, li, sync, lw1.data_ptr(), lw2.data_ptr())
-                m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
-                t = m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20)
+            # rowsync_one_launch: both GEMMs in one launch (the handle gives GEMM2 the tile of GEMM1, which from 512 rows
+            # on costs this chain more than the launch saves); *_repacked: W2's rows are 16 KiB, the handle's copies pad them
+            modes = (("stream", api.SYNC.STREAM, {}), ("rowsync", api.SYNC.ROW, {}), ("tilesync", api.SYNC.TILE, {}),
+                     ("stridedsync", api.SYNC.STRIDED, {}), ("rowsync_one_launch", api.SYNC.ROW, {"one_launch": True}),
+                     ("stream_repacked", api.SYNC.STREAM, {"repack_weights": True}), ("rowsync_repacked", api.SYNC.ROW, {"repack_weights": True}))
+            ms = [api.Mlp(api.MODEL.LLAMA, b, lh, li, sync, lw1.data_ptr(), lw2.data_ptr(), **kw) for _, sync, kw in modes]
+            t, _ = rounds(ms, lambda m: (m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=1), None))
+            for (name, sync, kw), m, tt in zip(modes, ms, t):
                 if m.stage_state(1).spin_timeouts:
                     sys.exit("bench.py: LLaMA consumer waits timed out — results invalid")
-                row[name + "_us"] = round(trimmed(t)[0], 2)
-                row[name + "_tiles"] = list(m.tiles())
-                m.destroy()
-            # both GEMMs in one launch (the handle gives GEMM2 the tile of GEMM1, which from 512 rows on costs this
-            # chain more than the launch saves)
-            m = api.Mlp(api.MODEL.LLAMA, b, lh, li, api.SYNC.ROW, lw1.data_ptr(), lw2.data_ptr(), one_launch=True)
-            m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
-            t = m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20)
-            if m.stage_state(1).spin_timeouts:
-                sys.exit("bench.py: LLaMA consumer waits timed out — results invalid")
-            row["rowsync_one_launch_us"] = round(trimmed(t)[0], 2)
-            row["rowsync_one_launch_tiles"] = list(m.tiles())
-            m.destroy()
-            for name, sync in (("stream", api.SYNC.STREAM), ("rowsync", api.SYNC.ROW)):      # W2's rows are 16 KiB
-                m = api.Mlp(api.MODEL.LLAMA, b, lh, li, sync, lw1.data_ptr(), lw2.data_ptr(), repack_weights=True)
-                m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=10)
-                row[name + "_repacked_us"] = round(trimmed(m.run(lx.data_ptr(), lhid.data_ptr(), ly.data_ptr(), runs=20))[0], 2)
+                row[name + "_us"] = round(trimmed(tt)[0], 2)
+                if not kw.get("repack_weights"):
+                    row[name + "_tiles"] = list(m.tiles())
                 m.destroy()
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "stridedsync_us", "rowsync_one_launch_us"))
             row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)
@@ -423,14 +492,14 @@ def main():
             torch.cuda.synchronize()
             row = {"shape": [n, hh, ww, cc], "gflop": round(2 * 2.0 * n * hh * ww * cc * 9 * cc / 1e9, 2)}
             # *_one_launch: both layers in one launch, same semaphores (no wait kernel, no second launch)
-            for name, sync, fused in (("stream", api.SYNC.STREAM, False), ("rowsync", api.SYNC.ROW, False), ("tilesync", api.SYNC.TILE, False),
-                                      ("rowsync_one_launch", api.SYNC.ROW, True), ("tilesync_one_launch", api.SYNC.TILE, True)):
-                ch = api.ConvChain(n, hh, ww, cc, [w.data_ptr() for w in ws], sync, fused=fused)
-                ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=10)
-                t = ch.run(xc.data_ptr(), [t.data_ptr() for t in ys], runs=20)
+            modes = (("stream", api.SYNC.STREAM, False), ("rowsync", api.SYNC.ROW, False), ("tilesync", api.SYNC.TILE, False),
+                     ("rowsync_one_launch", api.SYNC.ROW, True), ("tilesync_one_launch", api.SYNC.TILE, True))
+            chs = [api.ConvChain(n, hh, ww, cc, [w.data_ptr() for w in ws], sync, fused=fused) for _, sync, fused in modes]
+            t, _ = rounds(chs, lambda ch: (ch.run(xc.data_ptr(), [v.data_ptr() for v in ys], runs=1), None))
+            for (name, sync, fused), ch, tt in zip(modes, chs, t):
                 if any(ch.stage_state(i).spin_timeouts for i in range(2)):
                     sys.exit("bench.py: convolution chain waits timed out — results invalid")
-                row[name + "_us"] = round(trimmed(t)[0], 2)
+                row[name + "_us"] = round(trimmed(tt)[0], 2)
                 row["tile"] = ch.tile()
                 ch.destroy()
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "rowsync_one_launch_us", "tilesync_one_launch_us"))
