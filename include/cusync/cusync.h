@@ -245,6 +245,9 @@ public:
   // First statement of a sync-aware kernel: returns the tile this workgroup
   // processes (a ticket through the tile order, or blockIdx with
   // AvoidCustomOrder / a null shared_storage) and raises the wait-kernel flag.
+  // The ticket is the workgroup's linear index when the launch has one workgroup
+  // per tile, otherwise the next value of the stage's dispenser
+  // (src/include/cusync/cusync_device_defs.h:77-103).
   CUSYNC_DEVICE dim3 tile(dim3* shared_storage);
 #endif
 };
@@ -309,13 +312,35 @@ CUSTAGE_METHOD(dim3) tile(dim3* shared_storage) {
     return dim3(blockIdx.x, blockIdx.y, blockIdx.z);
   }
   if (leader) {
-    const uint32_t ticket = dev::ticketAdd(tileCounter, 1);
-    if (ticket == numTiles() - 1) {
-      // Last ticket: every workgroup of this run has started, so none of them
-      // can be kept off the device by a spinning consumer.  Re-arm the
-      // dispenser and let the consumer's stream go.
-      dev::storeRelaxed(tileCounter, 0);
-      if (raisesFlag) raiseFlag();
+    const uint32_t launched = gridDim.x * gridDim.y * gridDim.z;
+    uint32_t ticket;
+    if (launched == numTiles()) {
+      // One workgroup per tile, the usual launch: the ticket is the workgroup's linear index, which the hardware
+      // hands out in increasing order, and nobody touches the dispenser (a device-wide atomic that every workgroup
+      // of a launch hits at kernel start costs the launch about 11 ns per workgroup, one after the other).
+      ticket = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+      if (raisesFlag) {
+        // Every workgroup of this run has started once all have been counted.  They are counted in eight lists by
+        // index modulo 8 (the workgroups of a list share an XCD, and the eight counters eight memory channels); the
+        // last of a list reports for it, the last list to report raises the flag.  Whoever closes a count re-arms it.
+        const uint32_t list = ticket & 7u, members = (launched - list + 7u) / 8u, lists = launched < 8u ? launched : 8u;
+        if (dev::ticketAdd(&xcdTickets_[list * 32], 1) == members - 1) {
+          dev::storeRelaxed(&xcdTickets_[list * 32], 0);
+          if (dev::ticketAdd(&xcdTickets_[8 * 32], 1) == lists - 1) {
+            dev::storeRelaxed(&xcdTickets_[8 * 32], 0);
+            raiseFlag();
+          }
+        }
+      }
+    } else {
+      ticket = dev::ticketAdd(tileCounter, 1);
+      if (ticket == numTiles() - 1) {
+        // Last ticket: every workgroup of this run has started, so none of them
+        // can be kept off the device by a spinning consumer.  Re-arm the
+        // dispenser and let the consumer's stream go.
+        dev::storeRelaxed(tileCounter, 0);
+        if (raisesFlag) raiseFlag();
+      }
     }
     *shared_storage = tileOrder[ticket];
   }

@@ -71,3 +71,24 @@ def test_static_workspace_without_slices_and_beyond_limit():
     assert L.cusync_gemm_run_static_workspace(C.byref(args), None) == api.ERR.NOT_INITIALIZED      # refused before any launch
     assert "workspace" in api.last_error()
     st.destroy()
+
+
+def test_static_workspace_calls_leave_device_memory_as_it_is():
+    """What the entry point is for: after one warm-up call on a device (which looks the kernel's occupancy and the
+    array's address up) further calls neither allocate nor free device memory."""
+    import torch
+    L = _lib.load()
+    M, N, K, tile, split = 200, 392, 1024, api.TILE.T128x128x32, 4
+    da, db = to_dev(uniform_f16((M, K), 61)), to_dev(normal_f16((K, N), 62, std=0.05))
+    dd = empty_dev((M, N), fill=float("nan"))
+    st = api.Stage(api.gemm_grid(tile, M, N, split), (1, 1, 1), api.no_sync(), api.no_sync())
+    args = api.gemm_args(st, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dd.data_ptr(), N, tile, split_k=split)
+    assert L.cusync_gemm_run_static_workspace(C.byref(args), None) == api.ERR.SUCCESS, api.last_error()      # warm-up
+    assert L.cusync_rt_device_sync() == 0
+    free_before, total = torch.cuda.mem_get_info()
+    for _ in range(5):
+        assert L.cusync_gemm_run_static_workspace(C.byref(args), None) == api.ERR.SUCCESS, api.last_error()
+        assert torch.cuda.mem_get_info()[0] == free_before          # also while the launch is in flight
+    assert L.cusync_rt_device_sync() == 0
+    assert torch.cuda.mem_get_info() == (free_before, total)
+    st.destroy()
