@@ -122,10 +122,14 @@ __device__ __forceinline__ float fastErf(float x) {
   return __builtin_copysignf(r, x);
 }
 
-__device__ __forceinline__ float applyEpilogue(float v, int epilogue) {
-  if (epilogue == CUSYNC_EPILOGUE_GELU) return 0.5f * v * (1.0f + fastErf(v * 0.70710678118654752f));
-  if (epilogue == CUSYNC_EPILOGUE_RELU) return v > 0.0f ? v : 0.0f;
-  return v;
+// The epilogue kind is a template argument: asked per value at run time, even the plain conversion cost the
+// 256x384 tile 8 us per tile in scalar compares and branches (its 192 values per lane), and GeLU 3 us more
+// than its arithmetic.  Callers branch once per pass of a tile (TileStore::pass).
+template<int EPILOGUE>
+__device__ __forceinline__ float applyEpilogue(float v) {
+  if constexpr (EPILOGUE == CUSYNC_EPILOGUE_GELU) return 0.5f * v * (1.0f + fastErf(v * 0.70710678118654752f));
+  else if constexpr (EPILOGUE == CUSYNC_EPILOGUE_RELU) return v > 0.0f ? v : 0.0f;
+  else return v;
 }
 
 __device__ __forceinline__ float siluf(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
@@ -232,6 +236,21 @@ struct TileStore {
     }
   }
 
+  // This wave's 32 rows x WTN columns of a pass into the buffer, one kind of epilogue applied.
+  template<int EPILOGUE, int PITCH, class V>
+  __device__ __forceinline__ void writeRows(V&& value) const {
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const floatx4 v = value(j, g);
+        half4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue<EPILOGUE>(v[e]);
+        *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = o;
+      }
+  }
+
   template<class V>
   __device__ __forceinline__ void pass(int i, uint32_t rows, V&& value) const {
     if (p.epilogue == CUSYNC_EPILOGUE_SWIGLU) { passPairs(i, rows, value); return; }
@@ -243,16 +262,9 @@ struct TileStore {
     static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
     __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
     if ((rows >> wm) & 1) {
-#pragma unroll
-      for (int j = 0; j < C::TN; j++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const floatx4 v = value(j, g);
-          half4 o;
-#pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (half_t)applyEpilogue(v[e], p.epilogue);
-          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = o;
-        }
+      if (p.epilogue == CUSYNC_EPILOGUE_GELU) writeRows<CUSYNC_EPILOGUE_GELU, PITCH>(value);
+      else if (p.epilogue == CUSYNC_EPILOGUE_RELU) writeRows<CUSYNC_EPILOGUE_RELU, PITCH>(value);
+      else writeRows<CUSYNC_EPILOGUE_NONE, PITCH>(value);
     }
     __syncthreads();
 #pragma unroll

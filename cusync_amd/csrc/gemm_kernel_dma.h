@@ -32,17 +32,18 @@
 // kt+1, so that the fragments of (kt+1, k-step 0) are read under the MFMAs of
 // (kt, k-step 1); the loads of chunk kt+STAGES-1 go into the stage of chunk kt-1.
 //
-// Alternating order (DmaCfg::PINGPONG, for the tiles whose accumulators leave no registers for a second set of
-// fragments: 256x384 is 192 accumulator registers per lane).  What binds these GEMMs is data moved per MFMA — bytes
-// from L2 into LDS through the CU's one vector memory path, bytes from LDS into registers, and the power both
-// cost — so the tile is made as large as the register file allows, and the overlap that a second set of fragments
-// gave a wavefront comes from its neighbour instead.  The eight wavefronts are two groups of four, one wavefront
-// of each group per SIMD.  A wavefront alternates a load phase (the fragments of one k-step from LDS, all at
-// once, into its only set of fragment registers) and a compute phase (that k-step's MFMAs, raised priority, the
-// direct loads of a later chunk issued between them); the second group runs one phase behind the first, so that
-// on every SIMD one wavefront computes while the other loads.  One barrier per chunk keeps the groups in step:
-// the first group meets it between two chunks, the second between the load and the compute phase of a chunk's
-// second k-step.
+// Assembly order (DmaCfg::PINGPONG, the 256x384x32 and 256x192x64 tiles: up to 192 accumulator registers per lane
+// leave the compiler no room to schedule a loop around them).  What binds these GEMMs is data moved per MFMA: bytes
+// from L2 into LDS through the CU's one vector memory path, which holds a bounded number of requests at once (so both
+// operands are fetched in whole 128-byte lines, A 64 columns of K at a time), bytes from LDS into registers, and
+// the power both cost; the tile is as large as the register file allows and has its CU to itself.  The K loop is
+// one asm statement written by gen_wide_steps.py (gemm_wide_steps.inc): all eight wavefronts run the same stream,
+// two per SIMD, so that one wavefront's waits fall under its partner's MFMAs; the fragments of k-step s+1 are read
+// from LDS progressively under the MFMAs of step s, every MFMA waiting for its own operands only; one barrier per
+// chunk, placed behind the first MFMAs of the preceding chunk's last k-step; the direct loads of the chunks two and
+// three ahead are issued between the MFMAs.  (An earlier form ran the wavefronts as two groups half a k-step out of
+// phase; the single stream measured 4 % faster.)  A tile-policy consumer waits for all its producer tiles before the
+// first load: the loop has no place for a poll.
 #pragma once
 
 #include "gemm_tiles.h"
@@ -53,7 +54,7 @@ namespace gemm {
 template<int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WAVES_PER_SIMD_ = 1, bool BT_ = false, bool PIPE_ = false, bool PINGPONG_ = false>
 struct DmaCfg {
   static constexpr bool PIPE = PIPE_;                      // barrier in the middle of a chunk, fragments prefetched across chunks
-  static constexpr bool PINGPONG = PINGPONG_;              // two groups of wavefronts half a k-step apart, fragments held once (see below)
+  static constexpr bool PINGPONG = PINGPONG_;              // K loop in assembly, operands in whole cache lines (see above)
   static constexpr bool BT = BT_;                          // B given as [N][K] (k contiguous), e.g. KRSC filters
   static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // register budget: 512 / this per lane
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
