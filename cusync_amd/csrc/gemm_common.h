@@ -2,6 +2,8 @@
 // loads, epilogue math and the instruction-order directives.
 #pragma once
 
+#include <type_traits>
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <utility>
@@ -177,6 +179,10 @@ __device__ __forceinline__ void schedPass() {
   }
 }
 
+// True for the tile configurations whose K loop is assembly (DmaCfg::PINGPONG).
+template<class C, class = void> struct IsAssemblyTile : std::false_type {};
+template<class C> struct IsAssemblyTile<C, std::enable_if_t<C::PINGPONG>> : std::true_type {};
+
 // Stores of an output tile.  Final values go through LDS so that global memory sees whole rows: a lane holds 4
 // consecutive columns of 32 different rows, which stored directly would be 8-byte pieces scattered over 32 cache
 // lines per instruction.  One pass per MFMA row tile: every wave writes its 32 rows x WTN columns (fp16, epilogue
@@ -193,13 +199,23 @@ struct TileStore {
   char* lds;
   uint32_t m0, n0;
   int wm, wn, lane;
+  uint32_t tid;        // threadIdx.x, opaque to the compiler where the K loop is assembly (see the constructor)
   bool through;
   __amdgpu_buffer_rsrc_t rD;
   static constexpr uint32_t kAllRows = (1u << C::WM) - 1;
 
   __device__ __forceinline__ TileStore(const GemmParams& p_, const cusync_dim3& t, int wm_, int wn_, int lane_, char* lds_)
-      : p(p_), lds(lds_), m0(t.y * C::BM), n0(t.x * C::BN), wm(wm_), wn(wn_), lane(lane_), through(p_.stage.storesThrough()),
-        rD(makeRsrc(p_.D, p_.M * p_.ldd * 2)) {}
+      : p(p_), lds(lds_), m0(t.y * C::BM), n0(t.x * C::BN), wm(wm_), wn(wn_), lane(lane_), tid(threadIdx.x), through(p_.stage.storesThrough()),
+        rD(makeRsrc(p_.D, p_.M * p_.ldd * 2)) {
+    // Everything the copy-out computes per thread (piece index -> row, column, offset) depends on the thread index
+    // only, so the compiler works it out once, ahead of the tile loop, and keeps it live across the K loop: where
+    // that loop is assembly with most registers named, those values wait in scratch and every tile's epilogue
+    // reloads them.  Made opaque here, they are computed where they are used.
+    if constexpr (IsAssemblyTile<C>::value) {
+      asm volatile("" : "+v"(tid));
+      asm volatile("" : "+v"(lane));
+    }
+  }
 
   template<class V>
   __device__ __forceinline__ void passPairs(int i, uint32_t rows, V&& value) const {
@@ -225,7 +241,7 @@ struct TileStore {
     __syncthreads();
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
-      const uint32_t idx = s * C::THREADS + threadIdx.x;
+      const uint32_t idx = s * C::THREADS + tid;
       const uint32_t lr = idx / CPR, c = idx % CPR;
       const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 / 2 + c * 8;
       const bool inside = m < p.M && n < p.N / 2 && ((rows >> (lr / 32)) & 1);
@@ -266,10 +282,35 @@ struct TileStore {
       else if (p.epilogue == CUSYNC_EPILOGUE_RELU) writeRows<CUSYNC_EPILOGUE_RELU, PITCH>(value);
       else writeRows<CUSYNC_EPILOGUE_NONE, PITCH>(value);
     }
+    copyOut(i, rows);
+  }
+
+  // The same pass for values that are final fp16 already (the epilogue applied and four columns packed into two
+  // registers): half4At(j, g).
+  template<class V>
+  __device__ __forceinline__ void passHalf(int i, uint32_t rows, V&& half4At) const {
+    constexpr int PITCH = C::BN * 2 + 16;
+    __syncthreads();
+    if ((rows >> wm) & 1) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+          *reinterpret_cast<half4*>(lds + (wm * 32 + (lane & 31)) * PITCH + (wn * C::WTN + j * 32 + 8 * g + 4 * (lane >> 5)) * 2) = half4At(j, g);
+    }
+    copyOut(i, rows);
+  }
+
+  // Second half of a pass: all threads copy the buffer out to global memory.
+  __device__ __forceinline__ void copyOut(int i, uint32_t rows) const {
+    constexpr int PITCH = C::BN * 2 + 16;
+    constexpr int ROWS = C::WM * 32;
+    constexpr int CPR = C::BN / 8;
+    constexpr int STEPS = ROWS * CPR / C::THREADS;
     __syncthreads();
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
-      const uint32_t idx = s * C::THREADS + threadIdx.x;
+      const uint32_t idx = s * C::THREADS + tid;
       const uint32_t lr = idx / CPR, c = idx % CPR;
       const uint32_t m = m0 + (lr / 32) * C::WTM + i * 32 + lr % 32, n = n0 + c * 8;
       // Every thread issues every store, those outside the matrix (or outside `rows`) with an offset the buffer
@@ -313,6 +354,31 @@ __device__ __forceinline__ bool finishTile(const GemmParams& p, floatx16 (&acc)[
                                            const cusync_dim3& t, int wm, int wn, int lane, uint32_t* sLast, char* lds) {
   if constexpr (SPLIT) { if (p.splitK > 1) return finishTileSplit<C>(p, acc, t, wm, wn, lane, sLast, lds); }
   const TileStore<C> store(p, t, wm, wn, lane, lds);
+  if constexpr (IsAssemblyTile<C>::value && C::TM * C::TN <= 6) {
+    // The 256x192x64 tile (96 accumulators per lane, K loop in assembly): epilogue and conversion come first, for
+    // the whole tile at once and in place (two results per register), and the passes move packed values only
+    // (GEMM1 of the 2048-row MLP with GeLU: 10.1 -> 8.4 us per tile).  Not for the 256x384 tile: with 192
+    // accumulators the same form made the compiler park twice as much in scratch (16 -> 28 us).
+    if (p.epilogue != CUSYNC_EPILOGUE_SWIGLU) {
+      half4 h[C::TM][C::TN][4];
+      auto packAll = [&](auto kind) {
+#pragma unroll
+        for (int i = 0; i < C::TM; i++)
+#pragma unroll
+          for (int j = 0; j < C::TN; j++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+              for (int e = 0; e < 4; e++) h[i][j][g][e] = (half_t)applyEpilogue<decltype(kind)::value>(acc[i][j][g * 4 + e]);
+      };
+      if (p.epilogue == CUSYNC_EPILOGUE_GELU) packAll(std::integral_constant<int, CUSYNC_EPILOGUE_GELU>{});
+      else if (p.epilogue == CUSYNC_EPILOGUE_RELU) packAll(std::integral_constant<int, CUSYNC_EPILOGUE_RELU>{});
+      else packAll(std::integral_constant<int, CUSYNC_EPILOGUE_NONE>{});
+#pragma unroll
+      for (int i = 0; i < C::TM; i++) store.passHalf(i, TileStore<C>::kAllRows, [&](int j, int g) { return h[i][j][g]; });
+      return true;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < C::TM; i++)
     store.pass(i, TileStore<C>::kAllRows, [&](int j, int g) {
