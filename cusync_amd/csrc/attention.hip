@@ -252,6 +252,9 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   auto inLines = [](int tile, uint32_t K) { return tile == CUSYNC_TILE_256x192x32 && K % 64 == 0 ? (int)CUSYNC_TILE_256x192x64 : tile; };
   L->tile1 = cfg->tile1 >= 0 ? cfg->tile1 : (3 * L->E) % 192 == 0 ? inLines(wide1, cfg->hidden) : dflt;
   L->tile3 = cfg->tile3 >= 0 ? cfg->tile3 : cfg->hidden % 192 == 0 ? inLines(wide3, L->E) : dflt;
+  // (above 1024 rows the output projection's five to eight row tiles of 256x384, at most one per CU, beat 128x192 at
+  // two workgroups per CU: the chain under RowSync 216 -> 212 us at 1280 rows, 267 -> 255 at 1536, 327 -> 311 at 2048)
+  if (cfg->tile3 < 0 && S > 1024 && cfg->hidden % 384 == 0 && L->E % 64 == 0) L->tile3 = CUSYNC_TILE_256x384x32;
   L->ws1 = L->ws3 = L->ws2 = nullptr;
   // Key ranges of 8 blocks (512 rows) or more are cut in two: under a causal mask the last row tiles walk the
   // longest ranges and the launch is as long as its longest workgroup.  Measured alone at 12 heads: 512 rows

@@ -238,13 +238,16 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
   }
   // Where K is a multiple of 64 the 256x192 tile with both operands fetched 64 columns at a time, in whole cache
   // lines, and its K loop in assembly takes over from the 32-column one (GPT-3 shard, same machine, stream-ordered:
-  // 512 rows 204 -> 196 us, 1024 rows 330 -> 308, 2048 rows 612 -> 562), and from 1664 rows on GEMM2 runs one
-  // 256x384 tile per CU where its width allows (12288 columns are 32 of them; 2048 rows: 562 -> 557 us; with fewer
-  // rows it would need k-slices, whose reduction costs it more than the tile gains).  Both wait for all their
+  // 512 rows 204 -> 196 us, 1024 rows 330 -> 308, 2048 rows 612 -> 562), and from 1025 rows on GEMM2 runs 256x384
+  // tiles, at most one per CU, where its width allows (12288 columns are 32 of them; 2048 rows: 562 -> 557 us; with
+  // fewer rows it would need k-slices, whose reduction costs it more than the tile gains).  Both wait for all their
   // producer tiles before the first load, whatever the policy.
   const uint32_t k1 = c.hidden, k2 = c.inner;
   if (a == CUSYNC_TILE_256x192x32 && k1 % 64 == 0) a = CUSYNC_TILE_256x192x64;
-  if (b == CUSYNC_TILE_256x192x32 && k2 % 64 == 0) b = c.batch > 1536 && n2 % 384 == 0 && !c.one_launch ? CUSYNC_TILE_256x384x32 : CUSYNC_TILE_256x192x64;
+  if (b == CUSYNC_TILE_256x192x32 && k2 % 64 == 0) b = CUSYNC_TILE_256x192x64;
+  // (1025 to 1536 rows, five or six row tiles: 160 or 192 tiles of 256x384 in one round against 128x192 at two
+  // workgroups per CU in one and a half: 1056 rows 397 -> 347 us, 1152: 404 -> 353, 1280: 407 -> 365, 1536: 444 -> 400)
+  if (big && c.batch > 1024 && !swiglu && k2 % 64 == 0 && n2 % 384 == 0 && !c.one_launch) b = CUSYNC_TILE_256x384x32;
   *t1 = c.tile1 >= 0 ? c.tile1 : a;
   *t2 = c.tile2 >= 0 ? c.tile2 : b;
   // both GEMMs in one launch share a kernel: the consumer takes the producer's tile
