@@ -244,8 +244,11 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   const int small = cfg->seq <= 32 ? CUSYNC_TILE_D32x128x64 : cfg->seq <= 64 ? CUSYNC_TILE_64x128x64 : CUSYNC_TILE_128x128x64;
   const int dflt = cfg->seq <= 128 ? small : cfg->seq <= 1024 ? CUSYNC_TILE_128x128x32 : CUSYNC_TILE_128x256x32;
   const uint32_t S = cfg->seq;
-  const int wide1 = S <= 32 ? small : S <= 320 ? CUSYNC_TILE_D64x192x64 : S > 640 && S <= 768 ? CUSYNC_TILE_256x192x32
-                    : S <= 1024 ? CUSYNC_TILE_128x192x32_ALONE : CUSYNC_TILE_256x192x32;
+  // (with the 256x192 tile's K loop in assembly, 256x192 in k-slices also leads from 321 to 512 rows and from 769 to
+  // 1024: the QKV projection 73 -> 67 us at 384 rows, 131 -> 115 at 896, 137 -> 120 at 1024; from 513 to 640 rows its
+  // third row tile is mostly padding and 128x192 stays, 87 against 102 us)
+  const int wide1 = S <= 32 ? small : S <= 320 ? CUSYNC_TILE_D64x192x64 : S > 512 && S <= 640 ? CUSYNC_TILE_128x192x32_ALONE
+                    : CUSYNC_TILE_256x192x32;
   const int wide3 = S <= 32 ? small : S <= 256 ? CUSYNC_TILE_D64x192x64 : S <= 512 ? CUSYNC_TILE_128x192x32_ALONE
                     : S <= 1024 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;
   // (where K is a multiple of 64, the 256x192 tile that fetches both operands 64 columns at a time, K loop in assembly)

@@ -33,7 +33,8 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
          api.TILE.T256x64x64: (4, 1, 2), api.TILE.T128x64x64: (2, 2, 2), api.TILE.T256x128x32: (2, 2, 3),
          api.TILE.T128x256x32: (2, 2, 3), api.TILE.T128x128x32: (2, 2, 3), api.TILE.T128x192x32: (2, 2, 3),
          api.TILE.T256x192x32: (4, 2, 4), api.TILE.D32x128x64: (1, 4, 4), api.TILE.D64x128x64: (1, 4, 3),
-         api.TILE.D64x192x64: (2, 2, 4), api.TILE.T128x192x32_ALONE: (2, 2, 4)}
+         api.TILE.D64x192x64: (2, 2, 4), api.TILE.T128x192x32_ALONE: (2, 2, 4), api.TILE.T256x384x32: (2, 4, 3),
+         api.TILE.T256x192x64: (4, 2, 4)}
 
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 
@@ -54,9 +55,9 @@ def candidates(batch, n1, n2):
     elif batch <= 128:
         tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x128x64, api.TILE.T128x128x32], [1, 2, 4, 8]
     elif batch <= 512:
-        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4, 8]
+        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x64, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4, 8]
     else:
-        tiles, splits = [api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
+        tiles, splits = [api.TILE.T256x192x64, api.TILE.T256x384x32, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
     if n1 % 192 or n2 % 192:        # the LLaMA shard (5504 and 8192 columns): also the 256-wide tiles
         if batch > 512:
             tiles = tiles + [api.TILE.T256x256x32, api.TILE.T128x192x32_ALONE]
@@ -214,9 +215,9 @@ def tune_attention(seq, log, hidden=12288, heads=12):
     if seq <= 256:
         tiles = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T128x128x32]
     elif seq <= 1024:
-        tiles = [api.TILE.T128x192x32_ALONE, api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.T128x128x32]
+        tiles = [api.TILE.T128x192x32_ALONE, api.TILE.T128x192x32, api.TILE.T256x192x64, api.TILE.T256x192x32, api.TILE.T128x128x32]
     else:
-        tiles = [api.TILE.T128x192x32, api.TILE.T256x192x32, api.TILE.T128x192x32_ALONE]
+        tiles = [api.TILE.T128x192x32, api.TILE.T256x192x64, api.TILE.T256x384x32, api.TILE.T256x192x32, api.TILE.T128x192x32_ALONE]
     run(api.SYNC.STREAM)        # clocks up
     best1 = best3 = None
     for t in tiles:
