@@ -182,6 +182,10 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     else if (c.batch <= 512) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_D64x128x64; }
     else if (c.batch <= 1024) { a = CUSYNC_TILE_128x192x32_ALONE; b = CUSYNC_TILE_128x256x32; }
     else a = b = CUSYNC_TILE_256x256x32;
+    // From 257 rows on GEMM1 (K = 8192) takes the 256x192 tile whose K loop is assembly, in as many k-slices as fill
+    // the device (the chain under RowSync: 384 rows 106 -> 92 us, 512: 117 -> 103, 768: 166 -> 131, 1024: 176 -> 156,
+    // 1536: 236 -> 203, 2048: 263 -> 246; level at 256 rows).  Its last column tile is ragged (5504 = 28.7 x 192).
+    if (c.batch > 256 && c.hidden % 64 == 0) a = CUSYNC_TILE_256x192x64;
     *t1 = c.tile1 >= 0 ? c.tile1 : a;
     *t2 = c.tile2 >= 0 ? c.tile2 : b;
     if (c.one_launch && sync != CUSYNC_SYNC_STREAM && c.tile2 < 0) *t2 = *t1;
