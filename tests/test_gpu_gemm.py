@@ -253,7 +253,9 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
             assert L.cusync_rt_event_record(ev, s1) == 0
         assert api.gemm(prod, M, N, K, da.data_ptr(), K, db.data_ptr(), N, dc.data_ptr(), N, tile1, stream=s1,
                         max_workgroups=max_wg, split_k=split[0], workspace=ws[0].data_ptr()) == api.ERR.SUCCESS, api.last_error()
-        if host_hold:      # the host waits until every producer workgroup has started, then launches the consumer
+        if host_hold == "library":      # cusync_hold_back: the library picks the host-side hold or the wait kernel from the launch it just made
+            assert L.cusync_hold_back(C.byref(prod.desc), s2) == api.ERR.SUCCESS, api.last_error()
+        elif host_hold:      # the host waits until every producer workgroup has started, then launches the consumer
             assert L.cusync_wait_producer_started(C.byref(prod.desc), 0) == api.ERR.SUCCESS, api.last_error()
         else:
             assert prod.invokeWaitKernel(s2, after=ev if ordered else None) == api.ERR.SUCCESS
@@ -454,6 +456,40 @@ def test_chained_gemms_consumer_held_back_by_the_host(policy_kind):
     # a stage whose producer never ran: the host-side wait gives up after its time-out, nothing hangs
     st = api.Stage((2, 2, 1), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128))
     assert L.cusync_wait_producer_started(C.byref(st.desc), 50) == api.ERR.DEVICE and "did not all start" in api.last_error()
+    st.destroy()
+
+
+@pytest.mark.parametrize("shape", [(2048, 6144, 256, "fills"), (512, 768, 256, "leaves slots free")])
+def test_chained_gemms_held_back_by_the_library(shape):
+    # cusync_hold_back behind a producer launch that takes every workgroup slot (host-side hold) and behind one that
+    # does not (wait kernel): what CuStage::invokeWaitKernel and the chain handles call
+    M, N, K, what = shape
+    print("chained, cusync_hold_back,", what, flush=True)
+    tile = api.TILE.T256x192x64
+    L = _lib.load()
+    a, b, d, c, e, ps, cs, want_sems = chained(M, N, K, tile, tile, "row", iters=3, host_hold="library")
+    rows = [0, 255, 256, M - 1]
+    assert_close(c[rows], orc.gemm(np.ascontiguousarray(a[rows]), b), "C rows")
+    assert_close(e[rows], orc.gemm(np.ascontiguousarray(c[rows]), d), "E rows")
+    assert cs.spin_timeouts == 0 and np.array_equal(ps.sems, want_sems) and ps.kernel_executed == 3
+
+
+def test_hold_back_error_paths():
+    L = _lib.load()
+    cons = api.Stage((2, 2, 1), (1, 1, 1), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128), api.no_sync())
+    assert L.cusync_hold_back(C.byref(cons.desc), None) == api.ERR.NOT_PRODUCER
+    cons.destroy()
+    assert L.cusync_hold_back(None, None) == api.ERR.NOT_INITIALIZED
+    # AvoidWaitKernel: nothing to hold back
+    prod = api.Stage((2, 2, 1), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128), opts=api.OPT.AVOID_WAIT_KERNEL)
+    assert L.cusync_hold_back(C.byref(prod.desc), None) == api.ERR.SUCCESS
+    prod.destroy()
+    # a producer no launcher has run: no note of a launch that filled the device, so the wait kernel (which gives up
+    # by itself and is counted)
+    st = api.Stage((2, 2, 1), (1, 1, 1), api.no_sync(), api.tile_sync(api.ORDER.TRANSPOSE_XY, 128, 128))
+    assert L.cusync_hold_back(C.byref(st.desc), None) == api.ERR.SUCCESS
+    assert L.cusync_rt_device_sync() == 0, api.last_error()
+    assert st.read_state().spin_timeouts == 1
     st.destroy()
 
 

@@ -295,3 +295,27 @@ def test_mlp_run_reports_waits_that_gave_up():
     assert err.value.code == api.ERR.DEVICE and "3 wait(s) gave up" in str(err.value)
     mlp.run(dx.data_ptr(), dh.data_ptr(), dy.data_ptr(), runs=1)       # the count did not move again: fine
     mlp.destroy()
+
+
+@pytest.mark.parametrize("model,hidden,inner", [(api.MODEL.GPT3, 12288, 6144), (api.MODEL.LLAMA, 8192, 2752)])
+def test_mlp_choice_is_what_the_handle_takes(model, hidden, inner):
+    """cusync_mlp_choice (the tile table without a handle) against the tiles and k-slices of a handle made from the
+    same configuration, for every benchmark batch size and sync mode; explicit tiles and slices pass through."""
+    import ctypes as C
+    from cusync_amd import _lib
+    L = _lib.load()
+    _, _, dw1, dw2 = weights(model, hidden, inner)
+    for batch in (1, 16, 64, 256, 512, 1024, 1280, 2048):
+        for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE):
+            cfg = _lib.MlpConfig(model, batch, hidden, inner, sync, -1, -1, -1, 1, 0, 0, 0, 0, 0, 0, 0)
+            t1, t2, s1, s2 = C.c_int(-1), C.c_int(-1), C.c_int(-1), C.c_int(-1)
+            assert L.cusync_mlp_choice(C.byref(cfg), C.byref(t1), C.byref(t2), C.byref(s1), C.byref(s2)) == 0, api.last_error()
+            m = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr())
+            assert m.tiles() == (t1.value, t2.value) and m.splits() == (s1.value, s2.value), (batch, sync)
+            m.destroy()
+    cfg = _lib.MlpConfig(model, 512, hidden, inner, api.SYNC.ROW, api.TILE.T128x128x32, api.TILE.T128x256x32, -1, 1, 2, 1, 0, 0, 0, 0, 0)
+    t1, t2, s1, s2 = C.c_int(-1), C.c_int(-1), C.c_int(-1), C.c_int(-1)
+    assert L.cusync_mlp_choice(C.byref(cfg), C.byref(t1), C.byref(t2), C.byref(s1), C.byref(s2)) == 0
+    assert (t1.value, t2.value, s1.value, s2.value) == (api.TILE.T128x128x32, api.TILE.T128x256x32, 2, 1)
+    empty = _lib.MlpConfig(model, 0, hidden, inner, api.SYNC.ROW, -1, -1, -1, 1, 0, 0, 0, 0, 0, 0, 0)
+    assert L.cusync_mlp_choice(C.byref(empty), None, None, None, None) == 1 and "empty" in api.last_error()
