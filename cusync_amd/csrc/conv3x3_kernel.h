@@ -7,13 +7,15 @@
 // taps of output pixel m are input pixels m + (r-1)*W + (s-1): the 128 output
 // pixels of a tile need the contiguous run of 128 + 2W + 2 input pixels around
 // them.  That run (the tile plus its halo) is loaded into LDS once; the A
-// fragment of tap (r, s) is then an LDS read at a shifted pixel index, zeroed
-// for lanes whose tap falls outside the image (the flat neighbour would be a
-// pixel of the next row or the next image).  Only the filter is streamed, one
-// 64-channel chunk of one tap per step, through a ring of stages as in the
-// GEMM kernel; it is small and comes from L2.
+// fragment of tap (r, s) is then an LDS read at a shifted pixel index.  A lane
+// whose tap falls outside the image (the flat neighbour would be a pixel of the
+// next row or the next image) reads a pixel of zeros kept behind the run
+// instead: one select on the address per tap, none on the fragments.  Only the
+// filter is streamed, one 64-channel chunk of one tap per step, through a ring
+// of stages as in the GEMM kernel; it is small and comes from L2 (a deeper ring
+// measured the same: four and five stages against three on 28x28x128).
 //
-// LDS: [filter stages of BN x 64 halfs][halo: (BM + 2W + 2) pixels x C halfs].
+// LDS: [filter stages of BN x 64 halfs][halo: (BM + 2W + 2) pixels x C halfs][one pixel of zeros].
 // A pixel's 16-byte channel chunks are stored at chunk ^ (pixel & (C/8 - 1)),
 // so the 32 consecutive pixels an MFMA fragment reads fall on distinct banks.
 //
@@ -27,6 +29,11 @@
 namespace cusync {
 namespace gemm {
 
+// How many 16-channel products ahead of their use the fragments are read from LDS.  Measured on the ResNet pairs
+// (56x56x64 / 28x28x128 / 14x14x256, stream-ordered, us): the compiler's own order 41.0 / 51.1 / 68.3; one ahead
+// 39.9 / 48.6 / 63.8; two 39.7 / 49.4 / 65.2; the whole step up front 39.9 / 52.3 / 71.6.
+constexpr int kFragsAhead = 1;
+
 template<int BM_, int BN_, int WM_, int WN_, int STAGES_, int OCC_>
 struct Halo3x3Cfg {
   static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_, STAGES = STAGES_, OCC = OCC_;
@@ -39,7 +46,7 @@ struct Halo3x3Cfg {
   static_assert(WM * WN == 4 && B_CPR == 8 && B_LOADS >= 1, "four wavefronts, 64-channel filter chunks");
   // Bytes of LDS a launch needs for images of width W with C channels.
   static uint32_t ldsBytes(uint32_t W, uint32_t C) {
-    const uint32_t haloBytes = (BM + 2 * W + 2) * C * 2;
+    const uint32_t haloBytes = (BM + 2 * W + 3) * C * 2;      // the run of input pixels and one pixel of zeros behind it
     return B_BYTES + (haloBytes + 1023) / 1024 * 1024;
   }
 };
@@ -61,7 +68,8 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
   const uint32_t pixBytes = Cc * 2, cprMask = Cc / 8 - 1;             // C is a power of two
   const uint32_t pixShift = 31 - __builtin_clz(pixBytes);
   const uint32_t haloPix = C::BM + 2 * W + 2;
-  const uint32_t haloLoads = (haloPix * pixBytes + 1023) / 1024;       // 1 KiB pieces
+  const uint32_t haloLoads = ((haloPix + 1) * pixBytes + 1023) / 1024;       // 1 KiB pieces; pixel haloPix is the pixel of zeros
+  const uint32_t zeroPixel = haloPix << pixShift;
   const uint32_t chunksPerTap = Cc / C::BK, steps = 9 * chunksPerTap;
   const uint4v rA = rawRsrc(p.A, p.M * Cc * 2);
   const uint4v rB = rawRsrc(p.B, p.N * p.ldb * 2);
@@ -177,30 +185,34 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
       const int32_t shift = ((int32_t)(tap / 3) - 1) * (int32_t)W + (int32_t)(tap % 3) - 1;
       const char* sb = smem + (it % C::STAGES) * C::B_STAGE;
       uint32_t aBase[C::TM], aSwz[C::TM];
-      bool aLive[C::TM];
 #pragma unroll
       for (int i = 0; i < C::TM; i++) {
         const uint32_t pl = (uint32_t)((int32_t)(aPixel0 + i * 32) + shift);
-        aBase[i] = pl << pixShift;
-        aSwz[i] = pl & cprMask;
-        aLive[i] = (tapMask[i] >> tap) & 1;
+        aBase[i] = (tapMask[i] >> tap) & 1 ? pl << pixShift : zeroPixel;
+        aSwz[i] = pl & cprMask;      // any slot of the pixel of zeros will do
       }
+      // The fragments of 16 channels are requested kFragsAhead products of 16 channels before they are used.
+      half8 fb[C::KS][C::TN], fa[C::KS][C::TM];
+      auto readFrags = [&](int kk) {
 #pragma unroll
-      for (int kk = 0; kk < C::KS; kk++) {
-        half8 fb[C::TN], fa[C::TM];
-#pragma unroll
-        for (int j = 0; j < C::TN; j++) fb[j] = *reinterpret_cast<const half8*>(sb + bFrag[kk] + j * 32 * C::B_ROW_BYTES);
+        for (int j = 0; j < C::TN; j++) fb[kk][j] = *reinterpret_cast<const half8*>(sb + bFrag[kk] + j * 32 * C::B_ROW_BYTES);
 #pragma unroll
         for (int i = 0; i < C::TM; i++) {
           const uint32_t chunk = cc * (C::BK / 8) + 2 * kk + hi;
-          fa[i] = *reinterpret_cast<const half8*>(halo + aBase[i] + ((chunk ^ aSwz[i]) << 4));
-          if (!aLive[i]) fa[i] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+          fa[kk][i] = *reinterpret_cast<const half8*>(halo + aBase[i] + ((chunk ^ aSwz[i]) << 4));
         }
+      };
+#pragma unroll
+      for (int kk = 0; kk < kFragsAhead && kk < C::KS; kk++) readFrags(kk);
+#pragma unroll
+      for (int kk = 0; kk < C::KS; kk++) {
+        __builtin_amdgcn_sched_barrier(0);      // left alone, the compiler issues each read two MFMAs before its use
+        if (kk + kFragsAhead < C::KS) readFrags(kk + kFragsAhead);
 #pragma unroll
         for (int i = 0; i < C::TM; i++)
 #pragma unroll
           for (int j = 0; j < C::TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
       }
     }
 

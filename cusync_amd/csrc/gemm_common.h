@@ -277,7 +277,6 @@ struct TileStore {
     constexpr int PITCH = C::BN * 2 + 16;
     constexpr int ROWS = C::WM * 32;
     constexpr int CPR = C::BN / 8;
-    constexpr int STEPS = ROWS * CPR / C::THREADS;
     static_assert(ROWS * PITCH <= C::LDS_BYTES, "epilogue buffer fits the pipeline stages");
     static_assert((ROWS * CPR) % C::THREADS == 0, "whole copy steps");
     __syncthreads();       // the buffer is free: main-loop reads, or the previous pass, are done
@@ -418,7 +417,7 @@ __device__ __forceinline__ bool finishTileSplit(const GemmParams& p, floatx16 (&
   constexpr uint32_t kPieceBytes = C::WN * C::TN * 4 * 1024;                    // 32 rows x BN columns of fp32
   const uint32_t perSlice = C::BM >= 128 && p.coopReduce ? kPieces / p.splitK : 0;
   const bool ownInLds = C::BM >= 128 && p.coopReduce && kEpiBytes + perSlice * kPieceBytes <= (uint32_t)C::LDS_BYTES;
-  auto ownedPiece = [&](int i) { return ((uint32_t)i * C::WM + (uint32_t)wm) / perSlice == t.z; };      // uniform per wavefront
+  auto ownedPiece = [&](int i) { return ((uint32_t)i * C::WM + (uint32_t)wm) / (perSlice ? perSlice : 1u) == t.z; };      // uniform per wavefront; asked under the shared reduction only
   auto ownSlot = [&](int i, int j, int g) {
     const uint32_t o = (uint32_t)i * C::WM + (uint32_t)wm - t.z * perSlice;
     return lds + kEpiBytes + ((o * C::WN + (uint32_t)wn) * (C::TN * 4) + (uint32_t)(j * 4 + g)) * 1024 + (uint32_t)lane * 16;

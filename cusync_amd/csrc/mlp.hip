@@ -349,7 +349,6 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->ldh = m->n1;
   m->w1p = m->w2p = nullptr;
   m->ldw1 = m->n1; m->ldw2 = m->n2;
-  const bool swiglu = llama && cfg->activation;
   Choice ch;
   if (!choose(*cfg, &ch)) { discard(m); return nullptr; }
   m->fused = ch.fused;
