@@ -151,7 +151,7 @@ SIGNATURES = {
     "cusync_mlp_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
     "cusync_mlp_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cusync_mlp_splits": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
-    "cusync_mlp_choice": (C.c_int, [C.POINTER(MlpConfig), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "cusync_mlp_choice": (C.c_int, [C.POINTER(MlpConfig)] + [C.POINTER(C.c_int)] * 5),
 }
 
 _lib = None

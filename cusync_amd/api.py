@@ -378,7 +378,8 @@ class Mlp:
     """Handle over cusync_mlp_* (the reference's libmlp C surface, src/ml-bench/transformer/mlp-lib.cu:555-618)."""
 
     def __init__(self, model, batch, hidden, inner, sync, w1_ptr, w2_ptr, tile1=-1, tile2=-1, opts=-1, activation=1,
-                 split_k1=0, split_k2=0, max_wg1=0, max_wg2=0, one_launch=False, swiglu_in_gemm2=0, repack_weights=False):
+                 split_k1=0, split_k2=0, max_wg1=0, max_wg2=0, one_launch=-1, swiglu_in_gemm2=0, repack_weights=False):
+        """one_launch: True / False, or -1 for the library's choice by model and batch size (see choice())."""
         self.L = _lib.load()
         self.cfg = MlpConfig(model, batch, hidden, inner, sync, tile1, tile2, opts, activation, split_k1, split_k2,
                              max_wg1, max_wg2, int(one_launch), int(swiglu_in_gemm2), int(repack_weights))
@@ -416,6 +417,13 @@ class Mlp:
             return list(times), list(g1), list(g2)
         check(self.L.cusync_mlp_run(self.h, x_ptr, h_ptr, y_ptr, runs, times), "cusync_mlp_run")
         return list(times)
+
+    def choice(self):
+        """(tile1, tile2, split_k1, split_k2, one_launch) the tile table gives for this handle's configuration."""
+        v = [C.c_int(-1) for _ in range(5)]
+        if self.L.cusync_mlp_choice(C.byref(self.cfg), *[C.byref(x) for x in v]) != 0:
+            raise RuntimeError("cusync_mlp_choice failed: " + last_error())
+        return tuple(x.value for x in v)
 
     def tiles(self):
         a, b = C.c_int(0), C.c_int(0)

@@ -305,9 +305,25 @@ void discard(cusync_mlp* m) {
 
 // What a handle for `c` runs with: where the activation is computed, the sync mode after the StridedSync
 // substitution, tiles and k-slices.  False (with the error text set) for a configuration no handle can be made of.
-struct Choice { bool fused, actStage; int aMode2, sync, tile1, tile2, split1, split2; };
-bool choose(const cusync_mlp_config& c, Choice* o) {
+struct Choice { bool fused, actStage, oneLaunch; int aMode2, sync, tile1, tile2, split1, split2; };
+
+// Both GEMMs in one launch need the same direct-to-LDS tile for both and a plain A operand in GEMM2.
+bool oneLaunchPossible(const Choice& o) {
+  uint32_t bk = 0;
+  if (cusync_gemm_tile_shape(o.tile1, nullptr, nullptr, &bk)) return false;
+  const bool direct = bk == 32 || o.tile1 >= CUSYNC_TILE_D32x128x64;      // the direct-to-LDS tiles
+  return o.tile1 == o.tile2 && direct && o.aMode2 == CUSYNC_A_PLAIN && !o.actStage;
+}
+
+bool choose(const cusync_mlp_config& given, Choice* o) {
+  cusync_mlp_config c = given;
   const bool llama = c.model == CUSYNC_MLP_LLAMA;
+  // one_launch < 0: where one launch measured ahead of two on the GPT-3 shard (1 to 64 rows under either policy:
+  // 1-5 us of 67-83; 512 to 1024 rows: 1-3 us of 172-284; behind at 256 rows and from 1025 on, and at every size of
+  // the LLaMA shard, whose GEMM2 wants a tile of its own) and the tiles are the table's
+  const bool automatic = c.one_launch < 0;
+  if (automatic) c.one_launch = c.sync != CUSYNC_SYNC_STREAM && !llama && c.tile1 < 0 && c.tile2 < 0 &&
+                                (c.batch <= 64 || (c.batch >= 512 && c.batch <= 1024));
   const uint32_t k1 = c.hidden, n1 = llama ? 2 * c.inner : c.inner, k2 = c.inner, n2 = c.hidden;
   const bool swiglu = llama && c.activation;
   // where silu(gate) * up is computed: 2 = GEMM1's epilogue (the built-in choice), -1 = a stage of its own, 1 = GEMM2's A loader
@@ -319,6 +335,16 @@ bool choose(const cusync_mlp_config& c, Choice* o) {
   o->sync = c.sync;
   if (swiglu && !o->fused && o->sync == CUSYNC_SYNC_TILE && c.inner % 128 == 0) o->sync = CUSYNC_SYNC_STRIDED;
   pickTiles(c, o->sync, o->aMode2 == CUSYNC_A_SWIGLU, o->fused, &o->tile1, &o->tile2);
+  o->oneLaunch = c.one_launch && o->sync != CUSYNC_SYNC_STREAM;
+  if (o->oneLaunch && !oneLaunchPossible(*o)) {
+    if (!automatic) {
+      setError("mlp: one launch for both GEMMs needs the same direct-to-LDS tile for both and a plain A operand");
+      return false;
+    }
+    c.one_launch = 0;
+    o->oneLaunch = false;
+    pickTiles(c, o->sync, o->aMode2 == CUSYNC_A_SWIGLU, o->fused, &o->tile1, &o->tile2);
+  }
   uint32_t bk1 = 0, bk2 = 0;
   if (cusync_gemm_tile_shape(o->tile1, nullptr, nullptr, &bk1) || cusync_gemm_tile_shape(o->tile2, nullptr, nullptr, &bk2)) {
     setError("mlp: unknown tile id");
@@ -351,6 +377,7 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
   m->ldw1 = m->n1; m->ldw2 = m->n2;
   Choice ch;
   if (!choose(*cfg, &ch)) { discard(m); return nullptr; }
+  m->cfg.one_launch = ch.oneLaunch;      // settled: the run asks this copy
   m->fused = ch.fused;
   m->actStage = ch.actStage;
   m->aMode2 = ch.aMode2;
@@ -423,16 +450,6 @@ cusync_mlp* cusync_mlp_create(const cusync_mlp_config* cfg, const void* w1, cons
       return nullptr;
   }
   if (cfg->opts >= 0) opts |= cfg->opts;
-  if (cfg->one_launch && sync != CUSYNC_SYNC_STREAM) {
-    uint32_t bk = 0;
-    cusync_gemm_tile_shape(m->tile1, nullptr, nullptr, &bk);
-    const bool direct = bk == 32 || m->tile1 >= CUSYNC_TILE_D32x128x64;      // the direct-to-LDS tiles
-    if (m->tile1 != m->tile2 || !direct || m->aMode2 != CUSYNC_A_PLAIN || m->actStage) {
-      setError("mlp: one launch for both GEMMs needs the same direct-to-LDS tile for both and a plain A operand");
-      discard(m);
-      return nullptr;
-    }
-  }
 
   // the edge into GEMM2 when the activation is a stage of its own: its 128 x 128 tiles under the same kind of policy
   cusync_policy_desc pol2 = pol;
@@ -619,7 +636,7 @@ int cusync_mlp_splits(const cusync_mlp* m, int* split_k1, int* split_k2) {
   return 0;
 }
 
-int cusync_mlp_choice(const cusync_mlp_config* cfg, int* tile1, int* tile2, int* split_k1, int* split_k2) {
+int cusync_mlp_choice(const cusync_mlp_config* cfg, int* tile1, int* tile2, int* split_k1, int* split_k2, int* one_launch) {
   if (!cfg || cfg->batch == 0 || cfg->hidden == 0 || cfg->inner == 0) { setError("mlp: empty shape"); return 1; }
   Choice ch;
   if (!choose(*cfg, &ch)) return 1;
@@ -627,6 +644,7 @@ int cusync_mlp_choice(const cusync_mlp_config* cfg, int* tile1, int* tile2, int*
   if (tile2) *tile2 = ch.tile2;
   if (split_k1) *split_k1 = ch.split1;
   if (split_k2) *split_k2 = ch.split2;
+  if (one_launch) *one_launch = ch.oneLaunch;
   return 0;
 }
 

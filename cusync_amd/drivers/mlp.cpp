@@ -6,7 +6,8 @@
 //       [--repack-weights true|false] [--one-launch true|false]
 //
 // --repack-weights: both chains read padded copies of the weights kept by the handle
-// (cusync_mlp_config.repack_weights); --one-launch: the CuSync chain runs both GEMMs in one launch.
+// (cusync_mlp_config.repack_weights); --one-launch: the CuSync chain runs both GEMMs in one launch (true), in one
+// launch each (false), or, when the option is not given, as the library's table says for the batch size.
 //
 // Output: "START-BASELINE:", one JSON object per timed run {"Total", "matmul1Time", "matmul2Time"} in
 // microseconds, "END-BASELINE:", then the same between START-OVERLAPPED: / END-OVERLAPPED: with {"Total"}
@@ -52,7 +53,7 @@ int main(int argc, char** argv) {
     c.activation = llama ? 0 : 1;        // the reference's LLaMA chain multiplies the gate half as is (mlp.cu:785-792)
     c.split_k1 = (int)drv::getInt(args, "split-k1", 0); c.split_k2 = (int)drv::getInt(args, "split-k2", 0);
     c.repack_weights = drv::getBool(args, "repack-weights", false) ? 1 : 0;
-    c.one_launch = (mode != CUSYNC_SYNC_STREAM && drv::getBool(args, "one-launch", false)) ? 1 : 0;
+    c.one_launch = mode == CUSYNC_SYNC_STREAM ? 0 : !args.count("one-launch") ? -1 : drv::getBool(args, "one-launch", false) ? 1 : 0;      // not given: the library picks
     cusync_mlp* m = cusync_mlp_create(&c, w1, w2);
     if (!m) { fprintf(stderr, "cusync_mlp_create failed: %s\n", cusync_rt_last_error()); exit(EXIT_FAILURE); }
     DRV_CHECK(cusync_mlp_run(m, x, h, y, warmup, nullptr));

@@ -271,7 +271,7 @@ int main(int argc, char** argv) {
       int tile1 = 0, tile2 = 0;
       Request rq;
       rq.row = row;
-      if (cusync_mlp_choice(&c, &tile1, &tile2, &rq.split_k1, &rq.split_k2) != 0) { fprintf(stderr, "no shapes for %d rows: %s\n", batch, cusync_rt_last_error()); return EXIT_FAILURE; }
+      if (cusync_mlp_choice(&c, &tile1, &tile2, &rq.split_k1, &rq.split_k2, nullptr) != 0) { fprintf(stderr, "no shapes for %d rows: %s\n", batch, cusync_rt_last_error()); return EXIT_FAILURE; }
       rq.runs = (int)drv::getInt(args, "runs", 20); rq.rounds = (int)drv::getInt(args, "rounds", 1); rq.warmup = 10;
       rq.withHandle = drv::getBool(args, "handle", true);
 

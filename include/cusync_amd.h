@@ -488,7 +488,9 @@ typedef struct cusync_mlp_config {
                                   the launch fills the device */
   int32_t max_wg1, max_wg2;    /* workgroups per launch of each GEMM; 0 = built-in choice, -1 = as many as stay resident */
   int32_t one_launch;          /* 1 (with a CuSync mode): both GEMMs in one launch, cusync_gemm_chain_run; needs the same
-                                  direct-to-LDS tile for both and a plain A operand in GEMM2 */
+                                  direct-to-LDS tile for both and a plain A operand in GEMM2.  0: one launch per GEMM on
+                                  two streams, as the reference runs them.  -1: whichever measured faster for this
+                                  model and batch size with the table's tiles (cusync_mlp_choice reports it) */
   int32_t swiglu_in_gemm2;     /* LLaMA with activation: where silu(gate)*up is computed.
                                   2: in GEMM1's epilogue (CUSYNC_EPILOGUE_SWIGLU).  create() copies w1 into a buffer of its
                                   own with the gate and up columns interleaved in groups of eight (call
@@ -537,11 +539,11 @@ cusync_error cusync_mlp_run_split(cusync_mlp *mlp, const void *x, void *h, void 
 /* Device state of the two stages for tests (see cusync_stage_read_state). */
 const cusync_stage_desc *cusync_mlp_stage(const cusync_mlp *mlp, int which /* 0 producer (GEMM1), 1 consumer (GEMM2), 2 the activation stage or NULL */);
 int cusync_mlp_tiles(const cusync_mlp *mlp, int *tile1, int *tile2);
-/* The tile table without a handle: the tiles and k-slices cusync_mlp_create would take for `cfg` on this device
- * (fields < 0 / 0 in cfg mean "choose", as there).  What a driver that wires its own stages and launchers looks
+/* The tile table without a handle: the tiles, k-slices and number of launches (*one_launch 1 or 0)
+ * cusync_mlp_create would take for `cfg` on this device (fields < 0 / 0 in cfg mean "choose", as there).  What a driver that wires its own stages and launchers looks
  * up per batch size, as the reference's build looks its shapes up in src/ml-bench/transformer/tile_sizes_db.py.
  * Returns 0, or 1 with cusync_rt_last_error() set. */
-int cusync_mlp_choice(const cusync_mlp_config *cfg, int *tile1, int *tile2, int *split_k1, int *split_k2);
+int cusync_mlp_choice(const cusync_mlp_config *cfg, int *tile1, int *tile2, int *split_k1, int *split_k2, int *one_launch);
 int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
 
 /* ------------------------------------------------------------------------- */

@@ -300,22 +300,33 @@ def test_mlp_run_reports_waits_that_gave_up():
 @pytest.mark.parametrize("model,hidden,inner", [(api.MODEL.GPT3, 12288, 6144), (api.MODEL.LLAMA, 8192, 2752)])
 def test_mlp_choice_is_what_the_handle_takes(model, hidden, inner):
     """cusync_mlp_choice (the tile table without a handle) against the tiles and k-slices of a handle made from the
-    same configuration, for every benchmark batch size and sync mode; explicit tiles and slices pass through."""
+    same configuration, for every benchmark batch size and sync mode; explicit tiles and slices pass through; the
+    number of launches is the table's where the configuration leaves it open (one_launch = -1)."""
     import ctypes as C
     from cusync_amd import _lib
     L = _lib.load()
     _, _, dw1, dw2 = weights(model, hidden, inner)
+
+    def choice(cfg):
+        v = [C.c_int(-1) for _ in range(5)]
+        assert L.cusync_mlp_choice(C.byref(cfg), *[C.byref(x) for x in v]) == 0, api.last_error()
+        return tuple(x.value for x in v)
+
     for batch in (1, 16, 64, 256, 512, 1024, 1280, 2048):
         for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE):
-            cfg = _lib.MlpConfig(model, batch, hidden, inner, sync, -1, -1, -1, 1, 0, 0, 0, 0, 0, 0, 0)
-            t1, t2, s1, s2 = C.c_int(-1), C.c_int(-1), C.c_int(-1), C.c_int(-1)
-            assert L.cusync_mlp_choice(C.byref(cfg), C.byref(t1), C.byref(t2), C.byref(s1), C.byref(s2)) == 0, api.last_error()
-            m = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr())
-            assert m.tiles() == (t1.value, t2.value) and m.splits() == (s1.value, s2.value), (batch, sync)
-            m.destroy()
-    cfg = _lib.MlpConfig(model, 512, hidden, inner, api.SYNC.ROW, api.TILE.T128x128x32, api.TILE.T128x256x32, -1, 1, 2, 1, 0, 0, 0, 0, 0)
-    t1, t2, s1, s2 = C.c_int(-1), C.c_int(-1), C.c_int(-1), C.c_int(-1)
-    assert L.cusync_mlp_choice(C.byref(cfg), C.byref(t1), C.byref(t2), C.byref(s1), C.byref(s2)) == 0
-    assert (t1.value, t2.value, s1.value, s2.value) == (api.TILE.T128x128x32, api.TILE.T128x256x32, 2, 1)
+            for one in (-1, 0):
+                m = api.Mlp(model, batch, hidden, inner, sync, dw1.data_ptr(), dw2.data_ptr(), one_launch=one)
+                got = choice(m.cfg)
+                assert m.choice() == got
+                assert m.tiles() == got[:2] and m.splits() == got[2:4], (batch, sync)
+                in_one = one == -1 and model == api.MODEL.GPT3 and sync != api.SYNC.STREAM and (batch <= 64 or 512 <= batch <= 1024)
+                assert got[4] == int(in_one), (batch, sync, one, got)
+                if in_one:
+                    assert got[0] == got[1]
+                m.destroy()
+    cfg = _lib.MlpConfig(model, 512, hidden, inner, api.SYNC.ROW, api.TILE.T128x128x32, api.TILE.T128x256x32, -1, 1, 2, 1, 0, 0, -1, 0, 0)
+    assert choice(cfg) == (api.TILE.T128x128x32, api.TILE.T128x256x32, 2, 1, 0)      # the caller's tiles: two launches
+    cfg.one_launch = 1
+    assert L.cusync_mlp_choice(C.byref(cfg), None, None, None, None, None) == 1 and "one launch" in api.last_error()
     empty = _lib.MlpConfig(model, 0, hidden, inner, api.SYNC.ROW, -1, -1, -1, 1, 0, 0, 0, 0, 0, 0, 0)
-    assert L.cusync_mlp_choice(C.byref(empty), None, None, None, None) == 1 and "empty" in api.last_error()
+    assert L.cusync_mlp_choice(C.byref(empty), None, None, None, None, None) == 1 and "empty" in api.last_error()
