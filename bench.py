@@ -186,6 +186,16 @@ def main():
         def close(self):
             self.m.destroy()
 
+    def default_one_launch(batch, sync):
+        """Whether the tile table runs this batch size in one launch when the caller leaves it open."""
+        import ctypes
+        from cusync_amd import _lib
+        cfg = _lib.MlpConfig(api.MODEL.GPT3, batch, HIDDEN, INNER, sync, args.tile1, args.tile2, -1, 1, 0, 0, 0, 0, -1, 0, 0)
+        one = ctypes.c_int(0)
+        if _lib.load().cusync_mlp_choice(ctypes.byref(cfg), None, None, None, None, ctypes.byref(one)) != 0:
+            raise RuntimeError("cusync_mlp_choice: " + api.last_error())
+        return bool(one.value)
+
     def interleaved(chains, warm, timed, split_first=False):
         """Runs the chains in turn, one step each per round: `warm` untimed rounds, then `timed` rounds.  Returns
         one list of step times per chain (for the first chain, with split_first, triples: step, GEMM1, GEMM2)."""
@@ -389,6 +399,8 @@ def main():
                 names.append("rowsync_one_launch_rp")
                 chains.append(Chain(b, api.SYNC.ROW, one_launch=True, repack=True))
             times = interleaved(chains, 10, 20, split_first=True)
+            # what a handle left to itself (one_launch = -1) runs under each policy: one launch or two
+            default_one = {k: default_one_launch(b, sy) for k, sy in (("rowsync", api.SYNC.ROW), ("tilesync", api.SYNC.TILE))}
             for c in chains:
                 c.close()
             t = dict(zip(names, times))
@@ -410,6 +422,10 @@ def main():
                 "rowsync_one_launch_us": round(m["rowsync_one_launch"][0], 2) if "rowsync_one_launch" in m else None,
                 "tilesync_one_launch_us": round(m["tilesync_one_launch"][0], 2) if "tilesync_one_launch" in m else None,
                 "one_launch_tiles": one_tiles,
+                # the mode the handle picks by itself (cusync_mlp_config.one_launch = -1) and its time from the columns above
+                "default_launches": {k: 1 if v else 2 for k, v in default_one.items()},
+                "rowsync_default_us": round(m["rowsync_one_launch" if default_one["rowsync"] and "rowsync_one_launch" in m else "rowsync"][0], 2),
+                "tilesync_default_us": round(m["tilesync_one_launch" if default_one["tilesync"] and "tilesync_one_launch" in m else "tilesync"][0], 2),
                 # medians of 60 steps in the driver's process: the launcher objects' loop, and the handle beside it there
                 "launcher_rowsync_us": launcher[(b, "rowsync")]["launcher_us"], "launcher_tilesync_us": launcher[(b, "tilesync")]["launcher_us"],
                 "launcher_vs_handle_pct": {k: round(launcher[(b, k)]["launcher_us"] / launcher[(b, k)]["handle_us"] * 100 - 100, 2)
