@@ -525,7 +525,12 @@ def main():
 
         # cost of the synchronisation itself (src/examples/sync-overhead/sync-overhead.cu and a ping-pong)
         with_sync, without = api.sync_overhead_pair(1280, 128, warmup=10, iters=100)
+        bare_with, bare_without = api.sync_overhead_bare(1280, 128, warmup=10, iters=100)
         other["sync_overhead"] = {
+            # the example's own kernels: a bare flag per block, no fences, one stream (what its percentage measures)
+            "bare_flags_with_us": round(bare_with, 2), "bare_flags_without_us": round(bare_without, 2),
+            "bare_flags_overhead_pct": round((bare_with - bare_without) / bare_without * 100, 1),
+            # the public CuStage tile/post/wait on two streams with the wait kernel: what a chain pays
             "pair_with_sync_us": round(with_sync, 2), "pair_without_sync_us": round(without, 2),
             "pair_overhead_pct": round((with_sync - without) / without * 100, 1),
             "handover_ns_same_xcd": round(api.sync_overhead_pingpong(8) / 2, 1),

@@ -141,6 +141,7 @@ SIGNATURES = {
     "cusync_attn_layer_stage": (C.POINTER(StageDesc), [vp, C.c_int]),
     "cusync_attn_layer_tiles": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cusync_sync_overhead_pair": (C.c_int, [u32, u32, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "cusync_sync_overhead_bare": (C.c_int, [u32, u32, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_sync_overhead_pingpong": (C.c_int, [u32, u32, C.POINTER(C.c_double)]),
     "cusync_probe_mfma_rate": (C.c_int, [C.c_int, u32, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_mlp_create": (vp, [C.POINTER(MlpConfig), vp, vp]),

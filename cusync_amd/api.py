@@ -358,6 +358,14 @@ def sync_overhead_pair(blocks=1280, threads=128, warmup=10, iters=100):
     return a.value, b.value
 
 
+def sync_overhead_bare(blocks=1280, threads=128, warmup=10, iters=100):
+    """(with_flags_us, without_flags_us) of the same pair with the example's own kernels: a bare flag array, no fences,
+    both kernels on one stream (src/examples/sync-overhead/sync-overhead.cu:40-59, 84-101)."""
+    a, b = C.c_double(0), C.c_double(0)
+    check(_lib.load().cusync_sync_overhead_bare(blocks, threads, warmup, iters, C.byref(a), C.byref(b)), "sync_overhead_bare")
+    return a.value, b.value
+
+
 def probe_mfma_rate(random_data=True, iters=2000, launches=10):
     """(TFLOP/s, shader clock in MHz) the matrix pipes sustain alone, on zero or random register operands."""
     t, f = C.c_double(0), C.c_double(0)

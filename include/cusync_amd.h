@@ -558,6 +558,12 @@ int cusync_mlp_splits(const cusync_mlp *mlp, int *split_k1, int *split_k2);
  * given up; otherwise CUSYNC_ERROR_DEVICE with the count in cusync_rt_last_error(). */
 cusync_error cusync_sync_overhead_pair(uint32_t blocks, uint32_t threads, int warmup, int iters,
                                        double *with_sync_us, double *without_sync_us);
+/* The same experiment with the example's own kernels (sync-overhead.cu:40-59, 84-101): the producer's first thread
+ * adds one to its block's word of a bare flag array behind a barrier, the consumer's first thread polls word 0, no
+ * fences, no tile order, both kernels on ONE stream, so that the flags are up when the consumer starts: the cost of
+ * touching the flags, which is what the example's percentage measures.  Same checks as above. */
+cusync_error cusync_sync_overhead_bare(uint32_t blocks, uint32_t threads, int warmup, int iters,
+                                       double *with_flags_us, double *without_flags_us);
 /* Latency of a post -> wait hand-over: workgroup 0 and workgroup `partner` (1..63) of one launch pass a
  * semaphore back and forth `rounds` times.  Workgroups go to the eight XCDs round-robin, so partner 8 shares
  * workgroup 0's XCD and partner 1 does not.  No counterpart in the reference, whose GPUs have one L2. */

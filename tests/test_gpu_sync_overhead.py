@@ -47,3 +47,15 @@ def test_mfma_rate_probe():
         assert 300.0 < tf < 2700.0            # cannot exceed the published dense rate
         assert 400.0 < mhz < 2700.0
     assert zero_tf > 0.9 * rand_tf
+
+
+def test_sync_overhead_with_the_examples_own_kernels():
+    # bare flag array, one stream (sync-overhead.cu:40-59, 84-101); the call checks the consumer's output itself
+    print("sync overhead, bare flags", flush=True)
+    with_flags, without = api.sync_overhead_bare(1280, 128, warmup=5, iters=30)
+    print("bare flags: with %.1f us, without %.1f us" % (with_flags, without))
+    assert 0 < without < 1e4 and 0 < with_flags < 1e4
+    for blocks, threads in ((1, 64), (300, 1024)):
+        api.sync_overhead_bare(blocks, threads, warmup=1, iters=3)
+    with pytest.raises(api.CuSyncError):
+        api.sync_overhead_bare(0, 128)
