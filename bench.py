@@ -338,7 +338,9 @@ def main():
     if args.profile_chain == "conv":
         g = torch.Generator(device="cuda").manual_seed(4)
         rows = []
-        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128)):
+        # the two pairs of the benchmark set, then the two deep layers of the reference's table
+        # (src/ml-bench/volta_conv2d/resnet_results.csv: 256 and 512 channels), whose few tiles the chain cuts into runs
+        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128), (32, 14, 14, 256), (32, 7, 7, 512)):
             xc = (torch.rand((n, hh, ww, cc), device="cuda", generator=g) * 2 - 1).half()
             ws = [(torch.randn((cc, 3, 3, cc), device="cuda", generator=g) * (2.0 / (9 * cc)) ** 0.5).half() for _ in range(2)]
             ys = [torch.empty((n, hh, ww, cc), dtype=torch.float16, device="cuda") for _ in range(2)]
@@ -502,7 +504,9 @@ def main():
             row["best_tflops"] = round(2.0 * b * lh * 3 * li / best / 1e6, 1)
             other["llama_mlp"].append(row)
         other["conv_pair"] = []
-        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128)):
+        # the two pairs of the benchmark set, then the two deep layers of the reference's table
+        # (src/ml-bench/volta_conv2d/resnet_results.csv: 256 and 512 channels), whose few tiles the chain cuts into runs
+        for n, hh, ww, cc in ((32, 56, 56, 64), (32, 28, 28, 128), (32, 14, 14, 256), (32, 7, 7, 512)):
             xc = (torch.rand((n, hh, ww, cc), device="cuda", generator=g) * 2 - 1).half()
             ws = [(torch.randn((cc, 3, 3, cc), device="cuda", generator=g) * (2.0 / (9 * cc)) ** 0.5).half() for _ in range(2)]
             ys = [torch.empty((n, hh, ww, cc), dtype=torch.float16, device="cuda") for _ in range(2)]
@@ -518,6 +522,8 @@ def main():
                     sys.exit("bench.py: convolution chain waits timed out — results invalid")
                 row[name + "_us"] = round(trimmed(tt)[0], 2)
                 row["tile"] = ch.tile()
+                if name == "stream":
+                    row["runs_per_tile"] = ch.split()
                 ch.destroy()
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "rowsync_one_launch_us", "tilesync_one_launch_us"))
             row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)

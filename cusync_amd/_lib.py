@@ -46,12 +46,12 @@ class GemmArgs(C.Structure):
 class Conv2dArgs(C.Structure):
     _fields_ = [("stage", StageDesc), ("N", u32), ("H", u32), ("W", u32), ("C", u32), ("K", u32), ("R", u32), ("S", u32),
                 ("pad", u32), ("stride", u32), ("x", vp), ("w", vp), ("y", vp),
-                ("epilogue", i32), ("tile", i32), ("max_workgroups", i32)]
+                ("epilogue", i32), ("tile", i32), ("max_workgroups", i32), ("split_k", i32), ("workspace", vp)]
 
 
 class ConvChainConfig(C.Structure):
     _fields_ = [("N", u32), ("H", u32), ("W", u32), ("C", u32), ("layers", u32), ("sync", i32), ("tile", i32),
-                ("opts", i32), ("relu", i32), ("fused", i32)]
+                ("opts", i32), ("relu", i32), ("fused", i32), ("split_k", i32)]
 
 
 class AttentionArgs(C.Structure):
@@ -120,6 +120,8 @@ SIGNATURES = {
     "cusync_gemm_run_static_workspace": (C.c_int, [C.POINTER(GemmArgs), vp]),
     "cusync_conv2d_tile_shape": (C.c_int, [C.c_int, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_conv2d_grid": (Dim3, [C.c_int, u32, u32, u32, u32, u32, u32, u32, u32]),
+    "cusync_conv2d_grid_split": (Dim3, [C.c_int, u32, u32, u32, u32, u32, u32, u32, u32, C.c_int]),
+    "cusync_conv2d_workspace_size": (sz, [C.POINTER(Conv2dArgs)]),
     "cusync_conv2d_can_implement": (C.c_int, [C.POINTER(Conv2dArgs)]),
     "cusync_conv2d_max_resident": (C.c_int, [C.c_int]),
     "cusync_conv2d_run": (C.c_int, [C.POINTER(Conv2dArgs), vp]),
@@ -128,6 +130,7 @@ SIGNATURES = {
     "cusync_conv_chain_run": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "cusync_conv_chain_stage": (C.POINTER(StageDesc), [vp, u32]),
     "cusync_conv_chain_tile": (C.c_int, [vp]),
+    "cusync_conv_chain_split": (C.c_int, [vp]),
     "cusync_attention_tile_shape": (C.c_int, [C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "cusync_attention_grid": (Dim3, [u32, u32]),
     "cusync_attention_grid_split": (Dim3, [u32, u32, u32, u32]),

@@ -20,7 +20,7 @@ EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2, SWIGLU=3)
 TILE = SimpleNamespace(T256x256x32=0, T256x128x64=1, T128x128x64=2, T64x128x64=3, T32x128x64=4,
                        T128x256x64=5, T256x64x64=6, T128x64x64=7, T256x128x32=8, T128x256x32=9, T128x128x32=10,
                        T128x192x32=11, T256x192x32=12, D32x128x64=13, D64x128x64=14, D64x192x64=15, T128x192x32_ALONE=16, T256x384x32=17, T256x192x64=18, COUNT=19)
-CONV_TILE = SimpleNamespace(T128x64x32=0, T128x128x32=1, T256x64x32=2, HALO_256x64x64=3, HALO_128x128x64=4, COUNT=5)
+CONV_TILE = SimpleNamespace(T128x64x32=0, T128x128x32=1, T256x64x32=2, HALO_256x64x64=3, HALO_128x128x64=4, HALO_64x128x64=5, COUNT=6)
 SYNC = SimpleNamespace(STREAM=0, ROW=1, TILE=2, STRIDED=3)
 MODEL = SimpleNamespace(GPT3=0, LLAMA=1)
 
@@ -211,17 +211,26 @@ def conv2d_tile_shape(tile):
     return m.value, n.value, k.value
 
 
-def conv2d_grid(tile, N, H, W, K, R=3, S=3, pad=1, stride=1):
-    return _lib.load().cusync_conv2d_grid(tile, N, H, W, K, R, S, pad, stride).tup()
+def conv2d_grid(tile, N, H, W, K, R=3, S=3, pad=1, stride=1, split_k=1):
+    return _lib.load().cusync_conv2d_grid_split(tile, N, H, W, K, R, S, pad, stride, split_k).tup()
 
 
-def conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, R=3, S=3, pad=1, stride=1, epilogue=EPI.NONE, max_workgroups=0):
+def conv2d_args(stage, N, H, W, Cc, K, x, w, y, tile, R=3, S=3, pad=1, stride=1, epilogue=EPI.NONE, max_workgroups=0,
+                split_k=1, workspace=None):
     a = Conv2dArgs()
     a.stage = stage.desc
     a.N, a.H, a.W, a.C, a.K, a.R, a.S, a.pad, a.stride = N, H, W, Cc, K, R, S, pad, stride
     a.x, a.w, a.y = x, w, y
     a.epilogue, a.tile, a.max_workgroups = epilogue, tile, max_workgroups
+    a.split_k, a.workspace = split_k, workspace
     return a
+
+
+def conv2d_workspace_size(N, H, W, Cc, K, tile, split_k, R=3, S=3, pad=1, stride=1):
+    a = Conv2dArgs()
+    a.N, a.H, a.W, a.C, a.K, a.R, a.S, a.pad, a.stride = N, H, W, Cc, K, R, S, pad, stride
+    a.tile, a.split_k = tile, split_k
+    return _lib.load().cusync_conv2d_workspace_size(C.byref(a))
 
 
 def conv2d(stage, N, H, W, Cc, K, x, w, y, tile, stream=None, **kw):
@@ -233,10 +242,11 @@ class ConvChain:
     """Handle over cusync_conv_chain_*: `layers` dependent 3x3 convolutions, stream-ordered or one CuSync
     stage per layer (src/ml-bench/volta_conv2d/resnet.cu, vgg.cu)."""
 
-    def __init__(self, N, H, W, Cc, weight_ptrs, sync, tile=-1, opts=-1, relu=True, fused=False):
+    def __init__(self, N, H, W, Cc, weight_ptrs, sync, tile=-1, opts=-1, relu=True, fused=False, split_k=0):
+        """split_k: runs a tile's steps are cut into (the reference's --split_k_slices); 1 = none, 0 = the library picks."""
         self.L = _lib.load()
         self.layers = len(weight_ptrs)
-        self.cfg = ConvChainConfig(N, H, W, Cc, self.layers, sync, tile, opts, int(relu), int(fused))
+        self.cfg = ConvChainConfig(N, H, W, Cc, self.layers, sync, tile, opts, int(relu), int(fused), split_k)
         arr = (C.c_void_p * self.layers)(*weight_ptrs)
         self.h = self.L.cusync_conv_chain_create(C.byref(self.cfg), arr)
         if not self.h:
@@ -253,6 +263,9 @@ class ConvChain:
 
     def tile(self):
         return self.L.cusync_conv_chain_tile(self.h)
+
+    def split(self):
+        return self.L.cusync_conv_chain_split(self.h)
 
     def stage_state(self, which):
         return _read_stage(self.L, self.L.cusync_conv_chain_stage(self.h, which).contents)

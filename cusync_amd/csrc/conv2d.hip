@@ -23,6 +23,7 @@
 #include "rt_internal.h"
 #include "gemm_kernel_dma.h"
 #include "conv3x3_kernel.h"
+#include "split_choice.h"
 
 namespace {
 
@@ -34,27 +35,30 @@ struct ConvTile {
   void (*kernel)(GemmParams);
   int residentPerCU;
   void (*chainKernel)(ConvChainParams);     // several layers in one launch; halo tiles only
+  void (*splitKernel)(GemmParams);          // the same tile with its steps cut into runs (split_k > 1); halo tiles only
 };
 
 #define CUSYNC_CONV_TILE(BM, BN, BK, WM, WN, ST, OCC) \
   { BM, BN, BK, (size_t)DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>::LDS_BYTES, \
-    gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>, kAConv>, -1, nullptr }
+    gemmDmaKernel<DmaCfg<BM, BN, BK, WM, WN, ST, OCC, true>, kAConv>, -1, nullptr, nullptr }
 
 using HaloA = Halo3x3Cfg<256, 64, 4, 1, 4, 2>;     // 64 output channels per tile: four waves of 64 x 64 stacked
 using HaloB = Halo3x3Cfg<128, 128, 2, 2, 3, 1>;    // 128 output channels per tile
+using HaloC = Halo3x3Cfg<64, 128, 2, 2, 3, 1>;     // 64 pixels: what fits beside the halo of 512-channel pixels (7 x 7 images)
 
 ConvTile g_convTiles[CUSYNC_CONV_TILE_COUNT] = {
   CUSYNC_CONV_TILE(128, 64, 32, 2, 2, 4, 3),    // CUSYNC_CONV_TILE_128x64x32
   CUSYNC_CONV_TILE(128, 128, 32, 2, 2, 4, 2),   // CUSYNC_CONV_TILE_128x128x32
   CUSYNC_CONV_TILE(256, 64, 32, 4, 1, 3, 2),    // CUSYNC_CONV_TILE_256x64x32
   // the halo tiles: 3x3 / pad 1 / stride 1 only; LDS size depends on the image width and channels
-  { HaloA::BM, HaloA::BN, HaloA::BK, 0, convHalo3x3Kernel<HaloA>, -1, convHalo3x3ChainKernel<HaloA> },   // CUSYNC_CONV_TILE_HALO_256x64x64
-  { HaloB::BM, HaloB::BN, HaloB::BK, 0, convHalo3x3Kernel<HaloB>, -1, convHalo3x3ChainKernel<HaloB> },   // CUSYNC_CONV_TILE_HALO_128x128x64
+  { HaloA::BM, HaloA::BN, HaloA::BK, 0, convHalo3x3Kernel<HaloA>, -1, convHalo3x3ChainKernel<HaloA>, convHalo3x3Kernel<HaloA, true> },   // CUSYNC_CONV_TILE_HALO_256x64x64
+  { HaloB::BM, HaloB::BN, HaloB::BK, 0, convHalo3x3Kernel<HaloB>, -1, convHalo3x3ChainKernel<HaloB>, convHalo3x3Kernel<HaloB, true> },   // CUSYNC_CONV_TILE_HALO_128x128x64
+  { HaloC::BM, HaloC::BN, HaloC::BK, 0, convHalo3x3Kernel<HaloC>, -1, convHalo3x3ChainKernel<HaloC>, convHalo3x3Kernel<HaloC, true> },   // CUSYNC_CONV_TILE_HALO_64x128x64
 };
 
-bool isHalo(int tile) { return tile == CUSYNC_CONV_TILE_HALO_256x64x64 || tile == CUSYNC_CONV_TILE_HALO_128x128x64; }
+bool isHalo(int tile) { return tile >= CUSYNC_CONV_TILE_HALO_256x64x64 && tile <= CUSYNC_CONV_TILE_HALO_64x128x64; }
 uint32_t haloLds(int tile, uint32_t W, uint32_t C) {
-  return tile == CUSYNC_CONV_TILE_HALO_256x64x64 ? HaloA::ldsBytes(W, C) : HaloB::ldsBytes(W, C);
+  return tile == CUSYNC_CONV_TILE_HALO_256x64x64 ? HaloA::ldsBytes(W, C) : tile == CUSYNC_CONV_TILE_HALO_128x128x64 ? HaloB::ldsBytes(W, C) : HaloC::ldsBytes(W, C);
 }
 constexpr uint32_t kMaxLds = 160 * 1024 - 1024;      // what one workgroup may ask for (the kernel has 8 bytes of static LDS)
 
@@ -95,6 +99,13 @@ int residentConv(ConvTile* ti, size_t lds) {
           CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, ti->chainKernel, kThreads, lds))) return 0;
       n = std::min(n, m);
     }
+    if (ti->splitKernel) {
+      int m = 0;
+      if (CUSYNC_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(ti->splitKernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds)) ||
+          CUSYNC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, ti->splitKernel, kThreads, lds))) return 0;
+      n = std::min(n, m);
+    }
     ti->residentPerCU = n;
     if (halo) g_haloLds[idx] = (uint32_t)lds;
   }
@@ -102,6 +113,11 @@ int residentConv(ConvTile* ti, size_t lds) {
 }
 
 uint32_t outExtent(uint32_t in, uint32_t filter, uint32_t pad, uint32_t stride) { return (in + 2 * pad - filter) / stride + 1; }
+
+size_t partialBytes(const cusync_conv2d_args* a, const ConvTile* ti) {
+  const cusync_dim3 g = cusync_conv2d_grid_split(a->tile, a->N, a->H, a->W, a->K, a->R, a->S, a->pad, a->stride, a->split_k);
+  return (size_t)g.z * g.y * g.x * ti->bm * ti->bn * sizeof(float);
+}
 
 // Kernel parameters of one convolution launched with `launched` workgroups.
 GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t launched) {
@@ -119,11 +135,20 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
   p.epilogue = a->epilogue;
   p.a_mode = CUSYNC_A_PLAIN;
   p.launched = launched;
-  p.splitK = 1;
-  p.kPerSlice = (p.K + ti->bk - 1) / ti->bk * ti->bk;
+  p.splitK = (uint32_t)std::max(1, a->split_k);
+  const uint32_t chunks = (p.K + ti->bk - 1) / ti->bk;
+  p.kPerSlice = (chunks + p.splitK - 1) / p.splitK * ti->bk;
   p.mPad = s.grid.y * ti->bm;
   p.waitRound = 1;
   p.coopReduce = 0; p.partialBytes = 0;
+  p.partials = nullptr; p.arrivals = nullptr;
+  if (p.splitK > 1) {
+    // [split_k][row tiles][column tiles][BM * BN] fp32 partial sums, then two counters per output tile, as the GEMM's
+    const size_t bytes = partialBytes(a, ti);
+    p.partials = (float*)a->workspace;
+    p.arrivals = (uint32_t*)((char*)a->workspace + bytes);
+    p.partialBytes = (uint32_t)bytes;
+  }
   cusync::rt::timeline(&p.timeline, &p.timelineCap);
   // Producer tiles are whole 128-byte lines of the activation tensor when a pixel's channels are.
   p.stage.lineAligned = !cusync::rt::forceAcquire() && s.in.kind != CUSYNC_POLICY_NOSYNC && (uintptr_t)a->x % 128 == 0 &&
@@ -131,6 +156,9 @@ GemmParams convParams(const cusync_conv2d_args* a, const ConvTile* ti, uint32_t 
                         (s.in.kind == CUSYNC_POLICY_ROWSYNC || (s.in.tileN * 2) % 128 == 0);
   p.stage.releaseAll = cusync::rt::forceRelease();
   p.stage.prepare(launched);
+  // the runs of a tile share the adding up when each has a workgroup of its own from the start (see gemm_f16.hip)
+  p.coopReduce = slicesShareReduction((int)p.splitK, true, true, p.stage.noDraws, launched, s.grid.x * s.grid.y * s.grid.z,
+                                      ti->bm, (s.opts & CUSYNC_OPT_AVOID_WAIT_KERNEL) != 0);
   return p;
 }
 
@@ -147,16 +175,28 @@ int cusync_conv2d_tile_shape(int tile, uint32_t* tileM, uint32_t* tileN, uint32_
   return 0;
 }
 
-cusync_dim3 cusync_conv2d_grid(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
-                               uint32_t pad, uint32_t stride) {
+cusync_dim3 cusync_conv2d_grid_split(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
+                                     uint32_t pad, uint32_t stride, int split_k) {
   cusync_dim3 g = {0, 0, 0};
   ConvTile* ti = convTile(tile);
   if (!ti || stride == 0 || H + 2 * pad < R || W + 2 * pad < S) return g;
   const uint32_t M = N * outExtent(H, R, pad, stride) * outExtent(W, S, pad, stride);
   g.x = (K + ti->bn - 1) / ti->bn;
   g.y = (M + ti->bm - 1) / ti->bm;
-  g.z = 1;
+  g.z = (uint32_t)std::max(1, split_k);
   return g;
+}
+
+cusync_dim3 cusync_conv2d_grid(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
+                               uint32_t pad, uint32_t stride) {
+  return cusync_conv2d_grid_split(tile, N, H, W, K, R, S, pad, stride, 1);
+}
+
+size_t cusync_conv2d_workspace_size(const cusync_conv2d_args* a) {
+  ConvTile* ti = a ? convTile(a->tile) : nullptr;
+  if (!ti || a->split_k <= 1) return 0;
+  const cusync_dim3 g = cusync_conv2d_grid_split(a->tile, a->N, a->H, a->W, a->K, a->R, a->S, a->pad, a->stride, a->split_k);
+  return partialBytes(a, ti) + 2 * (size_t)g.x * g.y * sizeof(uint32_t);
 }
 
 cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
@@ -181,9 +221,15 @@ cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args* a) {
   }
   if (((uintptr_t)a->x | (uintptr_t)a->w | (uintptr_t)a->y) % 16) { setError("conv2d: misaligned operand"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (a->epilogue < 0 || a->epilogue > CUSYNC_EPILOGUE_RELU) { setError("conv2d: unknown epilogue"); return CUSYNC_ERROR_NOT_INITIALIZED; }
-  const cusync_dim3 g = cusync_conv2d_grid(a->tile, a->N, a->H, a->W, a->K, a->R, a->S, a->pad, a->stride);
+  if (a->split_k > 1) {
+    if (!ti->splitKernel) { setError("conv2d: split_k > 1 needs a halo tile"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if ((uint32_t)a->split_k > a->R * a->S * (a->C / ti->bk)) { setError("conv2d: more runs than steps (9 * C / 64)"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (!a->workspace || (uintptr_t)a->workspace % 16) { setError("conv2d: split_k > 1 needs a 16-byte aligned workspace of cusync_conv2d_workspace_size bytes"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+    if (partialBytes(a, ti) >= 0x80000000ull) { setError("conv2d: partial sums larger than 2 GiB"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  }
+  const cusync_dim3 g = cusync_conv2d_grid_split(a->tile, a->N, a->H, a->W, a->K, a->R, a->S, a->pad, a->stride, a->split_k);
   const cusync_stage_desc& s = a->stage;
-  if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("conv2d: stage grid does not match cusync_conv2d_grid"); return CUSYNC_ERROR_NOT_INITIALIZED; }
+  if (s.grid.x != g.x || s.grid.y != g.y || s.grid.z != g.z) { setError("conv2d: stage grid does not match cusync_conv2d_grid_split"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (!s.tileOrder || !s.tileCounter || !s.startCounter || !s.spinTimeouts || !s.xcdTickets) { setError("conv2d: stage not allocated"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (s.out.kind != CUSYNC_POLICY_NOSYNC && !s.tileStatusWrite) { setError("conv2d: producer stage without semaphores"); return CUSYNC_ERROR_NOT_INITIALIZED; }
   if (s.in.kind != CUSYNC_POLICY_NOSYNC) {
@@ -219,7 +265,7 @@ cusync_error cusync_conv2d_run(const cusync_conv2d_args* a, void* stream) {
   if (a->max_workgroups > 0) launched = std::min<uint32_t>(launched, (uint32_t)a->max_workgroups);
 
   GemmParams p = convParams(a, ti, launched);
-  hipLaunchKernelGGL(ti->kernel, dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(a->split_k > 1 ? ti->splitKernel : ti->kernel, dim3(launched), dim3(kThreads), lds, (hipStream_t)stream, p);
   if (CUSYNC_HIP(hipGetLastError())) return CUSYNC_ERROR_DEVICE;
   cusync::rt::noteLaunch(a->stage, launched >= (uint32_t)resident);
   return CUSYNC_SUCCESS;
@@ -235,6 +281,8 @@ struct cusync_conv_chain {
   std::vector<cusync_stage_desc> st;
   std::vector<hipStream_t> stream;
   std::vector<hipEvent_t> ev;        // layers + 1 events: start, after each layer
+  std::vector<void*> ws;             // per layer: partial sums and counters of the runs a tile's steps are cut into
+  int splitK = 1;
   uint32_t timeoutsSeen = 0;         // sum of the stages' give-up counters when the last run returned
 };
 
@@ -258,6 +306,7 @@ cusync_policy_desc noSyncDesc() {
 void freeChain(cusync_conv_chain* c) {
   for (auto s : c->stream) (void)hipStreamSynchronize(s);
   for (auto& d : c->st) cusync_stage_free(&d);
+  for (auto w : c->ws) (void)hipFree(w);
   for (auto e : c->ev) (void)hipEventDestroy(e);
   for (auto s : c->stream) (void)hipStreamDestroy(s);
   delete c;
@@ -276,6 +325,7 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
   if (c->cfg.tile < 0)
     c->cfg.tile = cfg->C % 128 == 0 && haloEligible(CUSYNC_CONV_TILE_HALO_128x128x64, cfg->W, cfg->C, 3, 3, 1, 1) ? CUSYNC_CONV_TILE_HALO_128x128x64
                   : haloEligible(CUSYNC_CONV_TILE_HALO_256x64x64, cfg->W, cfg->C, 3, 3, 1, 1) ? CUSYNC_CONV_TILE_HALO_256x64x64
+                  : cfg->C % 128 == 0 && haloEligible(CUSYNC_CONV_TILE_HALO_64x128x64, cfg->W, cfg->C, 3, 3, 1, 1) ? CUSYNC_CONV_TILE_HALO_64x128x64
                   : cfg->C % 128 == 0 ? CUSYNC_CONV_TILE_128x128x32 : CUSYNC_CONV_TILE_256x64x32;
   uint32_t tm = 0, tn = 0;
   if (cusync_conv2d_tile_shape(c->cfg.tile, &tm, &tn, nullptr)) { setError("conv chain: unknown tile id"); delete c; return nullptr; }
@@ -285,8 +335,32 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
     delete c;
     return nullptr;
   }
-  const cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);
+  cusync_dim3 g = cusync_conv2d_grid(c->cfg.tile, cfg->N, cfg->H, cfg->W, cfg->C, 3, 3, 1, 1);
   if (g.x == 0 || g.y == 0) { setError("conv chain: empty shape"); delete c; return nullptr; }
+  // Layers whose tiles leave most of the device idle (14 x 14 x 256 at batch 32: 98 tiles; 7 x 7 x 512: 100) have the
+  // 9 * C / 64 steps of a tile cut into runs, a workgroup each, whose partial sums are put together as the GEMM's
+  // k-slices are: as many runs as stay resident together, of at least nine steps each (measured, pairs in us without
+  // runs -> with: 32x14x14x256 63 -> 54 in two; 32x7x7x512 82 -> 59 in two; 8x14x14x256 65 -> 50 in four;
+  // 1x7x7x512 82 -> 43 in eight; with shorter runs the exchange costs more than the idle CUs: 1x56x56x64 35 -> 50
+  // in nine runs of one step), and a number the 32-row pieces of a 128-row tile divide among, so that the runs
+  // share the adding up.
+  c->splitK = 1;
+  if (cfg->split_k > 1) c->splitK = cfg->split_k;
+  else if (cfg->split_k == 0 && isHalo(c->cfg.tile) && !(c->cfg.fused && cfg->sync != CUSYNC_SYNC_STREAM)) {
+    ConvTile* ti = convTile(c->cfg.tile);
+    const int resident = residentConv(ti, haloLds(c->cfg.tile, cfg->W, cfg->C));
+    const uint32_t tiles = g.x * g.y, steps = 9 * (cfg->C / 64);
+    uint32_t s = resident > 0 && tiles * 2 <= (uint32_t)g_convNumCUs ? std::min<uint32_t>((uint32_t)resident / tiles, steps / 9) : 1u;
+    if (tm >= 128) s = s >= 4 ? 4 : s == 3 ? 2 : s;      // a 128-row tile's four pieces divide among two or four runs
+    while (s > 1 && (steps + s - 1) / s * (s - 1) >= steps) s--;      // no run without steps
+    c->splitK = (int)std::max(1u, s);
+  }
+  if (c->splitK > 1 && (!isHalo(c->cfg.tile) || (c->cfg.fused && cfg->sync != CUSYNC_SYNC_STREAM))) {
+    setError("conv chain: cutting a tile's steps into runs needs a halo tile and one launch per layer");
+    delete c;
+    return nullptr;
+  }
+  g.z = (uint32_t)c->splitK;
 
   // Edge policies: what a layer posts and what the next one waits on
   // (src/ml-bench/volta_conv2d/resnet.cu:107-116; in vgg.cu the middle layers are consumer and producer at once).
@@ -337,6 +411,18 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
     if (CUSYNC_HIP(hipEventCreate(&e))) { freeChain(c); return nullptr; }
     c->ev.push_back(e);
   }
+  if (c->splitK > 1) {
+    cusync_conv2d_args a;
+    memset(&a, 0, sizeof a);
+    a.N = cfg->N; a.H = cfg->H; a.W = cfg->W; a.C = cfg->C; a.K = cfg->C; a.R = a.S = 3; a.pad = 1; a.stride = 1;
+    a.tile = c->cfg.tile; a.split_k = c->splitK;
+    const size_t bytes = cusync_conv2d_workspace_size(&a);
+    for (uint32_t i = 0; i < cfg->layers; i++) {
+      void* w = nullptr;
+      if (CUSYNC_HIP(hipMalloc(&w, bytes)) || CUSYNC_HIP(hipMemset(w, 0, bytes))) { if (w) (void)hipFree(w); freeChain(c); return nullptr; }
+      c->ws.push_back(w);
+    }
+  }
   return c;
 }
 
@@ -360,6 +446,8 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain* c, const void* x, void* co
     a.y = ys[i];
     a.epilogue = (c->cfg.relu && i + 1 < n) ? CUSYNC_EPILOGUE_RELU : CUSYNC_EPILOGUE_NONE;
     a.tile = c->cfg.tile;
+    a.split_k = c->splitK;
+    a.workspace = c->splitK > 1 ? c->ws[i] : nullptr;
     return a;
   };
   if (overlapped && c->cfg.fused) {
@@ -430,5 +518,6 @@ const cusync_stage_desc* cusync_conv_chain_stage(const cusync_conv_chain* c, uin
 }
 
 int cusync_conv_chain_tile(const cusync_conv_chain* c) { return c ? c->cfg.tile : -1; }
+int cusync_conv_chain_split(const cusync_conv_chain* c) { return c ? c->splitK : -1; }
 
 }  // extern "C"

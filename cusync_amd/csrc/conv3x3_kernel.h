@@ -51,8 +51,11 @@ struct Halo3x3Cfg {
   }
 };
 
-// One layer: all tiles of stage p.stage that this workgroup draws.
-template<class C>
+// One layer: all tiles of stage p.stage that this workgroup draws.  SPLIT: the launch may cut the 9 * C/64 steps of
+// a tile into p.splitK runs (grid z), each a workgroup's, whose partial sums are put together as the GEMM's k-slices
+// are (finishTile); the layers whose tiles are fewer than half the CUs are run that way.  A kernel without it does
+// not carry the exchange's code.
+template<class C, bool SPLIT>
 __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   __shared__ uint32_t sTicket, sLast;
@@ -113,6 +116,9 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     const cusync_dim3 t = stage.ticketToTile(ticket);
     const unsigned long long tl0 = p.timeline ? wall_clock64() : 0;
     const uint32_t m0 = t.y * C::BM, n0 = t.x * C::BN;
+    // this workgroup's steps of the tile: all of them, or run t.z of p.kPerSlice / 64 steps
+    const uint32_t itBegin = SPLIT ? min(steps, t.z * (p.kPerSlice / C::BK)) : 0;
+    const uint32_t itEnd = SPLIT ? min(steps, itBegin + p.kPerSlice / C::BK) : steps;
 
     // Which of the nine taps of this lane's output pixels lie inside the image: bit 3r + s.
     uint32_t tapMask[C::TM];
@@ -152,18 +158,18 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
       const bool inside = m0 + pl >= W + 1 && flat < p.M && pl < haloPix;
       loadToLds(rA, __builtin_amdgcn_readfirstlane(ldsHalo + q * 1024), inside ? (flat * Cc + chunk * 8) * 2 : kOutOfRange);
     }
-    // Filter chunk `it` (tap it / chunksPerTap, channels (it % chunksPerTap) * 64 ..) into stage it % STAGES.
+    // Filter chunk `it` (tap it / chunksPerTap, channels (it % chunksPerTap) * 64 ..) into stage (it - itBegin) % STAGES.
     auto issueB = [&](uint32_t it) {
-      const uint32_t lds = ldsBase + (it % C::STAGES) * C::B_STAGE + wave * C::B_LOADS * 1024;
+      const uint32_t lds = ldsBase + ((it - itBegin) % C::STAGES) * C::B_STAGE + wave * C::B_LOADS * 1024;
 #pragma unroll
       for (int q = 0; q < C::B_LOADS; q++) {
-        const bool live = it < steps && n0 + bLoadRow[q] < p.N;
+        const bool live = it < itEnd && n0 + bLoadRow[q] < p.N;
         loadToLds(rB, __builtin_amdgcn_readfirstlane(lds + q * 1024),
                   live ? ((n0 + bLoadRow[q]) * p.ldb + it * C::BK + bLoadChunk[q] * 8) * 2 : kOutOfRange);
       }
     };
 #pragma unroll
-    for (uint32_t it = 0; it < C::STAGES - 1; it++) issueB(it);
+    for (uint32_t it = 0; it < C::STAGES - 1; it++) issueB(itBegin + it);
     if (tid == 0 && round == 0) stage.finishStart(startToken, p.launched);
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
@@ -176,14 +182,14 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
         for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     const uint32_t aPixel0 = wm * C::WTM + (lane & 31) + W + 1;       // this lane's first output pixel inside the halo
-    for (uint32_t it = 0; it < steps; it++) {
+    for (uint32_t it = itBegin; it < itEnd; it++) {
       waitVmcnt<(C::STAGES - 2) * C::B_LOADS>();     // chunk `it` (and, the first time, the halo) has landed
       __builtin_amdgcn_s_barrier();                   // ... for everyone; everyone is done with chunk it-1
       asm volatile("" ::: "memory");
       issueB(it + C::STAGES - 1);
       const uint32_t tap = it / chunksPerTap, cc = it % chunksPerTap;
       const int32_t shift = ((int32_t)(tap / 3) - 1) * (int32_t)W + (int32_t)(tap % 3) - 1;
-      const char* sb = smem + (it % C::STAGES) * C::B_STAGE;
+      const char* sb = smem + ((it - itBegin) % C::STAGES) * C::B_STAGE;
       uint32_t aBase[C::TM], aSwz[C::TM];
 #pragma unroll
       for (int i = 0; i < C::TM; i++) {
@@ -221,7 +227,7 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
     waitVmcnt<0>();
     const unsigned long long tl2 = p.timeline ? wall_clock64() : 0;
     if (tid == 0) nextRaw = stage.drawBegin(dryXcds, noDraws);     // settled after the epilogue
-    const bool completed = finishTile<C, false>(p, acc, t, wm, wn, lane, &sLast, smem);
+    const bool completed = finishTile<C, SPLIT>(p, acc, t, wm, wn, lane, &sLast, smem);
     cusync_dim3 done = {m0, n0, 0};
     if (completed && stage.isProducer()) stage.post(done, 1, stage.storesThrough());
     else __syncthreads();
@@ -229,9 +235,9 @@ __device__ __forceinline__ void convHalo3x3Layer(const GemmParams& p) {
   }
 }
 
-template<class C>
+template<class C, bool SPLIT = false>
 __global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3Kernel(GemmParams p) {
-  convHalo3x3Layer<C>(p);
+  convHalo3x3Layer<C, SPLIT>(p);
 }
 
 // A chain of layers in ONE launch: every workgroup works through the tiles of layer 0 it can draw, then those
@@ -250,7 +256,7 @@ struct ConvChainParams {
 template<class C>
 __global__ __launch_bounds__(kThreads, C::OCC) void convHalo3x3ChainKernel(ConvChainParams cp) {
   for (uint32_t l = 0; l < cp.layers; l++) {
-    convHalo3x3Layer<C>(cp.layer[l]);
+    convHalo3x3Layer<C, false>(cp.layer[l]);
     __syncthreads();        // everyone has read the last ticket of this layer before the next one's is written
   }
 }

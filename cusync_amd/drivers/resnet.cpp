@@ -2,6 +2,7 @@
 // (options :309-345, output :754-759, 825-827).
 //
 //   resnet --n 32 --h 56 --w 56 --c 64 [--layers 2] [--iterations 20] [--ref-check] [--sync rowsync|tilesync]
+//          [--split_k_slices n]
 //
 // `layers` 3x3 convolutions with c input and c output channels (2 = the ResNet block, 4 = the VGG block),
 // NHWC fp16, ReLU between the layers.  Output: START-BASELINE: / END-BASELINE: {Total, Conv1, ...} micro seconds,
@@ -11,13 +12,14 @@
 int main(int argc, char** argv) {
   auto args = drv::parseArgs(argc, argv);
   if (args.count("help")) {
-    printf("resnet --n <int> --h <int> --w <int> --c <int> [--layers <int>] [--iterations <int>] [--ref-check] [--sync rowsync|tilesync]\n");
+    printf("resnet --n <int> --h <int> --w <int> --c <int> [--layers <int>] [--iterations <int>] [--ref-check] [--sync rowsync|tilesync] [--split_k_slices <int>]\n");
     return 0;
   }
   const uint32_t n = (uint32_t)drv::getInt(args, "n", 32), h = (uint32_t)drv::getInt(args, "h", 56), w = (uint32_t)drv::getInt(args, "w", 56),
                  c = (uint32_t)drv::getInt(args, "c", 64), layers = (uint32_t)drv::getInt(args, "layers", 2);
   const int runs = (int)drv::getInt(args, "iterations", 20), warmup = 10;
   const bool check = drv::getBool(args, "ref-check", false);
+  const int splitK = (int)drv::getInt(args, "split_k_slices", 0);      // 0: the library picks (the reference's default is none)
   const std::string syncName = drv::get(args, "sync", "tilesync");
   const int sync = syncName == "rowsync" ? CUSYNC_SYNC_ROW : CUSYNC_SYNC_TILE;
   if (layers < 1 || layers > 16) { fprintf(stderr, "--layers must be 1..16\n"); return EXIT_FAILURE; }
@@ -39,6 +41,7 @@ int main(int argc, char** argv) {
     cusync_conv_chain_config cfg;
     memset(&cfg, 0, sizeof cfg);
     cfg.N = n; cfg.H = h; cfg.W = w; cfg.C = c; cfg.layers = layers; cfg.sync = mode; cfg.tile = -1; cfg.opts = -1; cfg.relu = 1;
+    cfg.split_k = splitK;      // --split_k_slices (resnet.cu:329); 0 = the library picks
     cusync_conv_chain* ch = cusync_conv_chain_create(&cfg, wd.data());
     if (!ch) { fprintf(stderr, "cusync_conv_chain_create failed: %s\n", cusync_rt_last_error()); exit(EXIT_FAILURE); }
     DRV_CHECK(cusync_conv_chain_run(ch, x, yd.data(), warmup, nullptr, nullptr));

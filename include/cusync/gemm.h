@@ -225,8 +225,10 @@ class CuSyncGemm {
 // padding and one stride for both directions, no dilation, no groups.
 struct Conv2dProblemSize {
   int N, H, W, C, K, R, S, pad, stride;
-  Conv2dProblemSize(int N_ = 0, int H_ = 0, int W_ = 0, int C_ = 0, int K_ = 0, int R_ = 3, int S_ = 3, int pad_ = 1, int stride_ = 1)
-      : N(N_), H(H_), W(W_), C(C_), K(K_), R(R_), S(S_), pad(pad_), stride(stride_) {}
+  int split_k_slices;      // runs the R*S*C/64 steps of a tile are cut into (src/ml-bench/volta_conv2d/resnet.cu:246, 689); 1 = none
+  Conv2dProblemSize(int N_ = 0, int H_ = 0, int W_ = 0, int C_ = 0, int K_ = 0, int R_ = 3, int S_ = 3, int pad_ = 1, int stride_ = 1,
+                    int split_k_slices_ = 1)
+      : N(N_), H(H_), W(W_), C(C_), K(K_), R(R_), S(S_), pad(pad_), stride(stride_), split_k_slices(split_k_slices_) {}
   int P() const { return (H + 2 * pad - R) / stride + 1; }
   int Q() const { return (W + 2 * pad - S) / stride + 1; }
 };
@@ -257,32 +259,43 @@ class CuSyncImplicitGemmConvolution {
     const half_bits* w;
     half_bits* y;
     int max_workgroups;
-    Params() : x(nullptr), w(nullptr), y(nullptr), max_workgroups(0) {}
+    void* workspace;
+    Params() : x(nullptr), w(nullptr), y(nullptr), max_workgroups(0), workspace(nullptr) {}
   };
   Params params_;
 
   static dim3 get_grid_shape(Conv2dProblemSize const& p) {
-    const cusync_dim3 g = cusync_conv2d_grid(TileId, (uint32_t)p.N, (uint32_t)p.H, (uint32_t)p.W, (uint32_t)p.K, (uint32_t)p.R, (uint32_t)p.S,
-                                            (uint32_t)p.pad, (uint32_t)p.stride);
+    const cusync_dim3 g = cusync_conv2d_grid_split(TileId, (uint32_t)p.N, (uint32_t)p.H, (uint32_t)p.W, (uint32_t)p.K, (uint32_t)p.R, (uint32_t)p.S,
+                                                  (uint32_t)p.pad, (uint32_t)p.stride, p.split_k_slices);
     return dim3(g.x, g.y, g.z);
   }
   static Status can_implement(Arguments const& args) {
     if (args.output_op.alpha != 1.0f || args.output_op.beta != 0.0f) return Status::kErrorNotSupported;
-    cusync_conv2d_args a = toArgs(args.custage, args.problem_size, args.ref_A.data(), args.ref_B.data(), args.ref_D.data(), 0);
+    // the workspace arrives with initialize(): any aligned address stands in for it here
+    cusync_conv2d_args a = toArgs(args.custage, args.problem_size, args.ref_A.data(), args.ref_B.data(), args.ref_D.data(), 0,
+                                  args.problem_size.split_k_slices > 1 ? (void*)args.ref_D.data() : nullptr);
     return cusync_conv2d_can_implement(&a) == CUSYNC_SUCCESS ? Status::kSuccess : Status::kErrorInvalidProblem;
   }
-  static size_t get_workspace_size(Arguments const&) { return 0; }
+  // Bytes initialize() wants for the runs' partial sums and counters (0 without runs).  The caller zeroes the
+  // buffer once; the kernels leave the counters at zero.
+  static size_t get_workspace_size(Arguments const& args) {
+    cusync_conv2d_args a = toArgs(args.custage, args.problem_size, nullptr, nullptr, nullptr, 0, nullptr);
+    return cusync_conv2d_workspace_size(&a);
+  }
   Status initialize(Arguments const& args, void* workspace = nullptr, void* stream = nullptr) {
-    (void)workspace; (void)stream;
+    (void)stream;
     const Status s = can_implement(args);
     if (s != Status::kSuccess) return s;
+    if (args.problem_size.split_k_slices > 1 && !workspace) return Status::kErrorWorkspaceNull;
+    params_.workspace = workspace;
     params_.custage = args.custage;
     params_.problem_size = args.problem_size;
     params_.x = args.ref_A.data(); params_.w = args.ref_B.data(); params_.y = args.ref_D.data();
     return Status::kSuccess;
   }
   Status run(void* stream = nullptr) {
-    cusync_conv2d_args a = toArgs(params_.custage, params_.problem_size, params_.x, params_.w, params_.y, params_.max_workgroups);
+    cusync_conv2d_args a = toArgs(params_.custage, params_.problem_size, params_.x, params_.w, params_.y, params_.max_workgroups,
+                                  params_.workspace);
     return cusync_conv2d_run(&a, stream) == CUSYNC_SUCCESS ? Status::kSuccess : Status::kErrorInternal;
   }
   Status run(bool overlap, int* kernelExecuted, void* stream = nullptr) { (void)overlap; (void)kernelExecuted; return run(stream); }
@@ -290,7 +303,7 @@ class CuSyncImplicitGemmConvolution {
 
  private:
   static cusync_conv2d_args toArgs(const CuStageImpl& stage, Conv2dProblemSize const& p, const half_bits* x, const half_bits* w,
-                                   half_bits* y, int max_workgroups) {
+                                   half_bits* y, int max_workgroups, void* workspace) {
     cusync_conv2d_args a;
     a.stage = stage.desc();
     a.N = (uint32_t)p.N; a.H = (uint32_t)p.H; a.W = (uint32_t)p.W; a.C = (uint32_t)p.C;
@@ -299,6 +312,8 @@ class CuSyncImplicitGemmConvolution {
     a.epilogue = Epilogue;
     a.tile = TileId;
     a.max_workgroups = max_workgroups;
+    a.split_k = p.split_k_slices;
+    a.workspace = workspace;
     return a;
   }
 };

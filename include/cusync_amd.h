@@ -342,7 +342,8 @@ enum {
   CUSYNC_CONV_TILE_HALO_256x64x64 = 3,   /* 3x3, pad 1, stride 1, C a power of two >= 64: the input tile and its halo
                                             stay in LDS, each pixel is fetched once instead of once per filter tap */
   CUSYNC_CONV_TILE_HALO_128x128x64 = 4,
-  CUSYNC_CONV_TILE_COUNT = 5
+  CUSYNC_CONV_TILE_HALO_64x128x64 = 5,   /* the halo tile that still fits with 512 channels (7 x 7 images) */
+  CUSYNC_CONV_TILE_COUNT = 6
 };
 
 typedef struct cusync_conv2d_args {
@@ -356,6 +357,10 @@ typedef struct cusync_conv2d_args {
   int32_t epilogue;            /* CUSYNC_EPILOGUE_* (the ResNet pair uses RELU after the first convolution) */
   int32_t tile;                /* CUSYNC_CONV_TILE_* */
   int32_t max_workgroups;      /* 0 = as many as stay resident */
+  int32_t split_k;             /* Conv2dProblemSize::split_k_slices (CV/resnet.cu:246, 689, 765): 0 or 1 = none; n (halo tiles):
+                                  the R*S*C/64 steps of a tile in n runs, grid z = n, partial sums added in run order */
+  void *workspace;             /* split_k > 1: cusync_conv2d_workspace_size bytes, 16-byte aligned; its counters (the last
+                                  2 * tiles words) zero before the first run, the kernel leaves them zero */
 } cusync_conv2d_args;
 
 int cusync_conv2d_tile_shape(int tile, uint32_t *tileM, uint32_t *tileN, uint32_t *tileK);
@@ -363,6 +368,12 @@ int cusync_conv2d_tile_shape(int tile, uint32_t *tileM, uint32_t *tileN, uint32_
  * (CC/gemm/threadblock/cusync_threadblock_swizzle.h:34-44). */
 cusync_dim3 cusync_conv2d_grid(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
                                uint32_t pad, uint32_t stride);
+/* The same with the tile's steps cut into split_k runs: (K_out tiles, N*P*Q tiles, split_k), as get_tiled_shape with
+ * split_k_slices gives it (CV/resnet.cu:765). */
+cusync_dim3 cusync_conv2d_grid_split(int tile, uint32_t N, uint32_t H, uint32_t W, uint32_t K, uint32_t R, uint32_t S,
+                                     uint32_t pad, uint32_t stride, int split_k);
+/* get_workspace_size (cusyncimplicit_gemm_convolution.h): 0 without runs. */
+size_t cusync_conv2d_workspace_size(const cusync_conv2d_args *args);
 cusync_error cusync_conv2d_can_implement(const cusync_conv2d_args *args);
 int cusync_conv2d_max_resident(int tile);
 /* operator()(stream) (cusyncimplicit_gemm_convolution.h:283-298).  A consumer stage waits, per producer
@@ -382,6 +393,8 @@ typedef struct cusync_conv_chain_config {
   int32_t fused;               /* 1 (sync ROW or TILE, halo tiles, at most 8 layers): all layers in ONE launch whose workgroups
                                   work through layer 0, then layer 1, ... with the same semaphores between them; no wait
                                   kernel and no second launch between a producer and its consumer */
+  int32_t split_k;             /* --split_k_slices (CV/resnet.cu:329): runs a tile's steps are cut into; 1 = none; 0 = the
+                                  library picks (runs only for layers whose tiles leave more than half the CUs idle) */
 } cusync_conv_chain_config;
 
 typedef struct cusync_conv_chain cusync_conv_chain;
@@ -396,6 +409,7 @@ cusync_error cusync_conv_chain_run(cusync_conv_chain *chain, const void *x, void
                                    double *times_us, double *layer_us);
 const cusync_stage_desc *cusync_conv_chain_stage(const cusync_conv_chain *chain, uint32_t which);
 int cusync_conv_chain_tile(const cusync_conv_chain *chain);
+int cusync_conv_chain_split(const cusync_conv_chain *chain);      /* runs per tile the chain runs with */
 
 /* ------------------------------------------------------------------------- */
 /* Fused multi-head attention stage: O = softmax(mask(Q K^T * scale)) V per    */

@@ -19,11 +19,12 @@ CONV_TILES = list(range(api.CONV_TILE.COUNT))
 def fits(tile, Cc, R=3, S=3, pad=1, stride=1, W=8):
     """The halo tiles only do 3x3 / pad 1 / stride 1 with a power-of-two channel count of at least 64, and
     need their rows plus 2W + 2 pixels of the image in LDS next to the filter stages."""
-    halo = {api.CONV_TILE.HALO_256x64x64: (256, 4 * 8192), api.CONV_TILE.HALO_128x128x64: (128, 3 * 16384)}
+    halo = {api.CONV_TILE.HALO_256x64x64: (256, 4 * 8192), api.CONV_TILE.HALO_128x128x64: (128, 3 * 16384),
+            api.CONV_TILE.HALO_64x128x64: (64, 3 * 16384)}
     if tile not in halo:
         return True
     rows, filt = halo[tile]
-    lds = filt + -(-(rows + 2 * W + 2) * Cc * 2 // 1024) * 1024
+    lds = filt + -(-(rows + 2 * W + 3) * Cc * 2 // 1024) * 1024      # the run of pixels and one pixel of zeros
     return (R, S, pad, stride) == (3, 3, 1, 1) and Cc >= 64 and Cc & (Cc - 1) == 0 and lds <= 159 * 1024
 
 
@@ -32,7 +33,7 @@ def he_filters(K, R, S, Cc, seed):
     return (rng.standard_normal((K, R, S, Cc)) * np.sqrt(2.0 / (R * S * Cc))).astype(np.float16)
 
 
-def run_conv(x, w, tile, pad=1, stride=1, epilogue=api.EPI.NONE, max_workgroups=0, launches=1):
+def run_conv(x, w, tile, pad=1, stride=1, epilogue=api.EPI.NONE, max_workgroups=0, launches=1, split_k=1):
     import torch
     L = _lib.load()
     N, H, W, Cc = x.shape
@@ -40,13 +41,15 @@ def run_conv(x, w, tile, pad=1, stride=1, epilogue=api.EPI.NONE, max_workgroups=
     P, Q = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
     dx, dw = to_dev(x), to_dev(w)
     dy = empty_dev((N, P, Q, K), fill=float("nan"))
+    ws = torch.zeros(max(16, api.conv2d_workspace_size(N, H, W, Cc, K, tile, split_k, R, S, pad, stride)), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
-    st = api.Stage(api.conv2d_grid(tile, N, H, W, K, R, S, pad, stride), (1, 1, 1), api.no_sync(), api.no_sync())
+    st = api.Stage(api.conv2d_grid(tile, N, H, W, K, R, S, pad, stride, split_k), (1, 1, 1), api.no_sync(), api.no_sync())
     for _ in range(launches):
         dy.fill_(float("nan"))
         torch.cuda.synchronize()
         rc = api.conv2d(st, N, H, W, Cc, K, dx.data_ptr(), dw.data_ptr(), dy.data_ptr(), tile, R=R, S=S, pad=pad,
-                        stride=stride, epilogue=epilogue, max_workgroups=max_workgroups)
+                        stride=stride, epilogue=epilogue, max_workgroups=max_workgroups, split_k=split_k,
+                        workspace=ws.data_ptr() if split_k > 1 else None)
         assert rc == api.ERR.SUCCESS, api.last_error()
         assert L.cusync_rt_device_sync() == 0, api.last_error()
     assert st.read_state().tile_counter == 0
@@ -103,6 +106,29 @@ def test_conv_matches_oracle(tile, geom):
     assert_close(got, orc.conv2d_nhwc(x, w, pad, stride), "y")
 
 
+HALO_TILES = [api.CONV_TILE.HALO_256x64x64, api.CONV_TILE.HALO_128x128x64, api.CONV_TILE.HALO_64x128x64]
+
+
+@pytest.mark.parametrize("tile", HALO_TILES)
+@pytest.mark.parametrize("geom,split", [((2, 12, 12, 64, 64), 2), ((2, 12, 12, 64, 64), 4),      # 9 steps in 4 runs: 3, 3, 3, 0
+                                        ((2, 12, 12, 64, 64), 9), ((3, 7, 9, 128, 72), 3), ((4, 14, 14, 256, 256), 2),
+                                        ((4, 14, 14, 256, 256), 4), ((1, 7, 7, 512, 136), 5), ((6, 7, 7, 512, 512), 2)])
+def test_conv_steps_cut_into_runs(tile, geom, split):
+    # the reference's --split_k_slices (resnet.cu:329, 689): partial sums of the runs put together, ReLU behind them,
+    # two launches through one workspace (the counters are left at zero)
+    print("conv in runs", tile, geom, split, flush=True)
+    N, H, W, Cc, K = geom
+    if not fits(tile, Cc, W=W):
+        pytest.skip("geometry outside the halo tile's domain")
+    x = uniform_f16((N, H, W, Cc), 15)
+    w = he_filters(K, 3, 3, Cc, 16)
+    got = run_conv(x, w, tile, epilogue=api.EPI.RELU, split_k=split, launches=2)
+    assert_close(got, orc.conv2d_nhwc(x, w, epilogue=orc.EPI_RELU), "y")
+    x = np.round(uniform_f16((N, H, W, Cc), 17) * 4).astype(np.float16)       # integers: every order of adding is exact
+    w = np.round(he_filters(K, 3, 3, Cc, 18) * 16).astype(np.float16)
+    assert np.array_equal(run_conv(x, w, tile, split_k=split), run_conv(x, w, tile))
+
+
 def test_conv_relu_and_persistent_launch():
     x = uniform_f16((4, 20, 20, 64), 7)
     w = he_filters(64, 3, 3, 64, 8)
@@ -144,6 +170,16 @@ def test_conv_can_implement_rejects():
     assert rc(tile=halo, Cc=96) != api.ERR.SUCCESS              # channels not a power of two
     assert rc(tile=halo, H=2, W=4096) != api.ERR.SUCCESS        # halo does not fit LDS (and the grid differs)
     st.destroy()
+    # a tile's steps in runs: halo tiles only, a workspace, no more runs than steps, the stage's grid with the runs in z
+    st2 = api.Stage(api.conv2d_grid(halo, 1, 8, 8, 64, split_k=2), (1, 1, 1), api.no_sync(), api.no_sync())
+    st = st2
+    assert rc(tile=halo, split_k=2, workspace=buf.data_ptr()) == api.ERR.SUCCESS
+    assert rc(tile=halo, split_k=2) != api.ERR.SUCCESS and "workspace" in api.last_error()
+    assert rc(tile=halo, split_k=3, workspace=buf.data_ptr()) != api.ERR.SUCCESS and "grid" in api.last_error()
+    assert rc(tile=halo, split_k=10, workspace=buf.data_ptr()) != api.ERR.SUCCESS and "more runs than steps" in api.last_error()
+    assert rc(tile=api.CONV_TILE.T128x64x32, split_k=2, workspace=buf.data_ptr()) != api.ERR.SUCCESS and "halo tile" in api.last_error()
+    assert api.conv2d_workspace_size(1, 8, 8, 64, 64, halo, 2) == 2 * 256 * 64 * 4 + 2 * 4 and api.conv2d_workspace_size(1, 8, 8, 64, 64, halo, 1) == 0
+    st2.destroy()
 
 
 def chained_convs(N, H, W, Cc, tile1, tile2, kind, iters=1, opts=0, max_wg=(0, 0), seed=20):
@@ -262,12 +298,16 @@ def run_chain(N, H, W, Cc, layers, sync, runs=2, seed=30, **kw):
         times += chain.run((dx if r == runs - 1 else dx_other).data_ptr(), [y.data_ptr() for y in dys], runs=1)
     states = [chain.stage_state(i) for i in range(layers)]
     tile = chain.tile()
+    run_chain.split = chain.split()
     chain.destroy()
     return x, ws, [to_host(y) for y in dys], states, tile, times
 
 
 @pytest.mark.parametrize("shape,layers", [((4, 20, 20, 64), 2), ((32, 56, 56, 64), 2), ((32, 28, 28, 128), 2),
-                                          ((2, 24, 24, 64), 4), ((8, 28, 28, 128), 4), ((16, 56, 56, 64), 4)])
+                                          ((2, 24, 24, 64), 4), ((8, 28, 28, 128), 4), ((16, 56, 56, 64), 4),
+                                          # the deep layers of the ResNet table (resnet_results.csv, 256 and 512 channels):
+                                          # few tiles, whose steps the chain cuts into runs by itself
+                                          ((32, 14, 14, 256), 2), ((32, 7, 7, 512), 2), ((4, 14, 14, 256), 2), ((1, 7, 7, 512), 4)])
 def test_conv_chain_all_sync_modes(shape, layers):
     # two layers: the ResNet block; four layers: the VGG block whose middle layers both wait and post
     print("conv chain", shape, layers, flush=True)
@@ -275,6 +315,10 @@ def test_conv_chain_all_sync_modes(shape, layers):
     for sync in (api.SYNC.STREAM, api.SYNC.ROW, api.SYNC.TILE):
         x, ws, ys, states, tile, _ = run_chain(*shape, layers, sync, runs=2)
         outs[sync] = ys
+        if shape[3] >= 256:
+            assert run_chain.split > 1 and tile in HALO_TILES, (tile, run_chain.split)
+        elif shape[0] == 32:      # the benchmark's pairs have tiles for every CU
+            assert run_chain.split == 1
         tm, tn, _ = api.conv2d_tile_shape(tile)
         for i, st in enumerate(states):
             assert st.spin_timeouts == 0 and st.tile_counter == 0 and st.start_counter == 0
@@ -300,7 +344,7 @@ def test_conv_chain_all_sync_modes(shape, layers):
 def test_conv_chain_in_one_launch(shape, layers, sync):
     # all layers in one launch: same semaphores, same results bit for bit as the stream-ordered chain
     print("conv chain, one launch", shape, layers, sync, flush=True)
-    x, ws, want, _, _, _ = run_chain(*shape, layers, api.SYNC.STREAM, runs=1)
+    x, ws, want, _, _, _ = run_chain(*shape, layers, api.SYNC.STREAM, runs=1, split_k=1)      # one launch never cuts a tile's steps
     _, _, got, states, tile, _ = run_chain(*shape, layers, sync, runs=3, fused=True)
     tm, tn, _ = api.conv2d_tile_shape(tile)
     for i, st in enumerate(states):
