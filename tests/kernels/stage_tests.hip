@@ -320,17 +320,19 @@ int run_launcher_mlp(int policy, uint32_t M, uint32_t K1, uint32_t N1, uint32_t 
 
 // ---- the ResNet pair on the convolution launcher (src/ml-bench/volta_conv2d/resnet.cu:107-116, 704-744) -------------
 // x [N][H][W][C], w1 and w2 [C][3][3][C], y1 and y2 [N][H][W][C].  out as above (semaphores: TileSync, all == iters).
-int run_launcher_conv_pair(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const void* x, const void* w1, void* y1, const void* w2, void* y2,
-                           int iters, int* out) {
-  constexpr int kTile = CUSYNC_CONV_TILE_128x64x32;
-  using Sync1 = TileSync<TransposeXYOrder, 128, 64>;
-  using Sync2 = Conv2DTileSync<TransposeXYOrder, 3, 3, 128, 64>;
+// splitK > 1: Conv2dProblemSize::split_k_slices (resnet.cu:689), with the workspace get_workspace_size asks for.
+extern "C++" {
+template<int kTile, int kTileM, int kTileN>
+static int launcherConvPairImpl(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const void* x, const void* w1, void* y1, const void* w2, void* y2,
+                                int splitK, int iters, int* out) {
+  using Sync1 = TileSync<TransposeXYOrder, kTileM, kTileN>;
+  using Sync2 = Conv2DTileSync<TransposeXYOrder, 3, 3, kTileM, kTileN>;
   using ProdCuStage = CuStage<TransposeXYOrder, NoSync, Sync1>;
   using ConsCuStage = CuStage<TransposeXYOrder, Sync2, NoSync>;
   using Conv1 = CuSyncImplicitGemmConvolution<ProdCuStage, kTile, CUSYNC_EPILOGUE_RELU>;
   using Conv2 = CuSyncImplicitGemmConvolution<ConsCuStage, kTile, CUSYNC_EPILOGUE_NONE>;
   int bad = 0;
-  const Conv2dProblemSize problem((int)N, (int)H, (int)W, (int)C, (int)C, 3, 3, 1, 1);
+  const Conv2dProblemSize problem((int)N, (int)H, (int)W, (int)C, (int)C, 3, 3, 1, 1, splitK);
   const dim3 grid = Conv1::get_grid_shape(problem);
   Sync1 sync1;
   Sync2 sync2;
@@ -345,8 +347,16 @@ int run_launcher_conv_pair(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const
   Conv1 conv1;
   Conv2 conv2;
   bad += Conv1::can_implement(args1) != Status::kSuccess;
-  bad += conv1.initialize(args1) != Status::kSuccess;
-  bad += conv2.initialize(args2) != Status::kSuccess;
+  void *ws1 = nullptr, *ws2 = nullptr;
+  const size_t wsBytes = Conv1::get_workspace_size(args1);
+  bad += (splitK > 1) != (wsBytes > 0);
+  if (wsBytes) {
+    bad += conv1.initialize(args1) != Status::kErrorWorkspaceNull;      // runs without a workspace are refused
+    HIP_OK(hipMalloc(&ws1, wsBytes)); HIP_OK(hipMalloc(&ws2, wsBytes));
+    HIP_OK(hipMemset(ws1, 0, wsBytes)); HIP_OK(hipMemset(ws2, 0, wsBytes));
+  }
+  bad += conv1.initialize(args1, ws1) != Status::kSuccess;
+  bad += conv2.initialize(args2, ws2) != Status::kSuccess;
   for (int r = 0; r < iters; r++) {
     bad += conv1.run(true, NULL, s1) != Status::kSuccess;
     bad += prod.invokeWaitKernel(s2) != CuSyncSuccess;
@@ -367,11 +377,28 @@ int run_launcher_conv_pair(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const
   out[1] = (int)timeouts;
   out[2] = (int)flag;
   int mismatches = 0;
-  for (uint32_t i = 0; i < tiles; i++) mismatches += sems[i] != (uint32_t)iters;
+  // one post per output tile, whatever the runs: grid.x * grid.y semaphores stand at `iters`, the others were never touched
+  uint32_t posted = 0;
+  for (uint32_t i = 0; i < tiles; i++) { posted += sems[i] == (uint32_t)iters; mismatches += sems[i] != 0 && sems[i] != (uint32_t)iters; }
+  mismatches += posted != grid.x * grid.y;
   out[3] = mismatches;
   prod.destroy(); cons.destroy();
   HIP_OK(hipStreamDestroy(s1)); HIP_OK(hipStreamDestroy(s2));
+  if (ws1) HIP_OK(hipFree(ws1));
+  if (ws2) HIP_OK(hipFree(ws2));
   return 0;
+}
+}  // extern "C++"
+
+int run_launcher_conv_pair(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const void* x, const void* w1, void* y1, const void* w2, void* y2,
+                           int iters, int* out) {
+  return launcherConvPairImpl<CUSYNC_CONV_TILE_128x64x32, 128, 64>(N, H, W, C, x, w1, y1, w2, y2, 1, iters, out);
+}
+
+// the same pair on the 128x128 halo tile with every tile's steps in `splitK` runs
+int run_launcher_conv_pair_runs(uint32_t N, uint32_t H, uint32_t W, uint32_t C, const void* x, const void* w1, void* y1, const void* w2, void* y2,
+                                int splitK, int iters, int* out) {
+  return launcherConvPairImpl<CUSYNC_CONV_TILE_HALO_128x128x64, 128, 128>(N, H, W, C, x, w1, y1, w2, y2, splitK, iters, out);
 }
 
 }  // extern "C"

@@ -74,6 +74,16 @@ def test_resnet_driver(shape, layers, sync):
     assert "check: passed" in out
 
 
+@pytest.mark.parametrize("shape,extra", [((8, 14, 14, 256), ()), ((2, 7, 7, 512), ("--split_k_slices", "3")), ((2, 7, 7, 512), ("--split_k_slices", "1"))])
+def test_resnet_driver_deep_layers(shape, extra):
+    # 256 and 512 channels (resnet_results.csv): the chain cuts the tiles' steps into runs by itself, or as --split_k_slices says
+    n, h, w, c = shape
+    out = run("resnet", "--n", str(n), "--h", str(h), "--w", str(w), "--c", str(c), "--iterations", "5", "--ref-check", "--sync", "rowsync", *extra)
+    _, end = between(out, "START-OVERLAP:", "END-OVERLAP")
+    assert float(re.search(r"Total: ([0-9.]+)", end).group(1)) > 0
+    assert "check: passed" in out
+
+
 def test_mlp_stages_driver_against_oracle(tmp_path):
     """The reference's own loop (CuStage + CuSyncGemm objects, invokeWaitKernel, incrementIter) at 256 and 2048 rows,
     both policies, on inputs this test writes; the launchers' H and Y against the CPU oracle on sampled rows, and

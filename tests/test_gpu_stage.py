@@ -174,3 +174,28 @@ def test_resnet_pair_on_the_convolution_launcher():
     y1, y2 = to_host(dy1), to_host(dy2)
     assert_close(y1, orc.conv2d_nhwc(x, w1, epilogue=orc.EPI_RELU), "y1")
     assert_close(y2, orc.conv2d_nhwc(y1, w2), "y2")
+
+
+@pytest.mark.parametrize("runs", [1, 2, 4])
+def test_resnet_pair_on_the_convolution_launcher_with_runs(runs):
+    """Conv2dProblemSize::split_k_slices (CV/resnet.cu:246, 689) on the launcher objects: get_workspace_size, initialize with the
+    workspace (refused without), the 128x128 halo tile, a deep layer's shape."""
+    import torch
+    from util import assert_close, to_dev, to_host, uniform_f16
+    T = _lib.load_stage_tests()
+    N, H, W, Cc = 4, 14, 14, 256
+    rng = np.random.default_rng(6)
+    x = uniform_f16((N, H, W, Cc), 7)
+    w1, w2 = ((rng.standard_normal((Cc, 3, 3, Cc)) * np.sqrt(2.0 / (9 * Cc))).astype(np.float16) for _ in range(2))
+    dx, dw1, dw2 = to_dev(x), to_dev(w1), to_dev(w2)
+    dy1 = torch.full((N, H, W, Cc), float("nan"), dtype=torch.float16, device="cuda")
+    dy2 = torch.full((N, H, W, Cc), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    out = (C.c_int * 4)(-1, -1, -1, -1)
+    rc = T.run_launcher_conv_pair_runs(C.c_uint32(N), C.c_uint32(H), C.c_uint32(W), C.c_uint32(Cc), C.c_void_p(dx.data_ptr()), C.c_void_p(dw1.data_ptr()),
+                                       C.c_void_p(dy1.data_ptr()), C.c_void_p(dw2.data_ptr()), C.c_void_p(dy2.data_ptr()), runs, 3, out)
+    assert rc == 0
+    assert list(out) == [0, 0, 3, 0], list(out)
+    y1, y2 = to_host(dy1), to_host(dy2)
+    assert_close(y1, orc.conv2d_nhwc(x, w1, epilogue=orc.EPI_RELU), "y1")
+    assert_close(y2, orc.conv2d_nhwc(y1, w2), "y2")
