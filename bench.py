@@ -474,12 +474,12 @@ def main():
             best = min(row[k] for k in ("rowsync_us", "tilesync_us", "consecutivesync_us"))
             row["gain_pct"] = round(100 - best / row["stream_us"] * 100, 2)
             other["attention"].append(row)
-        # LLaMA MLP shard (X[B,8192] x [W1|V][8192,2*2752] -> silu(g)*u fused into GEMM2's A operand -> x W2[2752,8192])
+        # LLaMA MLP shard (X[B,8192] x [W1|V][8192,2*2752] -> silu(g)*u in GEMM1's epilogue -> x W2[2752,8192])
         other["llama_mlp"] = []
         lh, li = 8192, 2752
         lw1 = (torch.randn((lh, 2 * li), device="cuda", generator=g) * 0.02).half()
         lw2 = (torch.randn((li, lh), device="cuda", generator=g) * 0.02).half()
-        for b in (1, 64, 512, 2048):
+        for b in BATCHES:      # the seven batch sizes of the GPT-3 sweep
             lx = (torch.rand((b, lh), device="cuda", generator=g) * 2 - 1).half()
             lhid = torch.empty((b, 2 * li), dtype=torch.float16, device="cuda")
             ly = torch.empty((b, lh), dtype=torch.float16, device="cuda")
