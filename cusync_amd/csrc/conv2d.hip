@@ -360,6 +360,11 @@ cusync_conv_chain* cusync_conv_chain_create(const cusync_conv_chain_config* cfg,
     delete c;
     return nullptr;
   }
+  if (c->splitK > 1 && (uint32_t)c->splitK > 9 * (cfg->C / 64)) {
+    setError("conv chain: more runs than a tile has steps (9 * C / 64)");
+    delete c;
+    return nullptr;
+  }
   g.z = (uint32_t)c->splitK;
 
   // Edge policies: what a layer posts and what the next one waits on

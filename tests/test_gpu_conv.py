@@ -364,3 +364,8 @@ def test_conv_chain_in_one_launch_rejects():
     torch.cuda.synchronize()
     with pytest.raises(RuntimeError):      # the implicit-GEMM tiles have no chain kernel
         api.ConvChain(4, 20, 20, 64, [t.data_ptr() for t in w], api.SYNC.ROW, tile=api.CONV_TILE.T256x64x32, fused=True)
+    # runs of a tile's steps: not in one launch for all layers, not on the implicit-GEMM tiles, no more than steps
+    for kw, what in ((dict(fused=True, split_k=2), "one launch per layer"), (dict(tile=api.CONV_TILE.T256x64x32, split_k=2), "halo tile"),
+                     (dict(split_k=10), "more runs")):
+        with pytest.raises(RuntimeError, match=what):
+            api.ConvChain(4, 20, 20, 64, [t.data_ptr() for t in w], api.SYNC.ROW, **kw)
