@@ -19,7 +19,7 @@ POLICY = SimpleNamespace(NOSYNC=0, ROWSYNC=1, TILESYNC=2, STRIDEDSYNC=3, CONV2DT
 EPI = SimpleNamespace(NONE=0, GELU=1, RELU=2, SWIGLU=3)
 TILE = SimpleNamespace(T256x256x32=0, T256x128x64=1, T128x128x64=2, T64x128x64=3, T32x128x64=4,
                        T128x256x64=5, T256x64x64=6, T128x64x64=7, T256x128x32=8, T128x256x32=9, T128x128x32=10,
-                       T128x192x32=11, T256x192x32=12, D32x128x64=13, D64x128x64=14, D64x192x64=15, T128x192x32_ALONE=16, T256x384x32=17, T256x192x64=18, COUNT=19)
+                       T128x192x32=11, T256x192x32=12, D32x128x64=13, D64x128x64=14, D64x192x64=15, T128x192x32_ALONE=16, T256x384x32=17, T256x192x64=18, D128x192x64=19, COUNT=20)
 CONV_TILE = SimpleNamespace(T128x64x32=0, T128x128x32=1, T256x64x32=2, HALO_256x64x64=3, HALO_128x128x64=4, HALO_64x128x64=5, COUNT=6)
 SYNC = SimpleNamespace(STREAM=0, ROW=1, TILE=2, STRIDED=3)
 MODEL = SimpleNamespace(GPT3=0, LLAMA=1)

@@ -247,7 +247,10 @@ cusync_attn_layer* cusync_attn_layer_create(const cusync_attn_layer_config* cfg,
   // (with the 256x192 tile's K loop in assembly, 256x192 in k-slices also leads from 321 to 512 rows and from 769 to
   // 1024: the QKV projection 73 -> 67 us at 384 rows, 131 -> 115 at 896, 137 -> 120 at 1024; from 513 to 640 rows its
   // third row tile is mostly padding and 128x192 stays, 87 against 102 us)
-  const int wide1 = S <= 32 ? small : S <= 320 ? CUSYNC_TILE_D64x192x64 : S > 512 && S <= 640 ? CUSYNC_TILE_128x192x32_ALONE
+  // (two full row tiles of 128, 193 to 256 rows: 128x192 with the operands fetched 64 columns of K at a time, the QKV
+  // projection 55 -> 52 us at 256 rows, 51 -> 49.5 at 224; level below, and at 320 rows its third row tile costs 17 us)
+  const int wide1 = S <= 32 ? small : S > 192 && S <= 256 && cfg->hidden % 64 == 0 ? CUSYNC_TILE_D128x192x64
+                    : S <= 320 ? CUSYNC_TILE_D64x192x64 : S > 512 && S <= 640 ? CUSYNC_TILE_128x192x32_ALONE
                     : CUSYNC_TILE_256x192x32;
   const int wide3 = S <= 32 ? small : S <= 256 ? CUSYNC_TILE_D64x192x64 : S <= 512 ? CUSYNC_TILE_128x192x32_ALONE
                     : S <= 1024 ? CUSYNC_TILE_256x192x32 : CUSYNC_TILE_128x192x32;

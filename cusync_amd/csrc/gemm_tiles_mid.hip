@@ -11,6 +11,7 @@ void fillDmaTilesMid(TileInfo* t) {
   t[CUSYNC_TILE_128x128x32] = CUSYNC_TILE_DMA(128, 128, 32, 2, 2, 3, 3);   // three workgroups per CU
   t[CUSYNC_TILE_128x192x32] = CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 3, 2);   // 6144 and 12288 columns are 32 and 64 tiles
   t[CUSYNC_TILE_128x192x32_ALONE] = CUSYNC_TILE_DMA(128, 192, 32, 2, 2, 4, 2, false, true);   // 80 KB of LDS, so one workgroup per CU
+  t[CUSYNC_TILE_D128x192x64] = CUSYNC_TILE_DMA(128, 192, 64, 2, 2, 3, 1);   // 120 KB of LDS; A rows arrive as whole 128-byte lines
 }
 
 }  // namespace gemm

@@ -186,6 +186,9 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // the device (the chain under RowSync: 384 rows 106 -> 92 us, 512: 117 -> 103, 768: 166 -> 131, 1024: 176 -> 156,
     // 1536: 236 -> 203, 2048: 263 -> 246; level at 256 rows).  Its last column tile is ragged (5504 = 28.7 x 192).
     if (c.batch > 256 && c.hidden % 64 == 0) a = CUSYNC_TILE_256x192x64;
+    // 129 to 256 rows: 128x192 with the operands fetched 64 columns of K at a time (a row of A as one 128-byte line;
+    // the chain under RowSync: 160 rows 77 -> 65 us, 256 rows 80 -> 72; level with 256x192x64 at 384 and 512 rows)
+    else if (c.batch > 128 && c.hidden % 64 == 0) a = CUSYNC_TILE_D128x192x64;
     *t1 = c.tile1 >= 0 ? c.tile1 : a;
     *t2 = c.tile2 >= 0 ? c.tile2 : b;
     if (c.one_launch && sync != CUSYNC_SYNC_STREAM && c.tile2 < 0) *t2 = *t1;
@@ -231,6 +234,13 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // (106 against 120 us for one row tile of 128 in eight and four).
     if (n1 % 192 == 0) a = CUSYNC_TILE_128x192x32;
     if (n2 % 192 == 0 && !swiglu) b = CUSYNC_TILE_128x192x32;
+    // The same tile with both operands fetched 64 columns of K at a time, a CU to itself: a row of A then arrives as
+    // one 128-byte line instead of two 64-byte pieces, and what bounds the loop here is the number of requests a CU's
+    // memory path holds, not their size (stream-ordered pair / best CuSync, us: 160 rows 126 / 122 -> 121 / 116,
+    // 192: 133 / 125 -> 124 / 118, 224: 140 / 131 -> 126 / 120, 256: 148 / 138 -> 128 / 124; level at 128 rows, and
+    // behind 256x192x64 in four and two k-slices from 257 rows on: 320 rows 156 against 173).
+    if (a == CUSYNC_TILE_128x192x32 && c.hidden % 64 == 0) a = CUSYNC_TILE_D128x192x64;
+    if (b == CUSYNC_TILE_128x192x32 && c.inner % 64 == 0) b = CUSYNC_TILE_D128x192x64;
   }
   // StridedSync needs the gate|up split on a column-tile boundary of GEMM1: 128- or 256-wide tiles where the
   // 192-wide ones do not divide `inner`, 64-wide ones where nothing else does (2752 = 43 * 64)

@@ -197,7 +197,8 @@ Result runPair(MLPParameters& mlpParams, const Request& rq) {
   X(CUSYNC_TILE_128x192x32, CUSYNC_TILE_128x192x32) X(CUSYNC_TILE_128x192x32_ALONE, CUSYNC_TILE_128x192x32_ALONE) \
   X(CUSYNC_TILE_256x192x64, CUSYNC_TILE_256x192x64) X(CUSYNC_TILE_256x192x64, CUSYNC_TILE_128x192x32)           \
   X(CUSYNC_TILE_256x192x64, CUSYNC_TILE_256x384x32) X(CUSYNC_TILE_256x192x32, CUSYNC_TILE_256x192x32)           \
-  X(CUSYNC_TILE_256x192x32, CUSYNC_TILE_256x384x32) X(CUSYNC_TILE_128x128x64, CUSYNC_TILE_128x128x64)
+  X(CUSYNC_TILE_256x192x32, CUSYNC_TILE_256x384x32) X(CUSYNC_TILE_128x128x64, CUSYNC_TILE_128x128x64)           \
+  X(CUSYNC_TILE_D128x192x64, CUSYNC_TILE_D128x192x64)
 
 bool dispatch(int tile1, int tile2, MLPParameters& p, const Request& rq, Result* out) {
 #define TRY_PAIR(A, B) \

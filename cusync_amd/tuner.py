@@ -34,7 +34,7 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
          api.TILE.T128x256x32: (2, 2, 3), api.TILE.T128x128x32: (2, 2, 3), api.TILE.T128x192x32: (2, 2, 3),
          api.TILE.T256x192x32: (4, 2, 4), api.TILE.D32x128x64: (1, 4, 4), api.TILE.D64x128x64: (1, 4, 3),
          api.TILE.D64x192x64: (2, 2, 4), api.TILE.T128x192x32_ALONE: (2, 2, 4), api.TILE.T256x384x32: (2, 4, 3),
-         api.TILE.T256x192x64: (4, 2, 4)}
+         api.TILE.T256x192x64: (4, 2, 4), api.TILE.D128x192x64: (2, 2, 3)}
 
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 

@@ -84,6 +84,7 @@ CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_D64x192x64, 64, 192, 64);
 CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_128x192x32_ALONE, 128, 192, 32);
 CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x384x32, 256, 384, 32);
 CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_256x192x64, 256, 192, 64);
+CUSYNC_GEMM_TILE_SHAPE(CUSYNC_TILE_D128x192x64, 128, 192, 64);
 #undef CUSYNC_GEMM_TILE_SHAPE
 
 // CuSyncGemm<CuStageImpl, TileId, Epilogue>: D = epilogue(A x B), fp16 row-major, fp32 accumulate.

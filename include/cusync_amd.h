@@ -259,7 +259,10 @@ enum {
   CUSYNC_TILE_256x192x64 = 18,       /* 256x192 with both operands fetched 64 columns of K at a time, in whole cache lines (A ring of two
                                         slots, B ring of three, one barrier per slot), K loop in assembly.  K (and every k-slice) a
                                         multiple of 64; a stage of a tile policy waits for all its producer tiles before its first load */
-  CUSYNC_TILE_COUNT = 19
+  CUSYNC_TILE_D128x192x64 = 19,      /* 128x192 with both operands fetched 64 columns of K at a time: A in whole cache lines, three
+                                        stages of 40 KB, a CU to itself: for 256 rows and thereabouts, where the loop waits on the
+                                        number of requests a CU's memory path holds and 64-byte pieces of A rows take as many as lines */
+  CUSYNC_TILE_COUNT = 20
 };
 
 typedef struct cusync_gemm_args {

@@ -107,7 +107,7 @@ def test_gemm_persistent_launch_smaller_than_grid():
 
 @pytest.mark.parametrize("tile", [api.TILE.T256x192x32, api.TILE.T256x256x32, api.TILE.T256x128x32, api.TILE.T128x128x32,
                                   api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x192x32_ALONE, api.TILE.D64x192x64,
-                                  api.TILE.T256x384x32, api.TILE.T256x192x64])
+                                  api.TILE.T256x384x32, api.TILE.T256x192x64, api.TILE.D128x192x64])
 @pytest.mark.parametrize("K", [24, 200, 1032])
 def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
     # 3 workgroups for 12 to 88 tiles with ragged edges: every workgroup goes from one tile's stores straight into
@@ -132,7 +132,7 @@ def test_gemm_several_tiles_per_workgroup_direct_to_lds(tile, K):
 
 
 @pytest.mark.parametrize("tile", [api.TILE.T128x128x64, api.TILE.T32x128x64, api.TILE.T128x256x32, api.TILE.T256x256x32,
-                                  api.TILE.T128x128x32, api.TILE.T256x384x32, api.TILE.T256x192x64])
+                                  api.TILE.T128x128x32, api.TILE.T256x384x32, api.TILE.T256x192x64, api.TILE.D128x192x64])
 @pytest.mark.parametrize("split", [2, 3, 8])
 def test_gemm_split_k(tile, split):
     print("split-k tile", tile, "slices", split, flush=True)
@@ -154,7 +154,8 @@ def test_gemm_split_k(tile, split):
 @pytest.mark.parametrize("tile,split", [(api.TILE.T256x192x32, 2), (api.TILE.T256x192x32, 4), (api.TILE.T256x192x32, 8),
                                         (api.TILE.T128x192x32_ALONE, 4), (api.TILE.D64x192x64, 2), (api.TILE.T256x256x32, 4),
                                         (api.TILE.T256x192x32, 3), (api.TILE.D32x128x64, 4), (api.TILE.T256x384x32, 2),
-                                        (api.TILE.T256x384x32, 4), (api.TILE.T256x192x64, 2), (api.TILE.T256x192x64, 4)])
+                                        (api.TILE.T256x384x32, 4), (api.TILE.T256x192x64, 2), (api.TILE.T256x192x64, 4),
+                                        (api.TILE.D128x192x64, 2), (api.TILE.D128x192x64, 4)])      # as the 256-row MLP runs it
 def test_gemm_split_k_with_the_reduction_shared_among_the_slices(tile, split):
     # every k-slice has a workgroup of its own, so the slices of a tile each add up and store a share of it (where
     # the tile has 128 rows or more and its 32-row pieces divide among them: not for 3 slices, not for the 64- and
@@ -278,7 +279,8 @@ def chained(M, N, K, tile1, tile2, policy_kind, iters=1, opts=0, max_wg=0, seed=
                                    (api.TILE.D64x192x64, api.TILE.T128x192x32),
                                    (api.TILE.T256x192x32, api.TILE.T256x384x32),      # consumer with the K loop in assembly
                                    (api.TILE.T256x384x32, api.TILE.T256x192x32),
-                                   (api.TILE.T256x192x64, api.TILE.T256x384x32)])     # as the 2048-row MLP runs them
+                                   (api.TILE.T256x192x64, api.TILE.T256x384x32),      # as the 2048-row MLP runs them
+                                   (api.TILE.D128x192x64, api.TILE.D128x192x64), (api.TILE.D64x192x64, api.TILE.D128x192x64)])
 def test_two_chained_gemms_config1(policy_kind, opts, tiles):
     # BASELINE config 1: M=256, N=K=1024, fp32 accumulate, inputs uniform from a seed
     print("chained", policy_kind, opts, tiles, flush=True)
