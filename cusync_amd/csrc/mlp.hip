@@ -237,8 +237,9 @@ void pickTiles(const cusync_mlp_config& c, int sync, bool swiglu, bool fused, in
     // The same tile with both operands fetched 64 columns of K at a time, a CU to itself: a row of A then arrives as
     // one 128-byte line instead of two 64-byte pieces, and what bounds the loop here is the number of requests a CU's
     // memory path holds, not their size (stream-ordered pair / best CuSync, us: 160 rows 126 / 122 -> 121 / 116,
-    // 192: 133 / 125 -> 124 / 118, 224: 140 / 131 -> 126 / 120, 256: 148 / 138 -> 128 / 124; level at 128 rows, and
-    // behind 256x192x64 in four and two k-slices from 257 rows on: 320 rows 156 against 173).
+    // 192: 133 / 125 -> 124 / 118, 224: 140 / 131 -> 126 / 120, 256: 148 / 138 -> 128 / 124, on other machines of the
+    // same kind 148 / 138 -> 143 / 135; level at 128 rows, and behind 256x192x64 in four and two k-slices from 257
+    // rows on: 320 rows 156 against 173).
     if (a == CUSYNC_TILE_128x192x32 && c.hidden % 64 == 0) a = CUSYNC_TILE_D128x192x64;
     if (b == CUSYNC_TILE_128x192x32 && c.inner % 64 == 0) b = CUSYNC_TILE_D128x192x64;
   }

@@ -55,7 +55,7 @@ def candidates(batch, n1, n2):
     elif batch <= 128:
         tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x128x64, api.TILE.T128x128x32], [1, 2, 4, 8]
     elif batch <= 512:
-        tiles, splits = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x64, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4, 8]
+        tiles, splits = [api.TILE.D64x192x64, api.TILE.D128x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T256x192x64, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x128x32], [1, 2, 4, 8]
     else:
         tiles, splits = [api.TILE.T256x192x64, api.TILE.T256x384x32, api.TILE.T256x192x32, api.TILE.T128x192x32, api.TILE.T128x256x32, api.TILE.T128x128x32], [1, 2]
     if n1 % 192 or n2 % 192:        # the LLaMA shard (5504 and 8192 columns): also the 256-wide tiles
@@ -213,7 +213,7 @@ def tune_attention(seq, log, hidden=12288, heads=12):
             layer.destroy()
 
     if seq <= 256:
-        tiles = [api.TILE.D64x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T128x128x32]
+        tiles = [api.TILE.D64x192x64, api.TILE.D128x192x64, api.TILE.T128x192x32_ALONE, api.TILE.T128x128x32]
     elif seq <= 1024:
         tiles = [api.TILE.T128x192x32_ALONE, api.TILE.T128x192x32, api.TILE.T256x192x64, api.TILE.T256x192x32, api.TILE.T128x128x32]
     else:
