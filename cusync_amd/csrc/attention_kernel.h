@@ -238,6 +238,13 @@ __global__ __launch_bounds__(kThreads, 2) void attentionKernel(AttnParams p) {
 #pragma unroll
     for (int s = 0; s < 8; s++)
       qf[s] = __builtin_bit_cast(half8, loadChunk(rReg, myq < p.S ? ((p.cached + myq) * p.ldq + head * kHD + 16 * s + 8 * hi) * 2 : kOutOfRange));
+    // The fragments are waited for here, once.  Left to the compiler the wait lands in the block loop, in front of
+    // each fragment's first use: it counts these eight loads as possibly outstanding on every pass and asks for
+    // "at most 7 - s loads in flight" there, and the loads in flight there are the direct loads of the blocks ahead,
+    // issued after these and invisible to its count: every block then waits for the blocks it has just requested.
+    // (At the benchmark's sizes those land within a block's time and the kernel measures the same either way.)
+#pragma unroll
+    for (int s = 0; s < 8; s++) asm volatile("" : "+v"(qf[s]));
     const unsigned long long tl1 = p.timeline ? wall_clock64() : 0;
 
     float rowMax = kMasked, rowSum = 0.0f;      // rowSum: this half-wave's share
