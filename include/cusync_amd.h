@@ -256,8 +256,8 @@ enum {
   CUSYNC_TILE_256x384x32 = 17,       /* direct-to-LDS, eight wavefronts of 128x96 in two alternating groups, 3 stages, a CU to itself:
                                         a third less data moved per MFMA than 256x192; 12288 columns are 32 tiles.  K must be a
                                         multiple of 32; a stage of a tile policy waits for all its producer tiles before its first load */
-  CUSYNC_TILE_256x192x64 = 18,       /* 256x192 with both operands fetched 64 columns of K at a time, in whole cache lines (A ring of two
-                                        slots, B ring of three, one barrier per slot), K loop in assembly.  K (and every k-slice) a
+  CUSYNC_TILE_256x192x64 = 18,       /* 256x192 with both operands fetched 64 columns of K at a time, in whole cache lines (A ring of three
+                                        slots, B ring of four 32-row stages, one barrier per 32 columns), K loop in assembly.  K (and every k-slice) a
                                         multiple of 64; a stage of a tile policy waits for all its producer tiles before its first load */
   CUSYNC_TILE_D128x192x64 = 19,      /* 128x192 with both operands fetched 64 columns of K at a time: A in whole cache lines, three
                                         stages of 40 KB, a CU to itself: for 256 rows and thereabouts, where the loop waits on the
