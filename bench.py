@@ -264,6 +264,9 @@ def main():
                     "k_loop_us": {"median": med(q[:, 4] - q[:, 3]), "min": round(float((q[:, 4] - q[:, 3]).min()) / 100.0, 2),
                                   "max": round(float((q[:, 4] - q[:, 3]).max()) / 100.0, 2)},
                     "epilogue_us": med(q[:, 5] - q[:, 4]),
+                    # the eight XCDs do not run at one speed: a launch of one tile per CU is as long as its slowest XCD
+                    "k_loop_us_by_xcd": [med((q[:, 4] - q[:, 3])[(q[:, 0] >> 40) & 0xf == x]) if np.any((q[:, 0] >> 40) & 0xf == x) else None
+                                         for x in range(8)],
                     "last_tile_done_us": round(float(q[:, 5].max() - t0) / 100.0, 2),
                 }
         c.close()
