@@ -232,7 +232,10 @@ def main():
     def roofline_leg(B, warm, timed):
         """Durations of the two GEMM launches, HIP events on the stream they run on."""
         c = Chain(B, api.SYNC.STREAM)
-        (t3,) = interleaved([c], warm, timed, split_first=True)
+        # The settling steps run on this very chain, with nothing between them and the timed ones: after an idle gap of
+        # tens of milliseconds (a handle being created is one) the device runs these launches at boost for 2 ms, then
+        # up to a quarter slower for several, and is back at its steady rate only after about 15 ms of load.
+        (t3,) = interleaved([c], max(warm, SETTLE_STEPS), timed, split_first=True)
         tiles = c.tiles
         timeline = None
         if args.timeline:
