@@ -36,6 +36,7 @@ PEAK_FP16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 SETTLE_STEPS = 40              # untimed steps of the timed shape before anything is measured: after a light load
                                # the device needs about 30 steps of this size until its clock settles
+MIN_WARM_S = 0.025             # the slow phase after an idle gap (handles being created) is over after about 15 ms of load
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_by_tile.md")
 MFMA_TABLE = os.path.join(ROOT, "profiles", "gemm_mfma_by_batch.md")
 
@@ -197,11 +198,14 @@ def main():
         return bool(one.value)
 
     def interleaved(chains, warm, timed, split_first=False):
-        """Runs the chains in turn, one step each per round: `warm` untimed rounds, then `timed` rounds.  Returns
+        """Runs the chains in turn, one step each per round: `warm` untimed rounds (and as many more as it takes to
+        keep the device under this load for MIN_WARM_S), then `timed` rounds.  Returns
         one list of step times per chain (for the first chain, with split_first, triples: step, GEMM1, GEMM2)."""
-        for _ in range(warm):
+        t0, done = time.perf_counter(), 0
+        while done < warm or time.perf_counter() - t0 < MIN_WARM_S:      # (steps return when their last kernel has ended)
             for c in chains:
                 c.step()
+            done += 1
         times = [[] for _ in chains]
         for _ in range(timed):
             for i, c in enumerate(chains):
@@ -211,9 +215,11 @@ def main():
     def rounds(objs, step, warm=10, timed=20):
         """The same turn-taking for the other chains' handles: `step(obj)` runs one pass and returns ([us], extra).
         Returns the step times and the extras, one list per object."""
-        for _ in range(warm):
+        t0, done = time.perf_counter(), 0
+        while done < warm or time.perf_counter() - t0 < MIN_WARM_S:
             for o in objs:
                 step(o)
+            done += 1
         times, extras = [[] for _ in objs], [[] for _ in objs]
         for _ in range(timed):
             for i, o in enumerate(objs):
@@ -562,6 +568,11 @@ def main():
         # tiles it draws, then the consumer's, waiting on the tiles' semaphores in between (no second stream)
         names += ["rowsync_one_launch", "tilesync_one_launch"]
         chains += [Chain(B, api.SYNC.ROW, one_launch=True), Chain(B, api.SYNC.TILE, one_launch=True)]
+    # settling on the chains that are timed (creating them left the device idle), then the --warmup rounds
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < MIN_WARM_S:
+        for c in chains:
+            c.step()
     for _ in range(args.warmup):
         for c in chains:
             c.step()
