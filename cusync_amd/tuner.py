@@ -24,6 +24,7 @@ import argparse
 import pprint
 import statistics
 import sys
+import time
 
 from . import api
 
@@ -36,6 +37,7 @@ WAVES = {api.TILE.T256x256x32: (4, 2, 4), api.TILE.T256x128x64: (2, 2, 2), api.T
          api.TILE.D64x192x64: (2, 2, 4), api.TILE.T128x192x32_ALONE: (2, 2, 4), api.TILE.T256x384x32: (2, 4, 3),
          api.TILE.T256x192x64: (4, 2, 4), api.TILE.D128x192x64: (2, 2, 3)}
 
+MIN_WARM_S = 0.025
 SHAPES = {"gpt3": (api.MODEL.GPT3, 12288, 6144), "llama": (api.MODEL.LLAMA, 8192, 2752)}
 
 
@@ -91,7 +93,12 @@ class Bench:
         torch.cuda.synchronize()
         m = api.Mlp(self.model, batch, self.hidden, self.inner, sync, self.w1.data_ptr(), self.w2.data_ptr(), **kw)
         try:
+            # after the idle gap a new handle leaves, the device runs big GEMMs up to a quarter slower from the 2nd to
+            # about the 15th millisecond of load: warm up for at least MIN_WARM_S before anything is timed
+            t0 = time.perf_counter()
             m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=warm)
+            while time.perf_counter() - t0 < MIN_WARM_S:
+                m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=5)
             out = m.run(x.data_ptr(), h.data_ptr(), y.data_ptr(), runs=timed, split=(sync == api.SYNC.STREAM))
             if m.stage_state(1).spin_timeouts:
                 return None
@@ -206,7 +213,10 @@ def tune_attention(seq, log, hidden=12288, heads=12):
     def run(sync, **kw):
         layer = api.AttnLayer(seq, hidden, heads, sync, wqkv.data_ptr(), wo.data_ptr(), **kw)
         try:
+            t0 = time.perf_counter()
             layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=10)
+            while time.perf_counter() - t0 < MIN_WARM_S:        # (see Bench.run)
+                layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=5)
             t, st = layer.run(x.data_ptr(), qkv.data_ptr(), o.data_ptr(), y.data_ptr(), runs=20, stages=True)
             return trimmed(t), [trimmed([v[i] for v in st]) for i in range(3)], layer.tiles()
         finally:
