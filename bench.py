@@ -244,7 +244,7 @@ def main():
         (t3,) = interleaved([c], max(warm, SETTLE_STEPS), timed, split_first=True)
         tiles = c.tiles
         timeline = None
-        if args.timeline:
+        if args.timeline or not args.roofline_only:      # (left out of the bare --roofline-only run the profiler's counters average over)
             # one record per finished tile: 100 MHz clock at kernel entry of the workgroup, tile drawn, first loads
             # issued, main loop done, epilogue (and post) done
             from cusync_amd import _lib
