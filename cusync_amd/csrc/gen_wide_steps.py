@@ -79,6 +79,8 @@ def batch(x):
     """The direct loads issued behind barrier x: chunk x+2 of B, and with x even A slot x/2+1.  Each entry is the
     instructions of one load."""
     out = []
+    if "noload" in OPTS:       # timing experiment: no direct loads in the loop (wrong results)
+        return [["s_nop 0"]]
     if x % 2 == 0:
         slot = (x // 2 + 1) % 2
         for q in range(4):
@@ -269,6 +271,8 @@ def frag_reads2(c, kk, s):
 def batch2(x):
     """Direct loads behind barrier x: chunk x+3 of B and, x even, A slot x/2+2.  soffA is 64 bytes x the B chunk."""
     out = []
+    if "noload" in OPTS:
+        return [["s_nop 0"]]
     if x % 2 == 0:
         slot = (x // 2 + 2) % 3
         for q in range(4):
